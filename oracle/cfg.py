@@ -1,0 +1,164 @@
+"""Restatement of the reference's cfg grammar and layer-geometry rules (test infrastructure).
+
+Grammar: src/parser.c:891-924 (read_cfg), src/option_list.c:52-77 (read_option),
+src/utils.c:302-313 (strip removes every blank, tab and newline before anything else).
+Geometry: parse_net_options src/parser.c:655-679; parse_convolutional :179-207 with
+convolutional_out_height/width src/convolutional_layer.c:66-74; parse_maxpool :483-498 with
+make_maxpool_layer src/maxpool_layer.c:21-36; parse_route :601-640; parse_shortcut :539-556
+with make_shortcut_layer src/shortcut_layer.c:9-24; parse_upsample :592-599 with
+make_upsample_layer src/upsample_layer.c:7-29; parse_yolo :306-342 with make_yolo_layer
+src/yolo_layer.c:13-32; parse_avgpool :500-511; parse_softmax :270-283.
+
+Pinned by tests/test_oracle_cfg.py against the layer table of the compiled reference.
+"""
+from __future__ import annotations
+
+import re
+
+SECTION_ALIASES = {
+    "[conv]": "convolutional", "[convolutional]": "convolutional",
+    "[max]": "maxpool", "[maxpool]": "maxpool",
+    "[avg]": "avgpool", "[avgpool]": "avgpool",
+    "[soft]": "softmax", "[softmax]": "softmax",
+    "[route]": "route", "[shortcut]": "shortcut", "[upsample]": "upsample", "[yolo]": "yolo",
+    "[net]": "net", "[network]": "net",
+}
+
+
+def _atoi(s: str) -> int:
+    m = re.match(r"[+-]?\d+", s)
+    return int(m.group(0)) if m else 0
+
+
+def _atof(s: str) -> float:
+    m = re.match(r"[+-]?(\d+\.?\d*([eE][+-]?\d+)?|\.\d+([eE][+-]?\d+)?)", s)
+    return float(m.group(0)) if m else 0.0
+
+
+def read_cfg(text: str):
+    """-> list of (section_name_with_brackets, {key: value}) in file order."""
+    sections = []
+    for raw in text.split("\n"):
+        line = raw.replace(" ", "").replace("\t", "").replace("\n", "")
+        if not line or line[0] in "#;":
+            continue
+        if line[0] == "[":
+            sections.append((line, {}))
+            continue
+        if "=" not in line:
+            continue
+        key, val = line.split("=", 1)
+        if val == "" :
+            continue
+        # option_find returns the first matching key in insertion order
+        sections[-1][1].setdefault(key, val)
+    return sections
+
+
+def parse(text: str) -> dict:
+    sections = read_cfg(text)
+    if not sections:
+        raise ValueError("Config file has no sections")
+    head, opts = sections[0]
+    if SECTION_ALIASES.get(head) != "net":
+        raise ValueError("First section must be [net] or [network]")
+    gi = lambda o, k, d: _atoi(o[k]) if k in o else d
+    gf = lambda o, k, d: _atof(o[k]) if k in o else d
+    batch = gi(opts, "batch", 1) // gi(opts, "subdivisions", 1) * gi(opts, "time_steps", 1)
+    net = {"batch": batch, "h": gi(opts, "height", 0), "w": gi(opts, "width", 0),
+           "c": gi(opts, "channels", 0)}
+    net["inputs"] = gi(opts, "inputs", net["h"] * net["w"] * net["c"])
+    h, w, c, inputs = net["h"], net["w"], net["c"], net["inputs"]
+    layers = []
+    for index, (name, o) in enumerate(sections[1:]):
+        kind = SECTION_ALIASES.get(name)
+        if kind is None:
+            raise NotImplementedError(f"layer type {name} is outside the checked path")
+        L = {"type": kind, "batch": batch, "h": h, "w": w, "c": c, "inputs": inputs}
+        if kind == "convolutional":
+            n = gi(o, "filters", 1)
+            size = gi(o, "size", 1)
+            stride = gi(o, "stride", 1)
+            padding = gi(o, "padding", 0)
+            if gi(o, "pad", 0):
+                padding = size // 2
+            groups = gi(o, "groups", 1)
+            L.update(n=n, size=size, stride=stride, pad=padding, groups=groups,
+                     activation=o.get("activation", "logistic"),
+                     batch_normalize=gi(o, "batch_normalize", 0),
+                     binary=gi(o, "binary", 0), xnor=gi(o, "xnor", 0))
+            L["out_h"] = (h + 2 * padding - size) // stride + 1
+            L["out_w"] = (w + 2 * padding - size) // stride + 1
+            L["out_c"] = n
+            L["nweights"] = c // groups * n * size * size
+        elif kind == "maxpool":
+            stride = gi(o, "stride", 1)
+            size = gi(o, "size", stride)
+            padding = gi(o, "padding", size - 1)
+            L.update(size=size, stride=stride, pad=padding)
+            L["out_h"] = (h + padding - size) // stride + 1
+            L["out_w"] = (w + padding - size) // stride + 1
+            L["out_c"] = c
+        elif kind == "avgpool":
+            L.update(out_h=1, out_w=1, out_c=c)
+        elif kind == "softmax":
+            L.update(groups=gi(o, "groups", 1), temperature=gf(o, "temperature", 1.0),
+                     out_h=0, out_w=0, out_c=0, outputs=inputs)
+            # parse_softmax sets l.w/h/c from params but leaves out_* at zero
+        elif kind == "upsample":
+            stride = gi(o, "stride", 2)
+            L.update(stride=stride, scale=gf(o, "scale", 1.0),
+                     out_h=h * stride, out_w=w * stride, out_c=c)
+        elif kind == "shortcut":
+            frm = _atoi(o["from"])
+            if frm < 0:
+                frm = index + frm
+            src = layers[frm]
+            # make_shortcut_layer: (w,h,c) of the layer become those of `from`'s output, the
+            # output geometry is that of the running input.
+            L.update(index=frm, activation=o.get("activation", "linear"),
+                     alpha=gf(o, "alpha", 1.0), beta=gf(o, "beta", 1.0),
+                     h=src["out_h"], w=src["out_w"], c=src["out_c"],
+                     out_h=h, out_w=w, out_c=c)
+        elif kind == "route":
+            ids = []
+            for tok in o["layers"].split(","):
+                i = _atoi(tok)
+                ids.append(index + i if i < 0 else i)
+            first = layers[ids[0]]
+            oh, ow, oc = first["out_h"], first["out_w"], first["out_c"]
+            for i in ids[1:]:
+                nxt = layers[i]
+                if nxt["out_w"] == first["out_w"] and nxt["out_h"] == first["out_h"]:
+                    oc += nxt["out_c"]
+                else:
+                    oh = ow = oc = 0
+            sizes = [layers[i]["outputs"] for i in ids]
+            L.update(input_layers=ids, input_sizes=sizes, out_h=oh, out_w=ow, out_c=oc,
+                     outputs=sum(sizes), n=len(ids), h=0, w=0, c=0)
+            L["inputs"] = L["outputs"]  # make_route_layer leaves h/w/c at zero
+        elif kind == "yolo":
+            classes = gi(o, "classes", 20)
+            total = gi(o, "num", 1)
+            mask = [_atoi(t) for t in o["mask"].split(",")] if "mask" in o else list(range(total))
+            L.update(classes=classes, total=total, mask=mask, n=len(mask),
+                     c=len(mask) * (classes + 5), out_h=h, out_w=w,
+                     out_c=len(mask) * (classes + 5))
+            if "anchors" in o:
+                L["anchors"] = [_atof(t) for t in o["anchors"].split(",")]
+            L["outputs"] = h * w * L["out_c"]
+            if L["outputs"] != inputs:
+                raise ValueError("yolo layer: outputs != inputs")
+        if "outputs" not in L:
+            L["outputs"] = L["out_h"] * L["out_w"] * L["out_c"]
+        layers.append(L)
+        h, w, c, inputs = L["out_h"], L["out_w"], L["out_c"], L["outputs"]
+    net["layers"] = layers
+    net["n"] = len(layers)
+    net["outputs"] = layers[-1]["outputs"]
+    return net
+
+
+def conv_flops(L: dict) -> float:
+    """The reference's own operation count: examples/darknet.c:88, src/convolutional_layer.c:325."""
+    return 2.0 * L["n"] * L["size"] * L["size"] * (L["c"] // L["groups"]) * L["out_h"] * L["out_w"]

@@ -1,0 +1,67 @@
+"""forward_network over a parsed layer table, on the CPU restatement (test infrastructure).
+
+Restates the CPU loop of src/network.c:188-211: each layer's forward reads the previous
+layer's output (``net.input = l.output``), route and shortcut reach back into earlier outputs.
+"""
+from __future__ import annotations
+
+import numpy as np
+
+from . import cfg as _cfg
+from .cpu import Oracle
+
+
+class OracleNet:
+    def __init__(self, cfg_text: str, fast: bool = False):
+        self.net = _cfg.parse(cfg_text)
+        self.orc = Oracle(fast=fast)
+        self.params = {}
+
+    @property
+    def layers(self):
+        return self.net["layers"]
+
+    def set_conv(self, i, weights, biases, scales=None, mean=None, var=None):
+        self.params[i] = tuple(None if a is None else np.ascontiguousarray(a, np.float32)
+                               for a in (weights, biases, scales, mean, var))
+
+    def forward_layer(self, i, x, outs):
+        L = self.layers[i]
+        o = self.orc
+        t = L["type"]
+        b = L["batch"]
+        if t == "convolutional":
+            w, bi, sc, mu, var = self.params[i]
+            return o.conv(x.reshape(b, L["c"], L["h"], L["w"]), w, bi, sc, mu, var, n=L["n"],
+                          size=L["size"], stride=L["stride"], pad=L["pad"], groups=L["groups"],
+                          batch_normalize=L["batch_normalize"], activation=L["activation"],
+                          xnor=L["xnor"])
+        if t == "maxpool":
+            return o.maxpool(x.reshape(b, L["c"], L["h"], L["w"]), L["size"], L["stride"], L["pad"])[0]
+        if t == "upsample":
+            return o.upsample(x.reshape(b, L["c"], L["h"], L["w"]), L["stride"], L["scale"])
+        if t == "shortcut":
+            add = outs[L["index"]].reshape(b, L["c"], L["h"], L["w"])
+            return o.shortcut(x.reshape(b, L["out_c"], L["out_h"], L["out_w"]), add,
+                              L["alpha"], L["beta"], L["activation"])
+        if t == "route":
+            return o.route([outs[j].reshape(b, -1) for j in L["input_layers"]])
+        if t == "yolo":
+            return o.yolo(x.reshape(b, L["c"], L["h"], L["w"]), L["n"], L["classes"])
+        if t == "avgpool":
+            return o.avgpool(x.reshape(b, L["c"], L["h"], L["w"]))
+        if t == "softmax":
+            return o.softmax(x.reshape(b, -1), L["groups"], L["temperature"])
+        raise NotImplementedError(t)
+
+    def forward(self, x, upto=None):
+        """Returns the list of every layer's output (flattened per image: [batch, outputs])."""
+        outs = []
+        cur = np.ascontiguousarray(x, np.float32)
+        n = self.net["n"] if upto is None else upto
+        for i in range(n):
+            y = self.forward_layer(i, cur, outs)
+            y = np.ascontiguousarray(y).reshape(self.layers[i]["batch"], -1)
+            outs.append(y)
+            cur = y
+        return outs

@@ -1,0 +1,409 @@
+/*
+ * TEST INFRASTRUCTURE, NOT PRODUCT CODE (see oracle.h).
+ *
+ * CPU restatement of darknet's inference forward path.  Each function names the reference
+ * lines whose behaviour it restates; paths are relative to the reference tree.  The arithmetic
+ * is spelled out with explicit float/double conversions where the reference relies on C's
+ * implicit promotions, because those promotions decide the last bit of the result.
+ *
+ * Build: `make -C oracle oracle` (strict -O2 -ffp-contract=off for parity work, and an
+ * -Ofast -fopenmp twin that is only ever timed).
+ */
+#include "oracle.h"
+
+#include <float.h>
+#include <math.h>
+#include <string.h>
+
+/* ---- im2col: src/im2col.c:3-12 (pixel fetch with zero outside), :16-39 (unroll) -------- */
+void orc_im2col(const float *im, int channels, int height, int width,
+                int ksize, int stride, int pad, float *col)
+{
+    const int oh = (height + 2 * pad - ksize) / stride + 1;
+    const int ow = (width + 2 * pad - ksize) / stride + 1;
+    const int rows = channels * ksize * ksize;
+    for (int r = 0; r < rows; ++r) {
+        const int kx = r % ksize;
+        const int ky = (r / ksize) % ksize;
+        const int ch = r / (ksize * ksize);
+        float *dst = col + (long)r * oh * ow;
+        for (int oy = 0; oy < oh; ++oy) {
+            const int iy = oy * stride + ky - pad;
+            for (int ox = 0; ox < ow; ++ox) {
+                const int ix = ox * stride + kx - pad;
+                float v = 0.f;
+                if (iy >= 0 && ix >= 0 && iy < height && ix < width)
+                    v = im[ix + width * (iy + height * ch)];
+                dst[oy * ow + ox] = v;
+            }
+        }
+    }
+}
+
+/* ---- gemm_nn: src/gemm.c:74-89.  C += (alpha*A[i][k]) * B[k][:] with k as the outer loop,
+ * accumulated into C in memory in that order; rows are the only parallel axis (:80). -------- */
+void orc_gemm_nn(int M, int N, int K, float alpha, const float *A, int lda,
+                 const float *B, int ldb, float *C, int ldc)
+{
+#pragma omp parallel for
+    for (int i = 0; i < M; ++i) {
+        float *crow = C + (long)i * ldc;
+        for (int k = 0; k < K; ++k) {
+            const float a = alpha * A[(long)i * lda + k];
+            const float *brow = B + (long)k * ldb;
+            for (int j = 0; j < N; ++j) crow[j] += a * brow[j];
+        }
+    }
+}
+
+/* ---- normalize_cpu: src/blas.c:147-158.  sqrt is taken in double, the 1e-6f epsilon is
+ * added outside the root, and the float numerator is divided in double. ------------------- */
+void orc_normalize(float *x, const float *mean, const float *variance,
+                   int batch, int filters, int spatial)
+{
+    for (int b = 0; b < batch; ++b)
+        for (int f = 0; f < filters; ++f) {
+            const double denom = sqrt((double)variance[f]) + (double).000001f;
+            float *p = x + ((long)b * filters + f) * spatial;
+            for (int i = 0; i < spatial; ++i) {
+                const float num = p[i] - mean[f];
+                p[i] = (float)((double)num / denom);
+            }
+        }
+}
+
+/* ---- scale_bias / add_bias: src/convolutional_layer.c:423-433, :411-421 ----------------- */
+void orc_scale_bias(float *x, const float *scales, int batch, int n, int size)
+{
+    for (int b = 0; b < batch; ++b)
+        for (int f = 0; f < n; ++f) {
+            float *p = x + ((long)b * n + f) * size;
+            for (int i = 0; i < size; ++i) p[i] *= scales[f];
+        }
+}
+
+void orc_add_bias(float *x, const float *biases, int batch, int n, int size)
+{
+    for (int b = 0; b < batch; ++b)
+        for (int f = 0; f < n; ++f) {
+            float *p = x + ((long)b * n + f) * size;
+            for (int i = 0; i < size; ++i) p[i] += biases[f];
+        }
+}
+
+/* ---- activations: src/activations.h:18-52 (scalar forms), src/activations.c:65-106
+ * (dispatch + array loop).  Literals such as .1 are doubles in the reference, so the product is
+ * formed in double and rounded to float on return. --------------------------------------- */
+static float act_one(float x, int a)
+{
+    const double xd = (double)x;
+    switch (a) {
+    case 0: /* logistic */ return (float)(1. / (1. + exp((double)(-x))));
+    case 1: /* relu */ return x * (float)(x > 0);
+    case 2: /* relie */ return (x > 0) ? x : (float)(.01 * xd);
+    case 3: /* linear */ return x;
+    case 4: /* ramp */ return (float)((double)(x * (float)(x > 0)) + .1 * xd);
+    case 5: /* tanh */ {
+        const double e = exp((double)(2 * x));
+        return (float)((e - 1) / (e + 1));
+    }
+    case 6: /* plse */
+        if (x < -4) return (float)(.01 * (double)(x + 4));
+        if (x > 4) return (float)(.01 * (double)(x - 4) + 1);
+        return (float)(.125 * xd + .5);
+    case 7: /* leaky */ return (x > 0) ? x : (float)(.1 * xd);
+    case 8: /* elu */ return (float)((double)((float)(x >= 0) * x) + (x < 0) * (exp(xd) - 1));
+    case 9: /* loggy */ return (float)(2. / (1. + exp((double)(-x))) - 1);
+    case 10: /* stair */ {
+        const int n = (int)floor(xd);
+        if (n % 2 == 0) return (float)floor(xd / 2.);
+        return (float)((double)(x - n) + floor(xd / 2.));
+    }
+    case 11: /* hardtan */
+        if (x < -1) return -1;
+        if (x > 1) return 1;
+        return x;
+    case 12: /* lhtan */
+        if (x < 0) return (float)(.001 * xd);
+        if (x > 1) return (float)(.001 * (double)(x - 1) + 1);
+        return x;
+    case 13: /* selu */
+        return (float)((x >= 0) * 1.0507 * xd + (x < 0) * 1.0507 * 1.6732 * (exp(xd) - 1));
+    default: return 0;
+    }
+}
+
+void orc_activate_array(float *x, long n, int activation)
+{
+    for (long i = 0; i < n; ++i) x[i] = act_one(x[i], activation);
+}
+
+/* ---- binarize_weights: src/convolutional_layer.c:28-41.  Sequential sum of |w| carried in
+ * a float (each partial sum rounded), mean = sum/size, zero maps to -mean. ----------------- */
+void orc_binarize_weights(const float *weights, int n, int size, float *binary)
+{
+    for (int f = 0; f < n; ++f) {
+        const float *w = weights + (long)f * size;
+        float mean = 0;
+        for (int i = 0; i < size; ++i) mean = (float)((double)mean + fabs((double)w[i]));
+        mean = mean / size;
+        for (int i = 0; i < size; ++i) binary[(long)f * size + i] = (w[i] > 0) ? mean : -mean;
+    }
+}
+
+/* ---- binarize_cpu: src/convolutional_layer.c:43-49.  0, -0 and NaN all map to -1. -------- */
+void orc_binarize_input(const float *input, long n, float *binary)
+{
+    for (long i = 0; i < n; ++i) binary[i] = (input[i] > 0) ? 1.f : -1.f;
+}
+
+/* ---- forward_convolutional_layer: src/convolutional_layer.c:445-485, with the inference
+ * branch of forward_batchnorm_layer (src/batchnorm_layer.c:135-155) as its tail.  A 1x1 kernel
+ * feeds the image to the GEMM directly, whatever the stride (:468-469). ------------------- */
+void orc_conv_forward(const float *input, const float *weights, const float *biases,
+                      const float *scales, const float *rolling_mean,
+                      const float *rolling_variance, float *output, float *workspace,
+                      float *binary_weights, float *binary_input,
+                      int batch, int c, int h, int w, int n, int groups, int size, int stride,
+                      int pad, int batch_normalize, int activation, int xnor)
+{
+    const int out_h = (h + 2 * pad - size) / stride + 1;
+    const int out_w = (w + 2 * pad - size) / stride + 1;
+    const long outputs = (long)out_h * out_w * n;
+    const int cg = c / groups;
+    const long nweights = (long)cg * n * size * size;
+
+    memset(output, 0, sizeof(float) * (size_t)(outputs * batch));
+
+    if (xnor) {
+        orc_binarize_weights(weights, n, cg * size * size, binary_weights);
+        weights = binary_weights;
+        orc_binarize_input(input, (long)c * h * w * batch, binary_input);
+        input = binary_input;
+    }
+
+    const int M = n / groups;
+    const int K = size * size * cg;
+    const int N = out_w * out_h;
+    for (int b = 0; b < batch; ++b)
+        for (int g = 0; g < groups; ++g) {
+            const float *A = weights + g * (nweights / groups);
+            const float *im = input + ((long)b * groups + g) * cg * h * w;
+            float *C = output + ((long)b * groups + g) * N * M;
+            const float *B = im;
+            if (size != 1) {
+                orc_im2col(im, cg, h, w, size, stride, pad, workspace);
+                B = workspace;
+            }
+            orc_gemm_nn(M, N, K, 1.f, A, K, B, N, C, N);
+        }
+
+    if (batch_normalize) {
+        orc_normalize(output, rolling_mean, rolling_variance, batch, n, out_h * out_w);
+        orc_scale_bias(output, scales, batch, n, out_h * out_w);
+        orc_add_bias(output, biases, batch, n, out_h * out_w);
+    } else {
+        orc_add_bias(output, biases, batch, n, out_h * out_w);
+    }
+    orc_activate_array(output, outputs * batch, activation);
+}
+
+static double act_one_f64(double x, int a)
+{
+    switch (a) {
+    case 0: return 1. / (1. + exp(-x));
+    case 1: return x > 0 ? x : 0;
+    case 2: return x > 0 ? x : .01 * x;
+    case 3: return x;
+    case 4: return (x > 0 ? x : 0) + .1 * x;
+    case 5: return tanh(x);
+    case 7: return x > 0 ? x : .1 * x;
+    case 8: return x >= 0 ? x : exp(x) - 1;
+    case 9: return 2. / (1. + exp(-x)) - 1;
+    default: return (double)act_one((float)x, a);
+    }
+}
+
+/* Referee (no reference counterpart by design): cross-correlation, NCHW, zero padding, groups,
+ * as the definition reads, in double. */
+void orc_conv_forward_f64(const float *input, const float *weights, const float *biases,
+                          const float *scales, const float *rolling_mean,
+                          const float *rolling_variance, double *output,
+                          int batch, int c, int h, int w, int n, int groups, int size,
+                          int stride, int pad, int batch_normalize, int activation)
+{
+    const int out_h = (h + 2 * pad - size) / stride + 1;
+    const int out_w = (w + 2 * pad - size) / stride + 1;
+    const int cg = c / groups;
+    const int ng = n / groups;
+    /* A 1x1 kernel in the reference ignores stride and pad (it multiplies the raw image), which
+     * is only shape-consistent when stride==1 and pad==0; the referee keeps to that case. */
+#pragma omp parallel for collapse(2)
+    for (int b = 0; b < batch; ++b)
+        for (int f = 0; f < n; ++f) {
+            const int g = f / ng;
+            double denom = 1, mean = 0, sc = 1;
+            if (batch_normalize) {
+                denom = sqrt((double)rolling_variance[f]) + (double).000001f;
+                mean = rolling_mean[f];
+                sc = scales[f];
+            }
+            for (int oy = 0; oy < out_h; ++oy)
+                for (int ox = 0; ox < out_w; ++ox) {
+                    double acc = 0;
+                    for (int ci = 0; ci < cg; ++ci)
+                        for (int ky = 0; ky < size; ++ky) {
+                            const int iy = oy * stride + ky - pad;
+                            if (iy < 0 || iy >= h) continue;
+                            for (int kx = 0; kx < size; ++kx) {
+                                const int ix = ox * stride + kx - pad;
+                                if (ix < 0 || ix >= w) continue;
+                                acc += (double)weights[((long)(f * cg + ci) * size + ky) * size + kx] *
+                                       (double)input[(((long)b * c + g * cg + ci) * h + iy) * w + ix];
+                            }
+                        }
+                    if (batch_normalize) acc = (acc - mean) / denom * sc;
+                    acc += biases[f];
+                    output[(((long)b * n + f) * out_h + oy) * out_w + ox] = act_one_f64(acc, activation);
+                }
+        }
+}
+
+/* ---- forward_maxpool_layer: src/maxpool_layer.c:79-114.  Window origin is (-pad)/2 in C
+ * integer division; cells outside the image count as -FLT_MAX; the first strict maximum in
+ * row-major window order wins and its flat input index is recorded (-1 if none). ----------- */
+void orc_maxpool(const float *input, float *output, int *indexes, int batch, int c, int h,
+                 int w, int size, int stride, int pad)
+{
+    const int off = -pad / 2;
+    const int oh = (h + pad - size) / stride + 1;
+    const int ow = (w + pad - size) / stride + 1;
+    for (int b = 0; b < batch; ++b)
+        for (int k = 0; k < c; ++k)
+            for (int oy = 0; oy < oh; ++oy)
+                for (int ox = 0; ox < ow; ++ox) {
+                    float best = -FLT_MAX;
+                    int best_i = -1;
+                    for (int dy = 0; dy < size; ++dy)
+                        for (int dx = 0; dx < size; ++dx) {
+                            const int iy = off + oy * stride + dy;
+                            const int ix = off + ox * stride + dx;
+                            const int idx = ix + w * (iy + h * (k + b * c));
+                            const int inside = iy >= 0 && iy < h && ix >= 0 && ix < w;
+                            const float v = inside ? input[idx] : -FLT_MAX;
+                            if (v > best) {
+                                best = v;
+                                best_i = idx;
+                            }
+                        }
+                    const long o = ox + (long)ow * (oy + (long)oh * (k + (long)c * b));
+                    output[o] = best;
+                    indexes[o] = best_i;
+                }
+}
+
+/* ---- forward_upsample_layer (non-reverse): src/upsample_layer.c:68-76 -> upsample_cpu
+ * src/blas.c:334-349.  Nearest neighbour, every output written once as scale*in. ----------- */
+void orc_upsample(const float *input, float *output, int batch, int c, int h, int w,
+                  int stride, float scale)
+{
+    const int oh = h * stride, ow = w * stride;
+    for (int b = 0; b < batch; ++b)
+        for (int k = 0; k < c; ++k) {
+            const float *src = input + ((long)b * c + k) * h * w;
+            float *dst = output + ((long)b * c + k) * oh * ow;
+            for (int y = 0; y < oh; ++y)
+                for (int x = 0; x < ow; ++x) dst[(long)y * ow + x] = scale * src[(y / stride) * w + x / stride];
+        }
+}
+
+/* ---- shortcut_cpu: src/blas.c:68-92 (called from src/shortcut_layer.c:62-67 after the layer
+ * input was copied into out).  (w1,h1,c1) is the `add` tensor, (w2,h2,c2) is out. ---------- */
+void orc_shortcut(int batch, int w1, int h1, int c1, const float *add, int w2, int h2, int c2,
+                  float s1, float s2, float *out)
+{
+    int stride = w1 / w2;
+    int sample = w2 / w1;
+    if (stride < 1) stride = 1;
+    if (sample < 1) sample = 1;
+    const int mw = w1 < w2 ? w1 : w2;
+    const int mh = h1 < h2 ? h1 : h2;
+    const int mc = c1 < c2 ? c1 : c2;
+    for (int b = 0; b < batch; ++b)
+        for (int k = 0; k < mc; ++k)
+            for (int j = 0; j < mh; ++j)
+                for (int i = 0; i < mw; ++i) {
+                    const long o = i * sample + (long)w2 * (j * sample + (long)h2 * (k + (long)c2 * b));
+                    const long a = i * stride + (long)w1 * (j * stride + (long)h1 * (k + (long)c1 * b));
+                    out[o] = s1 * out[o] + s2 * add[a];
+                }
+}
+
+/* ---- forward_route_layer: src/route_layer.c:74-87, one source at a time: image j of the
+ * source lands at dst + dst_offset + j*dst_stride. ---------------------------------------- */
+void orc_route_copy(const float *src, int src_size, float *dst, int dst_stride, int dst_offset,
+                    int batch)
+{
+    for (int j = 0; j < batch; ++j)
+        memcpy(dst + dst_offset + (long)j * dst_stride, src + (long)j * src_size,
+               sizeof(float) * (size_t)src_size);
+}
+
+/* ---- forward_yolo_layer, inference part of the CPU build: src/yolo_layer.c:132-148 with
+ * entry_index :125-130.  Layout [b][anchor][entry][h][w]; entries 0,1 and 4..4+classes get the
+ * logistic, entries 2,3 stay raw. ---------------------------------------------------------- */
+void orc_yolo(const float *input, float *output, int batch, int w, int h, int n_anchors,
+              int classes)
+{
+    const long plane = (long)w * h;
+    const long per_anchor = plane * (4 + classes + 1);
+    const long outputs = per_anchor * n_anchors;
+    memcpy(output, input, sizeof(float) * (size_t)(outputs * batch));
+    for (int b = 0; b < batch; ++b)
+        for (int a = 0; a < n_anchors; ++a) {
+            float *base = output + b * outputs + a * per_anchor;
+            orc_activate_array(base, 2 * plane, 0);
+            orc_activate_array(base + 4 * plane, (1 + classes) * plane, 0);
+        }
+}
+
+/* ---- forward_avgpool_layer: src/avgpool_layer.c:40-55.  Sequential float sum, then divided
+ * by the int h*w converted to float. ------------------------------------------------------ */
+void orc_avgpool(const float *input, float *output, int batch, int c, int h, int w)
+{
+    const int area = h * w;
+    for (int b = 0; b < batch; ++b)
+        for (int k = 0; k < c; ++k) {
+            const float *p = input + ((long)b * c + k) * area;
+            float s = 0;
+            for (int i = 0; i < area; ++i) s += p[i];
+            output[k + b * c] = s / area;
+        }
+}
+
+/* ---- softmax / softmax_cpu: src/blas.c:305-321, :324-332 (called from
+ * src/softmax_layer.c:39-57 with n=inputs/groups, batch_offset=inputs, group_offset=n,
+ * stride=1).  The exponent's argument is formed in float, exp itself runs in double. ------- */
+static void softmax_one(const float *in, int n, float temp, int stride, float *out)
+{
+    float sum = 0;
+    float largest = -FLT_MAX;
+    for (int i = 0; i < n; ++i)
+        if (in[i * stride] > largest) largest = in[i * stride];
+    for (int i = 0; i < n; ++i) {
+        const float arg = in[i * stride] / temp - largest / temp;
+        const float e = (float)exp((double)arg);
+        sum += e;
+        out[i * stride] = e;
+    }
+    for (int i = 0; i < n; ++i) out[i * stride] /= sum;
+}
+
+void orc_softmax(const float *input, int n, int batch, int batch_offset, int groups,
+                 int group_offset, int stride, float temp, float *output)
+{
+    for (int b = 0; b < batch; ++b)
+        for (int g = 0; g < groups; ++g)
+            softmax_one(input + b * batch_offset + g * group_offset, n, temp, stride,
+                        output + b * batch_offset + g * group_offset);
+}

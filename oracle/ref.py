@@ -1,0 +1,131 @@
+"""Bindings to the compiled reference under oracle/_ref (test infrastructure, optional).
+
+``make -C oracle ref`` builds it where the reference tree is present; the built libraries travel
+with the working tree, the reference sources do not.  ``available()`` says whether it is there.
+"""
+from __future__ import annotations
+
+import ctypes as C
+import os
+
+import numpy as np
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+_F = C.POINTER(C.c_float)
+_I = C.POINTER(C.c_int)
+
+# LAYER_TYPE enum order of the reference (include/darknet.h:60-91)
+LAYER_TYPES = ["convolutional", "deconvolutional", "connected", "maxpool", "softmax", "detection",
+               "dropout", "crop", "route", "cost", "normalization", "avgpool", "local", "shortcut",
+               "active", "rnn", "gru", "lstm", "crnn", "batchnorm", "network", "xnor", "region",
+               "yolo", "iseg", "reorg", "upsample", "logxent", "l2norm", "blank"]
+ACTIVATIONS = ["logistic", "relu", "relie", "linear", "ramp", "tanh", "plse", "leaky", "elu",
+               "loggy", "stair", "hardtan", "lhtan", "selu"]
+
+_IV = ["type", "batch", "h", "w", "c", "out_h", "out_w", "out_c", "n", "size", "stride", "pad",
+       "groups", "batch_normalize", "activation", "binary", "xnor", "index", "inputs", "outputs",
+       "nweights", "classes", "total", "reverse", "workspace_floats", "nbiases", "truths",
+       "max_boxes"]
+_FV = ["alpha", "beta", "scale", "temperature"]
+
+
+def _path(variant: str) -> str:
+    return os.path.join(_HERE, "_ref", "librefh.so" if variant == "fast" else "librefh_o2.so")
+
+
+def available(variant: str = "o2") -> bool:
+    return os.path.exists(_path(variant))
+
+
+def raw(variant: str = "o2"):
+    """The reference library itself (plain-pointer functions such as im2col_cpu, gemm)."""
+    name = "libdarknet_ref.so" if variant == "fast" else "libdarknet_ref_o2.so"
+    return C.CDLL(os.path.join(_HERE, "_ref", name), mode=C.RTLD_GLOBAL)
+
+
+class RefNet:
+    """A network parsed and run by the compiled reference (CPU build)."""
+
+    def __init__(self, cfg_path: str, variant: str = "o2"):
+        raw(variant)
+        self.h = C.CDLL(_path(variant))
+        H = self.h
+        H.refh_load.restype = C.c_void_p
+        H.refh_load.argtypes = [C.c_char_p]
+        H.refh_free.argtypes = [C.c_void_p]
+        H.refh_nlayers.argtypes = [C.c_void_p]
+        H.refh_net_info.argtypes = [C.c_void_p, _I]
+        H.refh_layer_info.argtypes = [C.c_void_p, C.c_int, _I, _F]
+        H.refh_route_inputs.argtypes = [C.c_void_p, C.c_int, _I, _I, C.c_int]
+        H.refh_yolo_mask.argtypes = [C.c_void_p, C.c_int, _I, C.c_int, _F, C.c_int]
+        H.refh_set_conv.argtypes = [C.c_void_p, C.c_int] + [_F] * 5
+        H.refh_predict.restype = _F
+        H.refh_predict.argtypes = [C.c_void_p, _F]
+        for f in ("refh_layer_output", "refh_layer_weights", "refh_layer_binary_weights",
+                  "refh_layer_binary_input"):
+            getattr(H, f).restype = _F
+            getattr(H, f).argtypes = [C.c_void_p, C.c_int]
+        H.refh_layer_indexes.restype = _I
+        H.refh_layer_indexes.argtypes = [C.c_void_p, C.c_int]
+        H.refh_forward_layer.argtypes = [C.c_void_p, C.c_int, _F]
+        self.net = H.refh_load(cfg_path.encode())
+        if not self.net:
+            raise RuntimeError("reference failed to parse " + cfg_path)
+        iv = (C.c_int * 8)()
+        H.refh_net_info(self.net, iv)
+        self.n, self.batch, self.height, self.width, self.channels, self.inputs, self.outputs = list(iv)[:7]
+        self.layers = [self._layer(i) for i in range(self.n)]
+
+    def _layer(self, i):
+        iv = (C.c_int * len(_IV))()
+        fv = (C.c_float * len(_FV))()
+        self.h.refh_layer_info(self.net, i, iv, fv)
+        d = dict(zip(_IV, list(iv)))
+        d.update(zip(_FV, [float(v) for v in fv]))
+        d["type"] = LAYER_TYPES[d["type"]]
+        d["activation"] = ACTIVATIONS[d["activation"]]
+        if d["type"] == "route":
+            a = (C.c_int * 16)()
+            b = (C.c_int * 16)()
+            k = self.h.refh_route_inputs(self.net, i, a, b, 16)
+            d["input_layers"] = list(a)[:k]
+            d["input_sizes"] = list(b)[:k]
+        if d["type"] == "yolo":
+            m = (C.c_int * 32)()
+            an = (C.c_float * 64)()
+            k = self.h.refh_yolo_mask(self.net, i, m, 32, an, 64)
+            d["mask"] = list(m)[:k]
+            d["anchors"] = [float(v) for v in an][:2 * d["total"]]
+        return d
+
+    def set_conv(self, i, weights, biases, scales=None, mean=None, var=None):
+        p = lambda a: None if a is None else np.ascontiguousarray(a, np.float32).ctypes.data_as(_F)
+        self.h.refh_set_conv(self.net, i, p(weights), p(biases), p(scales), p(mean), p(var))
+
+    def predict(self, x):
+        x = np.ascontiguousarray(x, np.float32)
+        assert x.size == self.inputs * self.batch
+        self.h.refh_predict(self.net, x.ctypes.data_as(_F))
+        return [self.layer_output(i) for i in range(self.n)]
+
+    def layer_output(self, i):
+        L = self.layers[i]
+        p = self.h.refh_layer_output(self.net, i)
+        return np.ctypeslib.as_array(p, shape=(L["batch"], L["outputs"])).copy()
+
+    def layer_indexes(self, i):
+        L = self.layers[i]
+        p = self.h.refh_layer_indexes(self.net, i)
+        return np.ctypeslib.as_array(p, shape=(L["batch"], L["outputs"])).copy()
+
+    def forward_layer(self, i, x):
+        """Run layer i alone on input x; returns its output."""
+        x = np.ascontiguousarray(x, np.float32)
+        self.h.refh_forward_layer(self.net, i, x.ctypes.data_as(_F))
+        return self.layer_output(i)
+
+    def binary_tensors(self, i):
+        L = self.layers[i]
+        bw = np.ctypeslib.as_array(self.h.refh_layer_binary_weights(self.net, i), shape=(L["nweights"],)).copy()
+        bi = np.ctypeslib.as_array(self.h.refh_layer_binary_input(self.net, i), shape=(L["batch"], L["inputs"])).copy()
+        return bw, bi

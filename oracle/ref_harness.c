@@ -1,0 +1,132 @@
+/*
+ * Test infrastructure only.  A thin driver around the *compiled reference* (CPU build of
+ * pjreddie/darknet, linked from oracle/_ref/libdarknet_ref*.so).  It is compiled against the
+ * reference's own public header, found through -I at build time, so the struct layouts are the
+ * reference's; nothing from the reference is copied here.  It flattens what the tests need out
+ * of `network` / `layer` (include/darknet.h:115-422, :430-496 of the reference) into plain int
+ * and float arrays so Python can read them without mirroring those structs.
+ */
+#include "darknet.h"
+#include <string.h>
+
+enum { REFH_NI = 28, REFH_NF = 4 };
+
+network *refh_load(char *cfg)
+{
+    return parse_network_cfg(cfg);
+}
+
+void refh_free(network *net)
+{
+    free_network(net);
+}
+
+int refh_nlayers(network *net) { return net->n; }
+
+void refh_net_info(network *net, int *iv)
+{
+    iv[0] = net->n;
+    iv[1] = net->batch;
+    iv[2] = net->h;
+    iv[3] = net->w;
+    iv[4] = net->c;
+    iv[5] = net->inputs;
+    iv[6] = net->outputs;
+    iv[7] = (int)(net->layers[net->n - 1].type);
+}
+
+void refh_layer_info(network *net, int i, int *iv, float *fv)
+{
+    layer l = net->layers[i];
+    int k = 0;
+    iv[k++] = (int)l.type;          /* 0 */
+    iv[k++] = l.batch;              /* 1 */
+    iv[k++] = l.h;                  /* 2 */
+    iv[k++] = l.w;                  /* 3 */
+    iv[k++] = l.c;                  /* 4 */
+    iv[k++] = l.out_h;              /* 5 */
+    iv[k++] = l.out_w;              /* 6 */
+    iv[k++] = l.out_c;              /* 7 */
+    iv[k++] = l.n;                  /* 8 */
+    iv[k++] = l.size;               /* 9 */
+    iv[k++] = l.stride;             /* 10 */
+    iv[k++] = l.pad;                /* 11 */
+    iv[k++] = l.groups;             /* 12 */
+    iv[k++] = l.batch_normalize;    /* 13 */
+    iv[k++] = (int)l.activation;    /* 14 */
+    iv[k++] = l.binary;             /* 15 */
+    iv[k++] = l.xnor;               /* 16 */
+    iv[k++] = l.index;              /* 17 */
+    iv[k++] = l.inputs;             /* 18 */
+    iv[k++] = l.outputs;            /* 19 */
+    iv[k++] = l.nweights;           /* 20 */
+    iv[k++] = l.classes;            /* 21 */
+    iv[k++] = l.total;              /* 22 */
+    iv[k++] = l.reverse;            /* 23 */
+    iv[k++] = (int)(l.workspace_size / sizeof(float)); /* 24 */
+    iv[k++] = l.nbiases;            /* 25 */
+    iv[k++] = l.truths;             /* 26 */
+    iv[k++] = l.max_boxes;          /* 27 */
+    fv[0] = l.alpha;
+    fv[1] = l.beta;
+    fv[2] = l.scale;
+    fv[3] = l.temperature;
+}
+
+int refh_route_inputs(network *net, int i, int *layers, int *sizes, int cap)
+{
+    layer l = net->layers[i];
+    int j;
+    for (j = 0; j < l.n && j < cap; ++j) {
+        layers[j] = l.input_layers[j];
+        sizes[j] = l.input_sizes[j];
+    }
+    return l.n;
+}
+
+int refh_yolo_mask(network *net, int i, int *mask, int cap, float *anchors, int acap)
+{
+    layer l = net->layers[i];
+    int j;
+    for (j = 0; j < l.n && j < cap; ++j) mask[j] = l.mask[j];
+    for (j = 0; j < 2 * l.total && j < acap; ++j) anchors[j] = l.biases[j];
+    return l.n;
+}
+
+/* Overwrite a convolutional layer's parameters; NULL leaves a vector as it is. */
+void refh_set_conv(network *net, int i, const float *weights, const float *biases,
+                   const float *scales, const float *mean, const float *variance)
+{
+    layer l = net->layers[i];
+    if (weights) memcpy(l.weights, weights, sizeof(float) * (size_t)l.nweights);
+    if (biases) memcpy(l.biases, biases, sizeof(float) * (size_t)l.n);
+    if (l.batch_normalize) {
+        if (scales) memcpy(l.scales, scales, sizeof(float) * (size_t)l.n);
+        if (mean) memcpy(l.rolling_mean, mean, sizeof(float) * (size_t)l.n);
+        if (variance) memcpy(l.rolling_variance, variance, sizeof(float) * (size_t)l.n);
+    }
+}
+
+float *refh_predict(network *net, float *input)
+{
+    return network_predict(net, input);
+}
+
+float *refh_layer_output(network *net, int i) { return net->layers[i].output; }
+int *refh_layer_indexes(network *net, int i) { return net->layers[i].indexes; }
+float *refh_layer_weights(network *net, int i) { return net->layers[i].weights; }
+float *refh_layer_binary_weights(network *net, int i) { return net->layers[i].binary_weights; }
+float *refh_layer_binary_input(network *net, int i) { return net->layers[i].binary_input; }
+
+/* Run one layer's CPU forward on a caller-supplied input (used to inject an input into a
+ * single XNOR layer, where end-to-end comparison is ill-posed). */
+void refh_forward_layer(network *net, int i, float *input)
+{
+    network copy = *net;
+    layer l = net->layers[i];
+    copy.input = input;
+    copy.train = 0;
+    copy.truth = 0;
+    copy.index = i;
+    l.forward(l, copy);
+}
