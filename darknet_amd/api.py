@@ -1,0 +1,190 @@
+"""Python face of the native library, in the spirit of the reference's ``python/darknet.py``
+(a ctypes wrapper over ``libdarknet.so``, python/darknet.py:48-115): ``load_net``, ``predict`` and
+a small ``Network`` convenience class.  All arithmetic happens in the native library; numpy is
+only the host-side container.
+"""
+from __future__ import annotations
+
+import ctypes as C
+import os
+import tempfile
+
+import numpy as np
+
+from . import lib as _lib
+
+LAYER_TYPES = ["convolutional", "deconvolutional", "connected", "maxpool", "softmax", "detection",
+               "dropout", "crop", "route", "cost", "normalization", "avgpool", "local", "shortcut",
+               "active", "rnn", "gru", "lstm", "crnn", "batchnorm", "network", "xnor", "region",
+               "yolo", "iseg", "reorg", "upsample", "logxent", "l2norm", "blank"]
+ACTIVATIONS = ["logistic", "relu", "relie", "linear", "ramp", "tanh", "plse", "leaky", "elu",
+               "loggy", "stair", "hardtan", "lhtan", "selu"]
+_IV = ["type", "batch", "h", "w", "c", "out_h", "out_w", "out_c", "n", "size", "stride", "pad",
+       "groups", "batch_normalize", "activation", "binary", "xnor", "index", "inputs", "outputs",
+       "nweights", "classes", "total", "reverse", "workspace_floats", "nbiases", "truths",
+       "max_boxes"]
+_FV = ["alpha", "beta", "scale", "temperature"]
+_F = C.POINTER(C.c_float)
+
+
+def _fp(a):
+    return a.ctypes.data_as(_F)
+
+
+def set_gpu(n: int = 0):
+    _lib.load().cuda_set_device(n)
+
+
+def load_net(cfg: str, weights: str = "", clear: int = 0):
+    """python/darknet.py:78-80 - returns an opaque ``network *``."""
+    return _lib.load().load_network(cfg.encode(), weights.encode() if weights else None, clear)
+
+
+def predict(net, x: np.ndarray) -> np.ndarray:
+    """python/darknet.py:56-58 - network_predict on a float32 array; the result is copied."""
+    L = _lib.load()
+    x = np.ascontiguousarray(x, np.float32)
+    iv = (C.c_int * 8)()
+    L.network_info(net, iv)
+    out = L.network_predict(net, _fp(x))
+    n = iv[1] * _last_outputs(net)
+    return np.ctypeslib.as_array(out, shape=(n,)).copy()
+
+
+def _last_outputs(net):
+    L = _lib.load()
+    iv = (C.c_int * len(_IV))()
+    fv = (C.c_float * len(_FV))()
+    L.network_layer_info(net, L.network_num_layers(net) - 1, iv, fv)
+    return iv[_IV.index("outputs")]
+
+
+class DeviceArray:
+    """A float32 (or int32) device buffer made with the library's own allocator."""
+
+    def __init__(self, data=None, n=None, dtype=np.float32):
+        L = _lib.load()
+        self.dtype = np.dtype(dtype)
+        if data is not None:
+            data = np.ascontiguousarray(data, self.dtype)
+            n = data.size
+        self.n = int(n)
+        if self.dtype == np.float32:
+            self.ptr = L.hip_make_array(_fp(data) if data is not None else None, self.n)
+        else:
+            p = data.ctypes.data_as(C.POINTER(C.c_int)) if data is not None else None
+            self.ptr = L.hip_make_int_array(p, self.n)
+            if data is None:
+                L.fill_gpu(self.n, 0.0, self.ptr, 1)
+
+    def numpy(self, shape=None):
+        L = _lib.load()
+        out = np.empty(self.n, self.dtype)
+        if self.dtype == np.float32:
+            L.hip_pull_array(self.ptr, _fp(out), self.n)
+        else:
+            L.hip_pull_int_array(self.ptr, out.ctypes.data_as(C.POINTER(C.c_int)), self.n)
+        return out.reshape(shape) if shape is not None else out
+
+    def free(self):
+        if self.ptr:
+            _lib.load().hip_free(self.ptr)
+            self.ptr = None
+
+    def __del__(self):
+        try:
+            self.free()
+        except Exception:
+            pass
+
+
+class Network:
+    """A parsed network living on the GPU."""
+
+    def __init__(self, cfg_text: str = None, cfg_path: str = None, weights: str = ""):
+        self.L = _lib.load()
+        if cfg_path is None:
+            with tempfile.NamedTemporaryFile("w", suffix=".cfg", delete=False) as f:
+                f.write(cfg_text)
+                cfg_path = f.name
+            self._tmp = cfg_path
+        else:
+            self._tmp = None
+        self.net = load_net(cfg_path, weights, 0)
+        if self._tmp:
+            os.unlink(self._tmp)
+        iv = (C.c_int * 8)()
+        self.L.network_info(self.net, iv)
+        self.n, self.batch, self.h, self.w, self.c, self.inputs, self.outputs = list(iv)[:7]
+        self.layers = [self._layer(i) for i in range(self.n)]
+
+    def _layer(self, i):
+        iv = (C.c_int * len(_IV))()
+        fv = (C.c_float * len(_FV))()
+        self.L.network_layer_info(self.net, i, iv, fv)
+        d = dict(zip(_IV, list(iv)))
+        d.update(zip(_FV, [float(v) for v in fv]))
+        d["type"] = LAYER_TYPES[d["type"]]
+        d["activation"] = ACTIVATIONS[d["activation"]]
+        if d["type"] == "route":
+            a = (C.c_int * 16)()
+            b = (C.c_int * 16)()
+            k = self.L.network_route_inputs(self.net, i, a, b, 16)
+            d["input_layers"] = list(a)[:k]
+            d["input_sizes"] = list(b)[:k]
+        return d
+
+    def set_conv(self, i, weights, biases, scales=None, mean=None, var=None):
+        arrs = [None if a is None else np.ascontiguousarray(a, np.float32)
+                for a in (weights, biases, scales, mean, var)]
+        self.L.network_set_conv(self.net, i, *[None if a is None else _fp(a) for a in arrs])
+
+    def predict(self, x):
+        x = np.ascontiguousarray(x, np.float32)
+        assert x.size == self.inputs * self.batch, (x.size, self.inputs, self.batch)
+        out = self.L.network_predict(self.net, _fp(x))
+        last = self.layers[-1]
+        return np.ctypeslib.as_array(out, shape=(self.batch, last["outputs"])).copy()
+
+    def push_input(self, x):
+        """Place a batch in the network's device input buffer (for forward_device)."""
+        x = np.ascontiguousarray(x, np.float32)
+        assert x.size == self.inputs * self.batch
+        self._in = x
+        ptr = self.input_gpu()
+        self.L.hip_push_array(ptr, _fp(x), x.size)
+
+    def input_gpu(self):
+        return self.L.network_input_gpu(self.net)
+
+    def forward_device(self):
+        self.L.forward_network_device(self.net)
+
+    def synchronize(self):
+        self.L.hip_synchronize()
+
+    def layer_output(self, i):
+        L = self.layers[i]
+        p = self.L.layer_output_host(self.net, i)
+        return np.ctypeslib.as_array(p, shape=(L["batch"], L["outputs"])).copy()
+
+    def layer_indexes(self, i):
+        L = self.layers[i]
+        p = self.L.layer_indexes_host(self.net, i)
+        return np.ctypeslib.as_array(p, shape=(L["batch"], L["outputs"])).copy()
+
+    def conv_flops(self):
+        return float(self.L.network_conv_flops(self.net))
+
+    def save_weights(self, path):
+        self.L.save_weights(self.net, path.encode())
+
+    def load_weights(self, path):
+        self.L.load_weights(self.net, path.encode())
+
+    def free(self):
+        if self.net:
+            self.L.free_network(self.net)
+            self.net = None
+
+

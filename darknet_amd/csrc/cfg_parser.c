@@ -1,0 +1,345 @@
+/*
+ * cfg_parser.c - builds a network from a cfg file: parse_network_cfg and the per-section
+ * parsers of the layer types on the inference path.  Option names, defaults and the geometry
+ * hand-over between consecutive layers follow the reference (src/parser.c:742-889 and the
+ * parse_* functions cited below); hyper-parameters that only training reads are accepted and
+ * ignored.  A section type outside this path ends the process with a message naming it.
+ */
+#include <stdio.h>
+#include <stdlib.h>
+#include <string.h>
+
+#include "host.h"
+
+typedef struct {
+    int batch, inputs, h, w, c, index;
+    network *net;
+} size_params;
+
+static const char *TRAINING_ONLY_NET_KEYS[] = {
+    "learning_rate", "momentum", "decay", "notruth", "random", "adam", "B1", "B2", "eps", "max_crop",
+    "min_crop", "max_ratio", "min_ratio", "center", "clip", "angle", "aspect", "saturation", "exposure",
+    "hue", "policy", "burn_in", "power", "step", "scale", "steps", "scales", "gamma", "max_batches", 0};
+
+static const char *PER_LAYER_KEYS[] = {"truth", "onlyforward", "stopbackward", "dontsave", "dontload",
+                                       "numload", "dontloadscales", "learning_rate", "smooth", 0};
+
+/* src/parser.c:47-85 */
+static LAYER_TYPE section_type(const char *t)
+{
+    if (!strcmp(t, "[shortcut]")) return SHORTCUT;
+    if (!strcmp(t, "[yolo]")) return YOLO;
+    if (!strcmp(t, "[conv]") || !strcmp(t, "[convolutional]")) return CONVOLUTIONAL;
+    if (!strcmp(t, "[net]") || !strcmp(t, "[network]")) return NETWORK;
+    if (!strcmp(t, "[max]") || !strcmp(t, "[maxpool]")) return MAXPOOL;
+    if (!strcmp(t, "[avg]") || !strcmp(t, "[avgpool]")) return AVGPOOL;
+    if (!strcmp(t, "[soft]") || !strcmp(t, "[softmax]")) return SOFTMAX;
+    if (!strcmp(t, "[route]")) return ROUTE;
+    if (!strcmp(t, "[upsample]")) return UPSAMPLE;
+    return BLANK;
+}
+
+/* src/activations.c:44-63 */
+ACTIVATION get_activation(char *s)
+{
+    static const char *names[] = {"logistic", "relu", "relie", "linear", "ramp", "tanh", "plse",
+                                  "leaky", "elu", "loggy", "stair", "hardtan", "lhtan", "selu"};
+    int i;
+    for (i = 0; i < 14; ++i)
+        if (strcmp(s, names[i]) == 0) return (ACTIVATION)i;
+    fprintf(stderr, "Couldn't find activation function %s, going with ReLU\n", s);
+    return RELU;
+}
+
+char *get_activation_string(ACTIVATION a)
+{
+    static char *names[] = {"logistic", "relu", "relie", "linear", "ramp", "tanh", "plse",
+                            "leaky", "elu", "loggy", "stair", "hardtan", "lhtan", "selu"};
+    if ((int)a < 0 || (int)a > 13) return "relu";
+    return names[a];
+}
+
+/* src/network.c:110-175 */
+char *get_layer_string(LAYER_TYPE a)
+{
+    switch (a) {
+    case CONVOLUTIONAL: return "convolutional";
+    case MAXPOOL: return "maxpool";
+    case AVGPOOL: return "avgpool";
+    case SOFTMAX: return "softmax";
+    case ROUTE: return "route";
+    case SHORTCUT: return "shortcut";
+    case UPSAMPLE: return "upsample";
+    case YOLO: return "yolo";
+    default: return "none";
+    }
+}
+
+static void need_image(size_params p, const char *what)
+{
+    if (!(p.h && p.w && p.c)) {
+        char buf[128];
+        snprintf(buf, sizeof buf, "Layer before %s layer must output image.", what);
+        dn_fatal(buf);
+    }
+}
+
+/* src/parser.c:179-207 */
+static layer parse_convolutional(cfg_section *o, size_params p)
+{
+    int n = cfg_find_int(o, "filters", 1);
+    int size = cfg_find_int(o, "size", 1);
+    int stride = cfg_find_int(o, "stride", 1);
+    int pad = cfg_find_int_quiet(o, "pad", 0);
+    int padding = cfg_find_int_quiet(o, "padding", 0);
+    int groups = cfg_find_int_quiet(o, "groups", 1);
+    char *act;
+    int bn, binary, xnor;
+    layer l;
+    if (pad) padding = size / 2;
+    act = cfg_find_str(o, "activation", "logistic");
+    need_image(p, "convolutional");
+    bn = cfg_find_int_quiet(o, "batch_normalize", 0);
+    binary = cfg_find_int_quiet(o, "binary", 0);
+    xnor = cfg_find_int_quiet(o, "xnor", 0);
+    l = make_convolutional_layer(p.batch, p.h, p.w, p.c, n, groups, size, stride, padding, get_activation(act),
+                                 bn, binary, xnor, 0);
+    l.flipped = cfg_find_int_quiet(o, "flipped", 0);
+    (void)cfg_find_float_quiet(o, "dot", 0);
+    return l;
+}
+
+/* src/parser.c:483-498 */
+static layer parse_maxpool(cfg_section *o, size_params p)
+{
+    int stride = cfg_find_int(o, "stride", 1);
+    int size = cfg_find_int(o, "size", stride);
+    int padding = cfg_find_int_quiet(o, "padding", size - 1);
+    need_image(p, "maxpool");
+    return make_maxpool_layer(p.batch, p.h, p.w, p.c, size, stride, padding);
+}
+
+/* src/parser.c:500-511 */
+static layer parse_avgpool(cfg_section *o, size_params p)
+{
+    (void)o;
+    need_image(p, "avgpool");
+    return make_avgpool_layer(p.batch, p.w, p.h, p.c);
+}
+
+/* src/parser.c:270-283 (tree and spatial modes are outside this path) */
+static layer parse_softmax(cfg_section *o, size_params p)
+{
+    int groups = cfg_find_int_quiet(o, "groups", 1);
+    layer l = make_softmax_layer(p.batch, p.inputs, groups);
+    l.temperature = cfg_find_float_quiet(o, "temperature", 1);
+    if (cfg_find_str(o, "tree", 0)) dn_fatal("softmax layer: tree= is not supported");
+    l.w = p.w;
+    l.h = p.h;
+    l.c = p.c;
+    if (cfg_find_float_quiet(o, "spatial", 0) != 0) dn_fatal("softmax layer: spatial= is not supported");
+    l.noloss = cfg_find_int_quiet(o, "noloss", 0);
+    return l;
+}
+
+/* src/parser.c:539-556 */
+static layer parse_shortcut(cfg_section *o, size_params p, network *net)
+{
+    char *from = cfg_find(o, "from");
+    int index;
+    layer src, s;
+    if (!from) dn_fatal("Shortcut layer must specify from");
+    index = atoi(from);
+    if (index < 0) index = p.index + index;
+    if (index < 0 || index >= p.index) dn_fatal("Shortcut layer: from is out of range");
+    src = net->layers[index];
+    s = make_shortcut_layer(p.batch, index, p.w, p.h, p.c, src.out_w, src.out_h, src.out_c);
+    s.activation = get_activation(cfg_find_str(o, "activation", "linear"));
+    s.alpha = cfg_find_float_quiet(o, "alpha", 1);
+    s.beta = cfg_find_float_quiet(o, "beta", 1);
+    return s;
+}
+
+/* src/parser.c:592-599 */
+static layer parse_upsample(cfg_section *o, size_params p)
+{
+    int stride = cfg_find_int(o, "stride", 2);
+    layer l = make_upsample_layer(p.batch, p.w, p.h, p.c, stride);
+    l.scale = cfg_find_float_quiet(o, "scale", 1);
+    return l;
+}
+
+static int count_commas(const char *s)
+{
+    int n = 1;
+    for (; *s; ++s)
+        if (*s == ',') ++n;
+    return n;
+}
+
+/* src/parser.c:601-640 */
+static layer parse_route(cfg_section *o, size_params p, network *net)
+{
+    char *l = cfg_find(o, "layers");
+    int n, i, *layers, *sizes;
+    layer r, first;
+    if (!l) dn_fatal("Route Layer must specify input layers");
+    n = count_commas(l);
+    layers = (int *)dn_calloc((size_t)n, sizeof(int));
+    sizes = (int *)dn_calloc((size_t)n, sizeof(int));
+    for (i = 0; i < n; ++i) {
+        int index = atoi(l);
+        char *next = strchr(l, ',');
+        l = next ? next + 1 : l + strlen(l);
+        if (index < 0) index = p.index + index;
+        if (index < 0 || index >= p.index) dn_fatal("Route layer: input layer out of range");
+        layers[i] = index;
+        sizes[i] = net->layers[index].outputs;
+    }
+    r = make_route_layer(p.batch, n, layers, sizes);
+    first = net->layers[layers[0]];
+    r.out_w = first.out_w;
+    r.out_h = first.out_h;
+    r.out_c = first.out_c;
+    for (i = 1; i < n; ++i) {
+        layer next = net->layers[layers[i]];
+        if (next.out_w == first.out_w && next.out_h == first.out_h)
+            r.out_c += next.out_c;
+        else
+            r.out_h = r.out_w = r.out_c = 0;
+    }
+    return r;
+}
+
+/* src/parser.c:285-342 */
+static layer parse_yolo(cfg_section *o, size_params p)
+{
+    int classes = cfg_find_int(o, "classes", 20);
+    int total = cfg_find_int(o, "num", 1);
+    int num = total;
+    char *a = cfg_find_str(o, "mask", 0);
+    int *mask = 0;
+    layer l;
+    if (a) {
+        int n = count_commas(a), i;
+        mask = (int *)dn_calloc((size_t)n, sizeof(int));
+        for (i = 0; i < n; ++i) {
+            char *next = strchr(a, ',');
+            mask[i] = atoi(a);
+            a = next ? next + 1 : a + strlen(a);
+        }
+        num = n;
+    }
+    l = make_yolo_layer(p.batch, p.w, p.h, num, total, mask, classes);
+    if (l.outputs != p.inputs) dn_fatal("yolo layer: the layer before it must output n*(classes+5) channels");
+    l.max_boxes = cfg_find_int_quiet(o, "max", 90);
+    l.jitter = cfg_find_float(o, "jitter", .2f);
+    l.ignore_thresh = cfg_find_float(o, "ignore_thresh", .5f);
+    l.truth_thresh = cfg_find_float(o, "truth_thresh", 1);
+    l.random = cfg_find_int_quiet(o, "random", 0);
+    if (cfg_find_str(o, "map", 0)) dn_fatal("yolo layer: map= is not supported");
+    a = cfg_find_str(o, "anchors", 0);
+    if (a) {
+        int n = count_commas(a), i;
+        for (i = 0; i < n && i < 2 * total; ++i) {
+            char *next = strchr(a, ',');
+            l.biases[i] = (float)atof(a);
+            a = next ? next + 1 : a + strlen(a);
+        }
+    }
+    return l;
+}
+
+/* src/parser.c:655-679: batch is divided by subdivisions and fixed here for the network's life */
+static void parse_net_options(cfg_section *o, network *net)
+{
+    int subdivs, i;
+    net->batch = cfg_find_int(o, "batch", 1);
+    subdivs = cfg_find_int(o, "subdivisions", 1);
+    net->time_steps = cfg_find_int_quiet(o, "time_steps", 1);
+    if (subdivs < 1) subdivs = 1;
+    net->batch /= subdivs;
+    net->batch *= net->time_steps;
+    net->subdivisions = subdivs;
+    net->h = cfg_find_int_quiet(o, "height", 0);
+    net->w = cfg_find_int_quiet(o, "width", 0);
+    net->c = cfg_find_int_quiet(o, "channels", 0);
+    net->inputs = cfg_find_int_quiet(o, "inputs", net->h * net->w * net->c);
+    if (!net->inputs && !(net->h && net->w && net->c)) dn_fatal("No input parameters supplied");
+    if (net->batch < 1) dn_fatal("batch/subdivisions must be at least 1");
+    for (i = 0; TRAINING_ONLY_NET_KEYS[i]; ++i) (void)cfg_find(o, TRAINING_ONLY_NET_KEYS[i]);
+}
+
+network *parse_network_cfg(char *filename)
+{
+    cfg_file *f = cfg_read(filename);
+    network *net;
+    size_params p;
+    int count, i;
+    if (f->n < 1) dn_fatal("Config file has no sections");
+    if (section_type(f->sections[0].type) != NETWORK) dn_fatal("First section must be [net] or [network]");
+    net = make_network(f->n - 1);
+    net->gpu_index = gpu_index;
+    if (gpu_index < 0) dn_fatal("this library has no CPU path: gpu_index must name a device");
+    hip_set_device(gpu_index);
+    parse_net_options(&f->sections[0], net);
+    cfg_report_unused(&f->sections[0]);
+    p.h = net->h;
+    p.w = net->w;
+    p.c = net->c;
+    p.inputs = net->inputs;
+    p.batch = net->batch;
+    p.net = net;
+    if (dn_verbose) fprintf(stderr, "layer     filters    size              input                output\n");
+    for (count = 0; count < net->n; ++count) {
+        cfg_section *o = &f->sections[count + 1];
+        LAYER_TYPE lt = section_type(o->type);
+        layer l;
+        p.index = count;
+        if (dn_verbose) fprintf(stderr, "%5d ", count);
+        switch (lt) {
+        case CONVOLUTIONAL: l = parse_convolutional(o, p); break;
+        case MAXPOOL: l = parse_maxpool(o, p); break;
+        case AVGPOOL: l = parse_avgpool(o, p); break;
+        case SOFTMAX: l = parse_softmax(o, p); break;
+        case ROUTE: l = parse_route(o, p, net); break;
+        case UPSAMPLE: l = parse_upsample(o, p); break;
+        case SHORTCUT: l = parse_shortcut(o, p, net); break;
+        case YOLO: l = parse_yolo(o, p); break;
+        default: {
+            char buf[256];
+            snprintf(buf, sizeof buf, "layer type %s (section %d) is outside the convolution forward path this "
+                     "library implements", o->type, count);
+            dn_fatal(buf);
+            memset(&l, 0, sizeof l);
+        }
+        }
+        l.truth = cfg_find_int_quiet(o, "truth", 0);
+        l.onlyforward = cfg_find_int_quiet(o, "onlyforward", 0);
+        l.dontload = cfg_find_int_quiet(o, "dontload", 0);
+        l.numload = cfg_find_int_quiet(o, "numload", 0);
+        l.dontloadscales = cfg_find_int_quiet(o, "dontloadscales", 0);
+        for (i = 0; PER_LAYER_KEYS[i]; ++i) (void)cfg_find(o, PER_LAYER_KEYS[i]);
+        cfg_report_unused(o);
+        net->layers[count] = l;
+        p.h = l.out_h;
+        p.w = l.out_w;
+        p.c = l.out_c;
+        p.inputs = l.outputs;
+    }
+    cfg_free(f);
+    {
+        layer out = get_network_output_layer(net);
+        layer *last = &net->layers[net->n - 1];
+        net->outputs = out.outputs;
+        net->truths = out.outputs;
+        if (last->truths) net->truths = last->truths;
+        /* the host sees the last layer's output after every forward (src/network.c:786) */
+        if (!last->output) last->output = (float *)dn_calloc((size_t)last->outputs * last->batch, sizeof(float));
+        net->output = last->output;
+        net->output_gpu = last->output_gpu;
+    }
+    net->input = (float *)dn_calloc((size_t)net->inputs * net->batch, sizeof(float));
+    net->input_gpu = hip_make_array(net->input, (size_t)net->inputs * net->batch);
+    return net;
+}

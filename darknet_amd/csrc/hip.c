@@ -1,0 +1,191 @@
+/*
+ * hip.c - device shim of the darknet forward path on HIP.  Takes the place of the reference's
+ * src/cuda.c: device selection, allocation, host<->device copies, error check.  There is no
+ * BLAS/DNN handle here on purpose: the convolution is this library's own kernel.
+ */
+#define __HIP_PLATFORM_AMD__ 1
+#include <hip/hip_runtime_api.h>
+
+#include <math.h>
+#include <stdio.h>
+#include <stdlib.h>
+#include <string.h>
+
+#include "hip.h"
+
+int gpu_index = 0;
+
+static hipStream_t g_stream = 0;
+static char g_name[640];
+
+void dn_fatal(const char *msg)
+{
+    fprintf(stderr, "darknet-hip: %s\n", msg);
+    fflush(stderr);
+    exit(-1);
+}
+
+void hip_check_error(int status)
+{
+    if (status != hipSuccess) {
+        char buf[320];
+        snprintf(buf, sizeof buf, "HIP Error: %s", hipGetErrorString((hipError_t)status));
+        dn_fatal(buf);
+    }
+    hipError_t prev = hipGetLastError();
+    if (prev != hipSuccess) {
+        char buf[320];
+        snprintf(buf, sizeof buf, "HIP Error Prev: %s", hipGetErrorString(prev));
+        dn_fatal(buf);
+    }
+}
+
+void dn_check_launch(const char *what)
+{
+    hipError_t e = hipPeekAtLastError();
+    if (e != hipSuccess) {
+        char buf[384];
+        snprintf(buf, sizeof buf, "kernel launch failed (%s): %s", what, hipGetErrorString(e));
+        dn_fatal(buf);
+    }
+}
+
+void hip_set_device(int n)
+{
+    gpu_index = n;
+    hip_check_error(hipSetDevice(n));
+}
+
+int hip_get_device(void)
+{
+    int n = 0;
+    hip_check_error(hipGetDevice(&n));
+    return n;
+}
+
+const char *hip_device_name(void)
+{
+    hipDeviceProp_t p;
+    hip_check_error(hipGetDeviceProperties(&p, hip_get_device()));
+    snprintf(g_name, sizeof g_name, "%s (%s, %d CUs)", p.name, p.gcnArchName, p.multiProcessorCount);
+    return g_name;
+}
+
+void *hip_get_stream(void) { return (void *)g_stream; }
+void hip_set_stream(void *stream) { g_stream = (hipStream_t)stream; }
+
+void hip_synchronize(void)
+{
+    hip_check_error(hipStreamSynchronize(g_stream));
+}
+
+float *hip_make_array(float *x, size_t n)
+{
+    float *x_gpu = 0;
+    size_t size = sizeof(float) * (n ? n : 1);
+    hip_check_error(hipMalloc((void **)&x_gpu, size));
+    if (!x_gpu) dn_fatal("hipMalloc returned a null pointer");
+    if (x) {
+        hip_check_error(hipMemcpy(x_gpu, x, sizeof(float) * n, hipMemcpyHostToDevice));
+    } else {
+        hip_check_error(hipMemset(x_gpu, 0, size));
+    }
+    return x_gpu;
+}
+
+int *hip_make_int_array(int *x, size_t n)
+{
+    int *x_gpu = 0;
+    size_t size = sizeof(int) * (n ? n : 1);
+    hip_check_error(hipMalloc((void **)&x_gpu, size));
+    if (!x_gpu) dn_fatal("hipMalloc returned a null pointer");
+    if (x) hip_check_error(hipMemcpy(x_gpu, x, sizeof(int) * n, hipMemcpyHostToDevice));
+    return x_gpu;
+}
+
+void hip_free(float *x_gpu)
+{
+    hip_check_error(hipFree(x_gpu));
+}
+
+/* The copies are synchronous, like the reference's cudaMemcpy (src/cuda.c:153-165); work
+ * queued on a non-null stream is drained first so the copy sees it. */
+void hip_push_array(float *x_gpu, float *x, size_t n)
+{
+    if (g_stream) hip_check_error(hipStreamSynchronize(g_stream));
+    hip_check_error(hipMemcpy(x_gpu, x, sizeof(float) * n, hipMemcpyHostToDevice));
+}
+
+void hip_pull_array(float *x_gpu, float *x, size_t n)
+{
+    if (g_stream) hip_check_error(hipStreamSynchronize(g_stream));
+    hip_check_error(hipMemcpy(x, x_gpu, sizeof(float) * n, hipMemcpyDeviceToHost));
+}
+
+void hip_pull_int_array(int *x_gpu, int *x, size_t n)
+{
+    if (g_stream) hip_check_error(hipStreamSynchronize(g_stream));
+    hip_check_error(hipMemcpy(x, x_gpu, sizeof(int) * n, hipMemcpyDeviceToHost));
+}
+
+float hip_mag_array(float *x_gpu, size_t n)
+{
+    float *tmp = (float *)calloc(n ? n : 1, sizeof(float));
+    double sum = 0;
+    size_t i;
+    hip_pull_array(x_gpu, tmp, n);
+    for (i = 0; i < n; ++i) sum += (double)tmp[i] * tmp[i];
+    free(tmp);
+    return (float)sqrt(sum);
+}
+
+float hip_compare(float *x_gpu, float *x, size_t n, char *s)
+{
+    float *tmp = (float *)calloc(n ? n : 1, sizeof(float));
+    double err = 0;
+    size_t i;
+    hip_pull_array(x_gpu, tmp, n);
+    for (i = 0; i < n; ++i) {
+        double d = (double)tmp[i] - x[i];
+        err += d * d;
+    }
+    free(tmp);
+    printf("Error %s: %f\n", s, sqrt(err / (double)(n ? n : 1)));
+    return (float)err;
+}
+
+void *hip_event_create(void)
+{
+    hipEvent_t ev;
+    hip_check_error(hipEventCreate(&ev));
+    return (void *)ev;
+}
+
+void hip_event_record(void *ev)
+{
+    hip_check_error(hipEventRecord((hipEvent_t)ev, g_stream));
+}
+
+float hip_event_elapsed_ms(void *start, void *stop)
+{
+    float ms = 0;
+    hip_check_error(hipEventSynchronize((hipEvent_t)stop));
+    hip_check_error(hipEventElapsedTime(&ms, (hipEvent_t)start, (hipEvent_t)stop));
+    return ms;
+}
+
+void hip_event_destroy(void *ev)
+{
+    hip_check_error(hipEventDestroy((hipEvent_t)ev));
+}
+
+/* The reference's spellings, for objects compiled against its src/cuda.h. */
+void cuda_set_device(int n) { hip_set_device(n); }
+int cuda_get_device(void) { return hip_get_device(); }
+float *cuda_make_array(float *x, size_t n) { return hip_make_array(x, n); }
+int *cuda_make_int_array(int *x, size_t n) { return hip_make_int_array(x, n); }
+void cuda_free(float *x_gpu) { hip_free(x_gpu); }
+void cuda_push_array(float *x_gpu, float *x, size_t n) { hip_push_array(x_gpu, x, n); }
+void cuda_pull_array(float *x_gpu, float *x, size_t n) { hip_pull_array(x_gpu, x, n); }
+float cuda_mag_array(float *x_gpu, size_t n) { return hip_mag_array(x_gpu, n); }
+float cuda_compare(float *x_gpu, float *x, size_t n, char *s) { return hip_compare(x_gpu, x, n, s); }

@@ -1,0 +1,24 @@
+/*
+ * hip.h - internal face of the device shim (hip.c) and of the kernel launchers.
+ * The exported C-ABI is include/darknet_hip.h; this header only adds what the library's own
+ * translation units share.
+ */
+#ifndef DN_HIP_INTERNAL_H
+#define DN_HIP_INTERNAL_H
+
+#include "darknet_hip.h"
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* Prints `msg` and ends the process, as the reference's error() does (src/utils.c:253-258). */
+void dn_fatal(const char *msg);
+/* Checks the sticky launch error after a kernel launch (check_error(cudaPeekAtLastError())
+ * follows every launch in the reference, e.g. src/blas_kernels.cu:27). */
+void dn_check_launch(const char *what);
+
+#ifdef __cplusplus
+}
+#endif
+#endif

@@ -1,0 +1,249 @@
+/*
+ * network.c - the inference runtime: forward_network / network_predict and the small helpers
+ * around them.  Restates the GPU branch of the reference's src/network.c for net.train == 0.
+ */
+#include <stdio.h>
+#include <stdlib.h>
+#include <string.h>
+
+#include "host.h"
+
+/* src/network.c:177-186 */
+network *make_network(int n)
+{
+    network *net = (network *)dn_calloc(1, sizeof(network));
+    net->n = n;
+    net->layers = (layer *)dn_calloc((size_t)n, sizeof(layer));
+    net->seen = (size_t *)dn_calloc(1, sizeof(size_t));
+    return net;
+}
+
+/* src/network.c:699-716 */
+void free_network(network *net)
+{
+    int i;
+    if (!net) return;
+    for (i = 0; i < net->n; ++i) free_layer(net->layers[i]);
+    free(net->layers);
+    free(net->input);
+    free(net->seen);
+    if (net->input_gpu) hip_free(net->input_gpu);
+    free(net);
+}
+
+/* src/network.c:689-697 */
+layer get_network_output_layer(network *net)
+{
+    int i;
+    for (i = net->n - 1; i >= 0; --i)
+        if (net->layers[i].type != COST) break;
+    if (i < 0) dn_fatal("network has no layers");
+    return net->layers[i];
+}
+
+float *network_output(network *net) { return get_network_output_layer(net).output; }
+int network_width(network *net) { return net->w; }
+int network_height(network *net) { return net->h; }
+
+/* src/network.c:339-356.  Buffers were sized at parse time, so the batch can only shrink. */
+void set_batch_network(network *net, int b)
+{
+    int i;
+    if (b < 1) dn_fatal("set_batch_network: batch must be at least 1");
+    for (i = 0; i < net->n; ++i)
+        if (b > net->layers[i].batch && net->layers[i].batch > 0 && b > net->batch)
+            dn_fatal("set_batch_network: buffers were allocated for a smaller batch (batch is fixed at parse time)");
+    net->batch = b;
+    for (i = 0; i < net->n; ++i) net->layers[i].batch = b;
+}
+
+/* The layer loop of src/network.c:773-785 without the copies around it. */
+void forward_network_device(network *netp)
+{
+    network net = *netp;
+    int i;
+    net.train = 0;
+    for (i = 0; i < net.n; ++i) {
+        layer l = net.layers[i];
+        net.index = i;
+        if (!l.forward_gpu) dn_fatal("layer without a GPU forward");
+        l.forward_gpu(l, net);
+        net.input_gpu = l.output_gpu;
+    }
+}
+
+/* src/network.c:1123-1127 */
+void pull_network_output(network *net)
+{
+    layer l = get_network_output_layer(net);
+    hip_pull_array(l.output_gpu, l.output, (size_t)l.outputs * l.batch);
+}
+
+/* src/network.c:762-788 */
+void forward_network_gpu(network *netp)
+{
+    network net = *netp;
+    int i;
+    hip_set_device(net.gpu_index);
+    hip_push_array(net.input_gpu, net.input, (size_t)net.inputs * net.batch);
+    forward_network_device(netp);
+    for (i = 0; i < net.n - 1; ++i) {
+        layer l = net.layers[i];
+        if (l.type == YOLO) hip_pull_array(l.output_gpu, l.output, (size_t)l.batch * l.outputs);
+    }
+    pull_network_output(netp);
+}
+
+/* src/network.c:188-211 */
+void forward_network(network *net)
+{
+    if (net->gpu_index < 0) dn_fatal("forward_network: this library has no CPU path (gpu_index < 0)");
+    forward_network_gpu(net);
+}
+
+/* src/network.c:497-508 */
+float *network_predict(network *net, float *input)
+{
+    network orig = *net;
+    float *out;
+    net->input = input;
+    net->truth = 0;
+    net->train = 0;
+    net->delta = 0;
+    forward_network(net);
+    out = net->output;
+    *net = orig;
+    return out;
+}
+
+/* src/network.c:53-63 */
+network *load_network(char *cfg, char *weights, int clear)
+{
+    network *net = parse_network_cfg(cfg);
+    if (weights && weights[0] != 0) load_weights(net, weights);
+    if (clear) *net->seen = 0;
+    return net;
+}
+
+/* ---- additions ---------------------------------------------------------------------------- */
+float *layer_output_host(network *net, int i)
+{
+    layer *l;
+    if (i < 0 || i >= net->n) dn_fatal("layer_output_host: layer index out of range");
+    l = &net->layers[i];
+    if (!l->output) {
+        l->output = (float *)dn_calloc((size_t)l->outputs * l->batch, sizeof(float));
+        if (i == net->n - 1) net->output = l->output;
+    }
+    hip_pull_array(l->output_gpu, l->output, (size_t)l->outputs * l->batch);
+    return l->output;
+}
+
+int *layer_indexes_host(network *net, int i)
+{
+    layer *l;
+    if (i < 0 || i >= net->n) dn_fatal("layer_indexes_host: layer index out of range");
+    l = &net->layers[i];
+    if (!l->indexes_gpu) dn_fatal("layer_indexes_host: layer has no indexes");
+    if (!l->indexes) l->indexes = (int *)dn_calloc((size_t)l->outputs * l->batch, sizeof(int));
+    hip_pull_int_array(l->indexes_gpu, l->indexes, (size_t)l->outputs * l->batch);
+    return l->indexes;
+}
+
+void network_set_conv(network *net, int i, const float *weights, const float *biases, const float *scales,
+                      const float *rolling_mean, const float *rolling_variance)
+{
+    layer l;
+    if (i < 0 || i >= net->n || net->layers[i].type != CONVOLUTIONAL)
+        dn_fatal("network_set_conv: not a convolutional layer");
+    l = net->layers[i];
+    if (weights) memcpy(l.weights, weights, sizeof(float) * (size_t)l.nweights);
+    if (biases) memcpy(l.biases, biases, sizeof(float) * (size_t)l.n);
+    if (l.batch_normalize) {
+        if (scales) memcpy(l.scales, scales, sizeof(float) * (size_t)l.n);
+        if (rolling_mean) memcpy(l.rolling_mean, rolling_mean, sizeof(float) * (size_t)l.n);
+        if (rolling_variance) memcpy(l.rolling_variance, rolling_variance, sizeof(float) * (size_t)l.n);
+    }
+    push_convolutional_layer(l);
+}
+
+int network_num_layers(network *net) { return net->n; }
+float *network_input_gpu(network *net) { return net->input_gpu; }
+
+void network_info(network *net, int *iv)
+{
+    iv[0] = net->n;
+    iv[1] = net->batch;
+    iv[2] = net->h;
+    iv[3] = net->w;
+    iv[4] = net->c;
+    iv[5] = net->inputs;
+    iv[6] = net->outputs;
+}
+
+void network_layer_info(network *net, int i, int *iv, float *fv)
+{
+    layer l;
+    int k = 0;
+    if (i < 0 || i >= net->n) dn_fatal("network_layer_info: layer index out of range");
+    l = net->layers[i];
+    iv[k++] = (int)l.type;
+    iv[k++] = l.batch;
+    iv[k++] = l.h;
+    iv[k++] = l.w;
+    iv[k++] = l.c;
+    iv[k++] = l.out_h;
+    iv[k++] = l.out_w;
+    iv[k++] = l.out_c;
+    iv[k++] = l.n;
+    iv[k++] = l.size;
+    iv[k++] = l.stride;
+    iv[k++] = l.pad;
+    iv[k++] = l.groups;
+    iv[k++] = l.batch_normalize;
+    iv[k++] = (int)l.activation;
+    iv[k++] = l.binary;
+    iv[k++] = l.xnor;
+    iv[k++] = l.index;
+    iv[k++] = l.inputs;
+    iv[k++] = l.outputs;
+    iv[k++] = l.nweights;
+    iv[k++] = l.classes;
+    iv[k++] = l.total;
+    iv[k++] = l.reverse;
+    iv[k++] = (int)(l.workspace_size / sizeof(float));
+    iv[k++] = l.nbiases;
+    iv[k++] = l.truths;
+    iv[k++] = l.max_boxes;
+    fv[0] = l.alpha;
+    fv[1] = l.beta;
+    fv[2] = l.scale;
+    fv[3] = l.temperature;
+}
+
+int network_route_inputs(network *net, int i, int *layers, int *sizes, int cap)
+{
+    layer l;
+    int j;
+    if (i < 0 || i >= net->n) dn_fatal("network_route_inputs: layer index out of range");
+    l = net->layers[i];
+    if (l.type != ROUTE) return 0;
+    for (j = 0; j < l.n && j < cap; ++j) {
+        layers[j] = l.input_layers[j];
+        sizes[j] = l.input_sizes[j];
+    }
+    return l.n;
+}
+
+/* numops of the reference (examples/darknet.c:81-114), convolution term only */
+double network_conv_flops(network *net)
+{
+    double ops = 0;
+    int i;
+    for (i = 0; i < net->n; ++i) {
+        layer l = net->layers[i];
+        if (l.type == CONVOLUTIONAL)
+            ops += 2.0 * l.n * l.size * l.size * (l.c / l.groups) * l.out_h * l.out_w;
+    }
+    return ops;
+}

@@ -1,0 +1,122 @@
+/*
+ * weights_io.c - darknet `.weights` files for the layer types on the inference path.
+ *
+ * Format (src/parser.c:1007-1079 save_weights_upto, :1218-1306 load_weights_upto): three ints
+ * major, minor, revision; then `seen` as size_t when major*10+minor >= 2 (and both < 1000),
+ * else as int; then, per layer in order, for a convolutional layer: biases[n]; if
+ * batch_normalize (and not dontloadscales) scales[n], rolling_mean[n], rolling_variance[n];
+ * weights[nweights] (src/parser.c:958-977, :1164-1215).  Other layer types on this path carry
+ * no parameters.  A load ends in push_convolutional_layer, which also refreshes the packed copy
+ * the MFMA kernel reads.
+ */
+#include <stdio.h>
+#include <stdlib.h>
+#include <string.h>
+
+#include "host.h"
+
+static void file_error(const char *s)
+{
+    fprintf(stderr, "Couldn't open file: %s\n", s);
+    exit(0);
+}
+
+static void read_floats(float *dst, size_t n, FILE *fp, const char *what)
+{
+    if (fread(dst, sizeof(float), n, fp) != n) {
+        char buf[160];
+        snprintf(buf, sizeof buf, "weights file ends inside %s", what);
+        dn_fatal(buf);
+    }
+}
+
+/* In-place transpose of a rows x cols matrix (src/parser.c:1110-1122), used by `flipped`. */
+static void transpose_matrix(float *a, int rows, int cols)
+{
+    float *t = (float *)dn_calloc((size_t)rows * cols, sizeof(float));
+    int x, y;
+    for (x = 0; x < rows; ++x)
+        for (y = 0; y < cols; ++y) t[y * rows + x] = a[x * cols + y];
+    memcpy(a, t, sizeof(float) * (size_t)rows * cols);
+    free(t);
+}
+
+static void load_convolutional_weights(layer l, FILE *fp)
+{
+    int num;
+    if (l.numload) l.n = l.numload;
+    num = l.c / l.groups * l.n * l.size * l.size;
+    read_floats(l.biases, (size_t)l.n, fp, "convolutional biases");
+    if (l.batch_normalize && !l.dontloadscales) {
+        read_floats(l.scales, (size_t)l.n, fp, "convolutional scales");
+        read_floats(l.rolling_mean, (size_t)l.n, fp, "convolutional rolling_mean");
+        read_floats(l.rolling_variance, (size_t)l.n, fp, "convolutional rolling_variance");
+    }
+    read_floats(l.weights, (size_t)num, fp, "convolutional weights");
+    if (l.flipped) transpose_matrix(l.weights, l.c * l.size * l.size, l.n);
+    push_convolutional_layer(l);
+}
+
+void load_weights_upto(network *net, char *filename, int start, int cutoff)
+{
+    FILE *fp;
+    int major, minor, revision, i;
+    hip_set_device(net->gpu_index);
+    if (dn_verbose) fprintf(stderr, "Loading weights from %s...", filename);
+    fp = fopen(filename, "rb");
+    if (!fp) file_error(filename);
+    if (fread(&major, sizeof(int), 1, fp) != 1 || fread(&minor, sizeof(int), 1, fp) != 1 ||
+        fread(&revision, sizeof(int), 1, fp) != 1)
+        dn_fatal("weights file is shorter than its header");
+    if ((major * 10 + minor) >= 2 && major < 1000 && minor < 1000) {
+        if (fread(net->seen, sizeof(size_t), 1, fp) != 1) dn_fatal("weights file is shorter than its header");
+    } else {
+        int iseen = 0;
+        if (fread(&iseen, sizeof(int), 1, fp) != 1) dn_fatal("weights file is shorter than its header");
+        *net->seen = (size_t)iseen;
+    }
+    for (i = start; i < net->n && i < cutoff; ++i) {
+        layer l = net->layers[i];
+        if (l.dontload) continue;
+        if (l.type == CONVOLUTIONAL) load_convolutional_weights(l, fp);
+    }
+    if (dn_verbose) fprintf(stderr, "Done!\n");
+    fclose(fp);
+}
+
+void load_weights(network *net, char *filename)
+{
+    load_weights_upto(net, filename, 0, net->n);
+}
+
+void save_weights_upto(network *net, char *filename, int cutoff)
+{
+    FILE *fp;
+    int major = 0, minor = 2, revision = 0, i;
+    hip_set_device(net->gpu_index);
+    if (dn_verbose) fprintf(stderr, "Saving weights to %s\n", filename);
+    fp = fopen(filename, "wb");
+    if (!fp) file_error(filename);
+    fwrite(&major, sizeof(int), 1, fp);
+    fwrite(&minor, sizeof(int), 1, fp);
+    fwrite(&revision, sizeof(int), 1, fp);
+    fwrite(net->seen, sizeof(size_t), 1, fp);
+    for (i = 0; i < net->n && i < cutoff; ++i) {
+        layer l = net->layers[i];
+        if (l.type != CONVOLUTIONAL) continue;
+        pull_convolutional_layer(l);
+        fwrite(l.biases, sizeof(float), (size_t)l.n, fp);
+        if (l.batch_normalize) {
+            fwrite(l.scales, sizeof(float), (size_t)l.n, fp);
+            fwrite(l.rolling_mean, sizeof(float), (size_t)l.n, fp);
+            fwrite(l.rolling_variance, sizeof(float), (size_t)l.n, fp);
+        }
+        fwrite(l.weights, sizeof(float), (size_t)l.nweights, fp);
+    }
+    fclose(fp);
+}
+
+void save_weights(network *net, char *filename)
+{
+    save_weights_upto(net, filename, net->n);
+}

@@ -1,0 +1,109 @@
+"""ctypes loader of the native library (``libdarknet_hip.so``).
+
+The library is the product; there is no Python or CPU fallback.  ``load()`` raises if the
+shared object is missing, and every entry point declared in ``include/darknet_hip.h`` and
+``include/darknet_amd.h`` is bound here, so a missing symbol fails at load time, not mid-run.
+"""
+from __future__ import annotations
+
+import ctypes as C
+import os
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(HERE, "libdarknet_hip.so")
+
+F = C.POINTER(C.c_float)
+I = C.POINTER(C.c_int)
+U = C.POINTER(C.c_uint)
+V = C.c_void_p
+i, f, z = C.c_int, C.c_float, C.c_size_t
+
+# name -> (restype, argtypes); kept in the order of the two public headers
+SIGNATURES = {
+    # ---- darknet_hip.h: device shim
+    "hip_set_device": (None, [i]), "hip_get_device": (i, []), "hip_check_error": (None, [i]),
+    "hip_make_array": (V, [F, z]), "hip_make_int_array": (V, [I, z]), "hip_free": (None, [V]),
+    "hip_push_array": (None, [V, F, z]), "hip_pull_array": (None, [V, F, z]),
+    "hip_mag_array": (f, [V, z]), "hip_compare": (f, [V, F, z, C.c_char_p]),
+    "hip_pull_int_array": (None, [V, I, z]), "hip_synchronize": (None, []),
+    "hip_get_stream": (V, []), "hip_set_stream": (None, [V]), "hip_device_name": (C.c_char_p, []),
+    "cuda_set_device": (None, [i]), "cuda_get_device": (i, []), "cuda_make_array": (V, [F, z]),
+    "cuda_make_int_array": (V, [I, z]), "cuda_free": (None, [V]),
+    "cuda_push_array": (None, [V, F, z]), "cuda_pull_array": (None, [V, F, z]),
+    "cuda_mag_array": (f, [V, z]), "cuda_compare": (f, [V, F, z, C.c_char_p]),
+    "hip_event_create": (V, []), "hip_event_record": (None, [V]),
+    "hip_event_elapsed_ms": (f, [V, V]), "hip_event_destroy": (None, [V]),
+    # ---- darknet_hip.h: element-wise helpers
+    "fill_gpu": (None, [i, f, V, i]), "copy_gpu": (None, [i, V, i, V, i]),
+    "copy_gpu_offset": (None, [i, V, i, i, V, i, i]), "activate_array_gpu": (None, [V, i, i]),
+    "normalize_gpu": (None, [V, V, V, i, i, i]), "scale_bias_gpu": (None, [V, V, i, i, i]),
+    "add_bias_gpu": (None, [V, V, i, i, i]),
+    "shortcut_gpu": (None, [i, i, i, i, V, i, i, i, f, f, V]),
+    "upsample_gpu": (None, [V, i, i, i, i, i, i, f, V]),
+    "softmax_gpu": (None, [V, i, i, i, i, i, i, f, V]),
+    "im2col_gpu": (None, [V, i, i, i, i, i, i, V]),
+    "binarize_gpu": (None, [V, i, V]), "binarize_weights_gpu": (None, [V, i, i, V]),
+    # ---- darknet_hip.h: fused layer forwards
+    "forward_convolutional_gpu": (None, [V] * 8 + [i] * 11),
+    "conv_packed_floats": (z, [i, i, i, i]), "conv_pack_weights_gpu": (None, [V, V, i, i, i, i]),
+    "conv_set_algo": (None, [i]),
+    "xnor_weight_words": (z, [i, i, i]), "xnor_input_words": (z, [i, i, i, i]),
+    "xnor_pack_weights_gpu": (None, [V, V, V, i, i, i]),
+    "xnor_pack_input_gpu": (None, [V, V, i, i, i, i]),
+    "forward_convolutional_xnor_gpu": (None, [V] * 10 + [i] * 10),
+    "forward_maxpool_gpu": (None, [V, V, V] + [i] * 7),
+    "forward_route_gpu": (None, [C.POINTER(V), I, i, V, i]),
+    "forward_shortcut_gpu": (None, [V, V, V] + [i] * 7 + [f, f, i]),
+    "forward_yolo_gpu": (None, [V, V] + [i] * 5),
+    "forward_avgpool_gpu": (None, [V, V] + [i] * 4),
+    # ---- darknet_amd.h: layer / network API
+    "parse_network_cfg": (V, [C.c_char_p]), "load_network": (V, [C.c_char_p, C.c_char_p, i]),
+    "load_weights": (None, [V, C.c_char_p]), "load_weights_upto": (None, [V, C.c_char_p, i, i]),
+    "save_weights": (None, [V, C.c_char_p]), "save_weights_upto": (None, [V, C.c_char_p, i]),
+    "get_activation": (i, [C.c_char_p]), "get_activation_string": (C.c_char_p, [i]),
+    "get_layer_string": (C.c_char_p, [i]),
+    "make_network": (V, [i]), "free_network": (None, [V]), "forward_network": (None, [V]),
+    "forward_network_gpu": (None, [V]), "network_predict": (F, [V, F]),
+    "set_batch_network": (None, [V, i]), "network_output": (F, [V]),
+    "pull_network_output": (None, [V]), "network_width": (i, [V]), "network_height": (i, [V]),
+    "forward_network_device": (None, [V]), "layer_output_host": (F, [V, i]),
+    "layer_indexes_host": (I, [V, i]), "network_set_verbose": (None, [i]),
+    "network_set_conv": (None, [V, i, F, F, F, F, F]),
+    "network_layer_info": (None, [V, i, I, F]), "network_route_inputs": (i, [V, i, I, I, i]),
+    "network_num_layers": (i, [V]), "network_input_gpu": (V, [V]), "network_info": (None, [V, I]),
+    "network_conv_flops": (C.c_double, [V]),
+}
+
+# exported but taking structs by value (bound by reference C code, not through ctypes)
+STRUCT_BY_VALUE = [
+    "make_convolutional_layer", "make_maxpool_layer", "make_route_layer", "make_shortcut_layer",
+    "make_upsample_layer", "make_yolo_layer", "make_avgpool_layer", "make_softmax_layer", "free_layer",
+    "forward_convolutional_layer_gpu", "forward_maxpool_layer_gpu", "forward_route_layer_gpu",
+    "forward_shortcut_layer_gpu", "forward_upsample_layer_gpu", "forward_yolo_layer_gpu",
+    "forward_avgpool_layer_gpu", "forward_softmax_layer_gpu", "push_convolutional_layer",
+    "pull_convolutional_layer", "get_network_output_layer",
+]
+
+_lib = None
+
+
+def load() -> C.CDLL:
+    """Load the library and bind every exported entry point; raise if anything is missing."""
+    global _lib
+    if _lib is not None:
+        return _lib
+    if not os.path.exists(LIB_PATH):
+        raise RuntimeError(
+            f"{LIB_PATH} is missing: build it with `python -m darknet_amd.build` "
+            "(there is no fallback implementation)")
+    lib = C.CDLL(LIB_PATH, mode=C.RTLD_GLOBAL)
+    for name, (res, args) in SIGNATURES.items():
+        fn = getattr(lib, name)  # AttributeError if the symbol is not exported
+        fn.restype = res
+        fn.argtypes = args
+    for name in STRUCT_BY_VALUE:
+        getattr(lib, name)
+    C.c_int.in_dll(lib, "gpu_index")
+    lib.network_set_verbose(0)
+    _lib = lib
+    return lib

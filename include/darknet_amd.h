@@ -1,0 +1,230 @@
+/*
+ * darknet_amd.h - the layer / network API of the darknet forward path, on top of the device
+ * layer in darknet_hip.h.
+ *
+ * This header mirrors the part of the reference's public header that inference uses
+ * (include/darknet.h of pjreddie/darknet): the ACTIVATION and LAYER_TYPE enums in the same
+ * order, `layer` and `network` with the reference's field names, the constructors the cfg parser
+ * calls, and parse_network_cfg / network_predict / forward_network with their reference
+ * signatures.  Both structs are passed BY VALUE to every forward function, as in the
+ * reference (include/darknet.h:119-124).  Only the GPU dispatch exists: `forward` (the CPU
+ * pointer) is always NULL and forward_network() ends the process if gpu_index < 0 - this library
+ * has no CPU path to fall back to.
+ *
+ * Training-only members (delta, updates, x, x_norm, adam state, cost) are not allocated:
+ * inference never reads them and at batch 64 they would triple the footprint.
+ *
+ * Citations: reference file:line each declaration stands in for.
+ */
+#ifndef DARKNET_AMD_H
+#define DARKNET_AMD_H
+
+#include <stddef.h>
+#include <stdio.h>
+
+#include "darknet_hip.h"
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* include/darknet.h:48-50 */
+typedef enum {
+    LOGISTIC, RELU, RELIE, LINEAR, RAMP, TANH, PLSE, LEAKY, ELU, LOGGY, STAIR, HARDTAN, LHTAN, SELU
+} ACTIVATION;
+
+/* include/darknet.h:60-91 */
+typedef enum {
+    CONVOLUTIONAL, DECONVOLUTIONAL, CONNECTED, MAXPOOL, SOFTMAX, DETECTION, DROPOUT, CROP, ROUTE,
+    COST, NORMALIZATION, AVGPOOL, LOCAL, SHORTCUT, ACTIVE, RNN, GRU, LSTM, CRNN, BATCHNORM, NETWORK,
+    XNOR, REGION, YOLO, ISEG, REORG, UPSAMPLE, LOGXENT, L2NORM, BLANK
+} LAYER_TYPE;
+
+struct network;
+typedef struct network network;
+struct layer;
+typedef struct layer layer;
+
+/* include/darknet.h:115-422, inference subset */
+struct layer {
+    LAYER_TYPE type;
+    ACTIVATION activation;
+    void (*forward)(struct layer, struct network);     /* always NULL here */
+    void (*forward_gpu)(struct layer, struct network);
+    int batch_normalize;
+    int batch;
+    int flipped;
+    int inputs;
+    int outputs;
+    int nweights;
+    int nbiases;
+    int truths;
+    int h, w, c;
+    int out_h, out_w, out_c;
+    int n;
+    int max_boxes;
+    int groups;
+    int size;
+    int stride;
+    int reverse;
+    int pad;
+    int index;
+    int binary;
+    int xnor;
+    int truth;
+    int classes;
+    int total;
+    int noloss;
+    int dontload;
+    int dontloadscales;
+    int numload;
+    int onlyforward;
+    int *mask;
+    float alpha;
+    float beta;
+    float scale;
+    float temperature;
+    float jitter;
+    float ignore_thresh;
+    float truth_thresh;
+    int random;
+
+    int *input_layers;
+    int *input_sizes;
+
+    /* host copies: parameters always; output only where the host reads it (yolo heads and the
+     * last layer), see layer_output_host() for the rest */
+    float *biases;
+    float *scales;
+    float *weights;
+    float *rolling_mean;
+    float *rolling_variance;
+    float *output;
+    int *indexes;
+
+    size_t workspace_size;
+
+    /* device buffers (include/darknet.h:334-421) */
+    int *indexes_gpu;
+    float *weights_gpu;
+    float *biases_gpu;
+    float *scales_gpu;
+    float *rolling_mean_gpu;
+    float *rolling_variance_gpu;
+    float *output_gpu;
+    float *binary_weights_gpu;
+    float *binary_input_gpu;
+
+    /* additions of this library */
+    float *weights_packed_gpu; /* MFMA layout of weights_gpu; refreshed by push_convolutional_layer */
+    unsigned *xnor_wbits_gpu;  /* xnor layers: packed sign(w), packed sign(x), mean|w| per filter */
+    unsigned *xnor_xbits_gpu;
+    float *xnor_wmean_gpu;
+};
+
+/* include/darknet.h:430-496, inference subset */
+typedef struct network {
+    int n;
+    int batch;
+    size_t *seen;
+    int subdivisions;
+    layer *layers;
+    float *output;
+    int time_steps;
+    int inputs;
+    int outputs;
+    int truths;
+    int h, w, c;
+    int gpu_index;
+    float *input;
+    float *truth;
+    float *delta;
+    float *workspace;
+    int train;
+    int index;
+    float *input_gpu;
+    float *truth_gpu;
+    float *delta_gpu;
+    float *output_gpu;
+} network;
+
+/* ---- cfg parsing (src/parser.c:742-889; list/option helpers src/list.c, src/option_list.c) */
+network *parse_network_cfg(char *filename);
+network *load_network(char *cfg, char *weights, int clear);          /* src/network.c:53-63 */
+void load_weights(network *net, char *filename);                      /* src/parser.c:1308 */
+void load_weights_upto(network *net, char *filename, int start, int cutoff); /* src/parser.c:1218 */
+void save_weights(network *net, char *filename);                      /* src/parser.c:1081 */
+void save_weights_upto(network *net, char *filename, int cutoff);     /* src/parser.c:1007 */
+ACTIVATION get_activation(char *s);                                   /* src/activations.c:44 */
+char *get_activation_string(ACTIVATION a);                            /* src/activations.c:8 */
+char *get_layer_string(LAYER_TYPE a);                                 /* src/network.c:110 */
+
+/* ---- layer constructors, reference signatures -------------------------------------------- */
+layer make_convolutional_layer(int batch, int h, int w, int c, int n, int groups, int size,
+                               int stride, int padding, ACTIVATION activation,
+                               int batch_normalize, int binary, int xnor,
+                               int adam);                 /* src/convolutional_layer.c:176 */
+layer make_maxpool_layer(int batch, int h, int w, int c, int size, int stride,
+                         int padding);                    /* src/maxpool_layer.c:21 */
+layer make_route_layer(int batch, int n, int *input_layers, int *input_sizes); /* src/route_layer.c:7 */
+layer make_shortcut_layer(int batch, int index, int w, int h, int c, int w2, int h2,
+                          int c2);                        /* src/shortcut_layer.c:9 */
+layer make_upsample_layer(int batch, int w, int h, int c, int stride); /* src/upsample_layer.c:7 */
+layer make_yolo_layer(int batch, int w, int h, int n, int total, int *mask,
+                      int classes);                       /* src/yolo_layer.c:13 */
+layer make_avgpool_layer(int batch, int w, int h, int c); /* src/avgpool_layer.c:5 */
+layer make_softmax_layer(int batch, int inputs, int groups); /* src/softmax_layer.c:11 */
+void free_layer(layer l);                                 /* src/layer.c:6 */
+
+/* ---- per-layer GPU forwards, the function-pointer targets (include/darknet.h:122) -------- */
+void forward_convolutional_layer_gpu(layer l, network net); /* src/convolutional_kernels.cu:73 */
+void forward_maxpool_layer_gpu(layer l, network net);       /* src/maxpool_layer_kernels.cu:87 */
+void forward_route_layer_gpu(layer l, network net);         /* src/route_layer.c:105 */
+void forward_shortcut_layer_gpu(layer l, network net);      /* src/shortcut_layer.c:77 */
+void forward_upsample_layer_gpu(layer l, network net);      /* src/upsample_layer.c:91 */
+void forward_yolo_layer_gpu(layer l, network net);          /* src/yolo_layer.c:347 */
+void forward_avgpool_layer_gpu(layer l, network net);       /* src/avgpool_layer_kernels.cu:46 */
+void forward_softmax_layer_gpu(layer l, network net);       /* src/softmax_layer.c:82 */
+void push_convolutional_layer(layer l);                     /* src/convolutional_kernels.cu:286 */
+void pull_convolutional_layer(layer l);                     /* src/convolutional_kernels.cu:270 */
+
+/* ---- network runtime ---------------------------------------------------------------------- */
+network *make_network(int n);                               /* src/network.c:177 */
+void free_network(network *net);                            /* src/network.c:699 */
+void forward_network(network *net);                         /* src/network.c:188 */
+void forward_network_gpu(network *net);                     /* src/network.c:762 */
+float *network_predict(network *net, float *input);         /* src/network.c:497 */
+void set_batch_network(network *net, int b);                /* src/network.c:339 (shrink only) */
+layer get_network_output_layer(network *net);               /* src/network.c:689 */
+float *network_output(network *net);                        /* src/network.c:755 */
+void pull_network_output(network *net);                     /* src/network.c:1123 */
+int network_width(network *net);                            /* src/network.c:674 */
+int network_height(network *net);                           /* src/network.c:675 */
+
+/* ---- additions (no reference twin) --------------------------------------------------------
+ * forward_network_device: the layer loop alone, on whatever net->input_gpu holds; no host<->
+ * device copies, returns without synchronising.  This is what the benchmark times.
+ * layer_output_host: pulls layer i's output into a host buffer owned by the layer.
+ * network_set_verbose: 0 silences the per-layer table the constructors print to stderr. */
+void forward_network_device(network *net);
+float *layer_output_host(network *net, int i);
+int *layer_indexes_host(network *net, int i);
+void network_set_verbose(int on);
+void network_set_conv(network *net, int i, const float *weights, const float *biases,
+                      const float *scales, const float *rolling_mean,
+                      const float *rolling_variance);
+/* Flat read-out of a layer for FFI callers that do not mirror the struct: iv receives
+ * type, batch, h, w, c, out_h, out_w, out_c, n, size, stride, pad, groups, batch_normalize,
+ * activation, binary, xnor, index, inputs, outputs, nweights, classes, total, reverse,
+ * workspace_floats, nbiases, truths, max_boxes (28 ints); fv alpha, beta, scale, temperature. */
+void network_layer_info(network *net, int i, int *iv, float *fv);
+int network_route_inputs(network *net, int i, int *layers, int *sizes, int cap);
+int network_num_layers(network *net);
+float *network_input_gpu(network *net); /* device buffer forward_network_device reads */
+void network_info(network *net, int *iv); /* n, batch, h, w, c, inputs, outputs */
+double network_conv_flops(network *net);   /* per image, the reference's count (examples/darknet.c:88) */
+
+#ifdef __cplusplus
+}
+#endif
+#endif

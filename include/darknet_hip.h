@@ -1,0 +1,177 @@
+/*
+ * darknet_hip.h - device layer of the darknet forward path on AMD MI355X (gfx950).
+ *
+ * This is the C-ABI a darknet tree binds in place of src/cuda.c, the src/ *_kernels.cu files and cuBLAS:
+ * plain pointers and sizes only.  Every pointer named *_gpu (and every `float *` argument of a
+ * *_gpu function) is device memory obtained from hip_make_array / cuda_make_array.  All work is
+ * issued on one stream (hip_get_stream(), the null stream unless changed) and is asynchronous
+ * with respect to the host except the push/pull copies, as in the reference.
+ *
+ * Error convention is the reference's (src/cuda.c:27-49, src/utils.c:253-258): a failed HIP
+ * call or an argument the kernels cannot honour prints a message to stderr and ends the
+ * process with exit(-1).  There is no CPU fallback anywhere in this library.
+ *
+ * Citations name the reference interface each entry point replaces (paths relative to the
+ * pjreddie/darknet tree).
+ */
+#ifndef DARKNET_HIP_H
+#define DARKNET_HIP_H
+
+#include <stddef.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* ACTIVATION codes, same order as the reference enum (include/darknet.h:48-50). */
+enum {
+    DN_LOGISTIC = 0, DN_RELU, DN_RELIE, DN_LINEAR, DN_RAMP, DN_TANH, DN_PLSE, DN_LEAKY, DN_ELU,
+    DN_LOGGY, DN_STAIR, DN_HARDTAN, DN_LHTAN, DN_SELU
+};
+
+/* ------------------------------------------------------------------------------------------
+ * Device shim: replaces src/cuda.c / src/cuda.h (and include/darknet.h:632-637).
+ * The cuda_* spellings are exported as real symbols as well, so reference objects that call
+ * them link unchanged.
+ * ---------------------------------------------------------------------------------------- */
+extern int gpu_index;                                   /* src/cuda.c:1 */
+void   hip_set_device(int n);                           /* cuda_set_device      src/cuda.c:12  */
+int    hip_get_device(void);                            /* cuda_get_device      src/cuda.c:19  */
+void   hip_check_error(int status);                     /* check_error          src/cuda.c:27  */
+float *hip_make_array(float *x, size_t n);              /* cuda_make_array      src/cuda.c:90  */
+int   *hip_make_int_array(int *x, size_t n);            /* cuda_make_int_array  src/cuda.c:133 */
+void   hip_free(float *x_gpu);                          /* cuda_free            src/cuda.c:147 */
+void   hip_push_array(float *x_gpu, float *x, size_t n);/* cuda_push_array      src/cuda.c:153 */
+void   hip_pull_array(float *x_gpu, float *x, size_t n);/* cuda_pull_array      src/cuda.c:160 */
+float  hip_mag_array(float *x_gpu, size_t n);           /* cuda_mag_array       src/cuda.c:167 */
+float  hip_compare(float *x_gpu, float *x, size_t n, char *s); /* cuda_compare  src/cuda.c:120 */
+void   hip_pull_int_array(int *x_gpu, int *x, size_t n);/* (maxpool indexes; no reference twin) */
+void   hip_synchronize(void);                           /* hipStreamSynchronize on the stream  */
+void  *hip_get_stream(void);                            /* hipStream_t the library launches on */
+void   hip_set_stream(void *stream);                    /* 0 selects the null stream           */
+const char *hip_device_name(void);
+
+void   cuda_set_device(int n);
+int    cuda_get_device(void);
+float *cuda_make_array(float *x, size_t n);
+int   *cuda_make_int_array(int *x, size_t n);
+void   cuda_free(float *x_gpu);
+void   cuda_push_array(float *x_gpu, float *x, size_t n);
+void   cuda_pull_array(float *x_gpu, float *x, size_t n);
+float  cuda_mag_array(float *x_gpu, size_t n);
+float  cuda_compare(float *x_gpu, float *x, size_t n, char *s);
+
+/* Event timing on the library's stream (used by the benchmark; no reference twin). */
+void  *hip_event_create(void);
+void   hip_event_record(void *ev);
+float  hip_event_elapsed_ms(void *start, void *stop);   /* synchronises on `stop` */
+void   hip_event_destroy(void *ev);
+
+/* ------------------------------------------------------------------------------------------
+ * Element-wise helpers with the reference's own names and argument order
+ * (src/blas.h:51-102, src/activations.h:15, src/im2col.h:10; kernels in src/blas_kernels.cu,
+ * src/activation_kernels.cu, src/im2col_kernels.cu).  Arithmetic follows the CPU forms the
+ * parity contract names: normalize uses (x-mean)/(sqrt(var)+1e-6f) (src/blas.c:154), leaky and
+ * logistic are evaluated in double (src/activations.h:32,39).
+ * ---------------------------------------------------------------------------------------- */
+void fill_gpu(int N, float ALPHA, float *X, int INCX);                       /* blas.h:100 */
+void copy_gpu(int N, float *X, int INCX, float *Y, int INCY);                /* blas.h:53  */
+void copy_gpu_offset(int N, float *X, int OFFX, int INCX, float *Y, int OFFY, int INCY); /* :54 */
+void activate_array_gpu(float *x, int n, int activation);                    /* activations.h:15 */
+void normalize_gpu(float *x, float *mean, float *variance, int batch, int filters, int spatial); /* blas.h:65 */
+void scale_bias_gpu(float *output, float *scales, int batch, int n, int size);  /* blas.h:76 */
+void add_bias_gpu(float *output, float *biases, int batch, int n, int size);    /* blas.h:79 */
+void shortcut_gpu(int batch, int w1, int h1, int c1, float *add, int w2, int h2, int c2,
+                  float s1, float s2, float *out);                           /* blas.h:75  */
+void upsample_gpu(float *in, int w, int h, int c, int batch, int stride, int forward,
+                  float scale, float *out);                                  /* blas.h:102 */
+void softmax_gpu(float *input, int n, int batch, int batch_offset, int groups, int group_offset,
+                 int stride, float temp, float *output);                     /* blas.h:96  */
+void im2col_gpu(float *im, int channels, int height, int width, int ksize, int stride, int pad,
+                float *data_col);                                            /* im2col.h:10 */
+void binarize_gpu(float *x, int n, float *binary);            /* convolutional_kernels.cu:23; x>0 as on the CPU */
+void binarize_weights_gpu(float *weights, int n, int size, float *binary); /* convolutional_kernels.cu:67 */
+
+/* ------------------------------------------------------------------------------------------
+ * Fused layer forwards.  Each replaces the body of the reference's forward_*_layer_gpu for
+ * the inference case (net.train == 0); a darknet tree calls them from those functions with the
+ * fields of `layer` / `network` spelled out (INTEGRATION.md shows the adapters).
+ * ---------------------------------------------------------------------------------------- */
+
+/* Convolution + batch-norm/bias + activation in one pass.
+ * Replaces forward_convolutional_layer_gpu (src/convolutional_kernels.cu:73-135), i.e. the
+ * fill_gpu / im2col_gpu / gemm_gpu(cublasSgemm) loop over batch x groups plus the
+ * normalize/scale/add_bias/activate passes; CPU semantics of src/convolutional_layer.c:445-485.
+ *   input   [batch][c][h][w]                  weights [n][c/groups][size][size]
+ *   output  [batch][n][out_h][out_w],  out = (in + 2*pad - size)/stride + 1
+ *   batch_normalize != 0: scales, rolling_mean, rolling_variance (n each) are read;
+ *   otherwise they may be NULL.  biases (n) are always read.
+ *   packed: NULL, or the buffer written by conv_pack_weights_gpu for these weights (skips the
+ *   per-call repack; must be refreshed whenever the weights change).
+ * A 1x1 kernel must come with stride 1 and pad 0 (the reference feeds the image straight to
+ * the GEMM in that case, src/convolutional_layer.c:468-469; every cfg in the tree obeys it). */
+void forward_convolutional_gpu(const float *input, const float *weights, const float *packed,
+                               const float *biases, const float *scales,
+                               const float *rolling_mean, const float *rolling_variance,
+                               float *output, int batch, int c, int h, int w, int n,
+                               int groups, int size, int stride, int pad, int batch_normalize,
+                               int activation);
+
+/* Weight repack for the MFMA kernel (the natural hook is push_convolutional_layer,
+ * src/convolutional_kernels.cu:286-297).  conv_packed_floats() == 0 means the layer does not
+ * use a packed copy (grouped convolutions). */
+size_t conv_packed_floats(int n, int c, int groups, int size);
+void conv_pack_weights_gpu(const float *weights, float *packed, int n, int c, int groups, int size);
+
+/* Selects the convolution kernel: 0 = automatic (default), 1 = always the plain direct
+ * kernel.  The direct kernel is the in-library cross-check of the MFMA kernel. */
+void conv_set_algo(int algo);
+
+/* XNOR convolution (xnor=1 layers): sign(x>0) inputs, sign(w>0)*mean|w| weights, zero padding,
+ * computed as XOR + popcount on bit-packed operands, then the same batch-norm/bias/activation
+ * tail.  Replaces the xnor branch of forward_convolutional_layer_gpu
+ * (src/convolutional_kernels.cu:77-87) with the CPU semantics of
+ * src/convolutional_layer.c:28-49,451-456.
+ *   wbits  : scratch, xnor_weight_words(n,c,size) uint32;  wmean: scratch, n floats
+ *   xbits  : scratch, xnor_input_words(batch,c,h,w) uint32 */
+size_t xnor_weight_words(int n, int c, int size);
+size_t xnor_input_words(int batch, int c, int h, int w);
+void xnor_pack_weights_gpu(const float *weights, unsigned *wbits, float *wmean, int n, int c, int size);
+void xnor_pack_input_gpu(const float *input, unsigned *xbits, int batch, int c, int h, int w);
+void forward_convolutional_xnor_gpu(const float *input, const float *weights, unsigned *wbits,
+                                    float *wmean, unsigned *xbits, const float *biases,
+                                    const float *scales, const float *rolling_mean,
+                                    const float *rolling_variance, float *output, int batch,
+                                    int c, int h, int w, int n, int size, int stride, int pad,
+                                    int batch_normalize, int activation);
+
+/* forward_maxpool_layer_gpu (src/maxpool_layer_kernels.cu:87-99), CPU semantics of
+ * src/maxpool_layer.c:79-114: window origin (-pad)/2, outside = -FLT_MAX, first maximum wins.
+ * indexes may be NULL (inference never reads them). */
+void forward_maxpool_gpu(const float *input, float *output, int *indexes, int batch, int c,
+                         int h, int w, int size, int stride, int pad);
+
+/* forward_route_layer_gpu (src/route_layer.c:105-118): all sources concatenated per image in
+ * one launch.  srcs[i] holds batch x sizes[i] floats; output is batch x sum(sizes). */
+void forward_route_gpu(const float *const *srcs, const int *sizes, int nsrc, float *output,
+                       int batch);
+
+/* forward_shortcut_layer_gpu (src/shortcut_layer.c:77-82): out = act(s1*in + s2*add) over the
+ * overlapping region, act(in) elsewhere; one pass instead of copy + shortcut + activate.
+ * (w1,h1,c1) describe add, (w2,h2,c2) describe in/out, as in shortcut_cpu (src/blas.c:68). */
+void forward_shortcut_gpu(const float *in, const float *add, float *out, int batch, int w1,
+                          int h1, int c1, int w2, int h2, int c2, float s1, float s2,
+                          int activation);
+
+/* forward_yolo_layer_gpu, inference part (src/yolo_layer.c:347-361 on the GPU; the CPU form
+ * src/yolo_layer.c:132-148 defines the result): copy + logistic on x,y,objectness,classes. */
+void forward_yolo_gpu(const float *input, float *output, int batch, int w, int h, int n_anchors,
+                      int classes);
+
+/* forward_avgpool_layer_gpu (src/avgpool_layer_kernels.cu:46-54). */
+void forward_avgpool_gpu(const float *input, float *output, int batch, int c, int h, int w);
+
+#ifdef __cplusplus
+}
+#endif
+#endif
