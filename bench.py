@@ -1,0 +1,261 @@
+#!/usr/bin/env python3
+"""Benchmark of the darknet convolution forward path on one MI355X.
+
+A step is one forward pass of the whole network over one batch of synthetic input that is
+already resident in device memory (the layer loop the reference runs inside
+forward_network_gpu, src/network.c:773-785, without the host<->device copies around it).
+Default workload: yolov3 at 416x416, batch 64, fp32 - the configuration the headline metric is
+quoted on.  Prints ONE JSON line on stdout; progress goes to stderr.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload yolov3-416|yolov3-tiny-416|
+                    resnext50-224|yolov3-608] [--batch B] [--per-layer FILE] [--no-cpu]
+
+The line carries, besides the driver's fields:
+  roofline      the dominant kernel's algorithmic FLOP/s against the fp32 MFMA peak, from HIP
+                events recorded between layers during the timed steps
+  cpu_baseline  the reference CPU path (compiled reference when oracle/_ref is present, else
+                this repository's restatement, both -Ofast -fopenmp) timed on the host cores
+                on a bounded sample of the same network
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import tempfile
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+PEAK_FP32_MFMA_TFLOPS = 157.3
+PEAK_HBM_GBS = 8000.0
+
+WORKLOADS = {
+    "yolov3-416": ("yolov3", 416),
+    "yolov3-608": ("yolov3", 608),
+    "yolov3-tiny-416": ("yolov3_tiny", 416),
+    "resnext50-224": ("resnext50", 224),
+}
+
+
+def log(*a):
+    print(*a, file=sys.stderr, flush=True)
+
+
+def fill_params(setter, layers, seed=1000):
+    """uniform(-1,1)*sqrt(2/(k*k*c/groups)) weights, biases 0, BN mean 0 / variance 1 / scale 1."""
+    from darknet_amd import synth
+    for i, L in enumerate(layers):
+        if L["type"] != "convolutional":
+            continue
+        w = synth.conv_weights(seed + i, L["n"], L["c"] // L["groups"], L["size"])
+        b, s, m, v = synth.bn_identity(L["n"])
+        if L["batch_normalize"]:
+            setter(i, w, b, s, m, v)
+        else:
+            setter(i, w, b, None, None, None)
+
+
+def layer_bytes(L):
+    """Algorithmic HBM bytes of one layer for the whole batch (read operands once, write once)."""
+    b = L["batch"]
+    t = L["type"]
+    if t == "convolutional":
+        wbytes = 4 * L["nweights"] + (16 * L["n"] if L["batch_normalize"] else 4 * L["n"])
+        return 4 * b * (L["inputs"] + L["outputs"]) + wbytes
+    if t == "maxpool":
+        return 4 * b * (L["inputs"] + 2 * L["outputs"])  # output + indexes
+    if t == "shortcut":
+        add = min(L["c"], L["out_c"]) * min(L["h"], L["out_h"]) * min(L["w"], L["out_w"])
+        return 4 * b * (2 * L["outputs"] + add)
+    if t in ("route", "yolo", "softmax"):
+        return 8 * b * L["outputs"]
+    return 4 * b * (L["inputs"] + L["outputs"])
+
+
+def cpu_baseline(kind_pref, cfg_name, size, budget_s=20.0):
+    """Time the reference CPU path on a bounded sample: the same network at a small batch."""
+    from darknet_amd import cfgs, synth
+    from oracle import ref
+    threads = int(os.environ.get("OMP_NUM_THREADS", os.cpu_count() or 1))
+    gen = getattr(cfgs, cfg_name)
+    if kind_pref == "reference" and ref.available("fast"):
+        kind = "reference"
+
+        def make(batch):
+            text = gen(batch, size)
+            with tempfile.NamedTemporaryFile("w", suffix=".cfg", delete=False) as f:
+                f.write(text)
+            # the reference prints its layer table to stderr; keep the bench's stderr readable
+            devnull = os.open(os.devnull, os.O_WRONLY)
+            saved = os.dup(2)
+            os.dup2(devnull, 2)
+            try:
+                net = ref.RefNet(f.name, "fast")
+            finally:
+                os.dup2(saved, 2)
+                os.close(devnull)
+                os.close(saved)
+                os.unlink(f.name)
+            fill_params(net.set_conv, net.layers)
+            return net, (lambda x: net.predict(x)), net.inputs
+    else:
+        kind = "port"
+        from oracle.net import OracleNet
+
+        def make(batch):
+            net = OracleNet(gen(batch, size), fast=True)
+            fill_params(net.set_conv, net.layers)
+            return net, (lambda x: net.forward(x)), net.net["inputs"]
+
+    # one image first to size the sample
+    net, run, inputs = make(1)
+    x = synth.uniform01(7, inputs)
+    run(x)  # warm-up
+    t0 = time.perf_counter()
+    run(x)
+    t1 = time.perf_counter() - t0
+    batch = int(max(1, min(8, budget_s / 2 / max(t1, 1e-3))))
+    reps = 2
+    if batch > 1:
+        net, run, inputs = make(batch)
+        x = synth.uniform01(7, inputs * batch)
+        run(x)
+    t0 = time.perf_counter()
+    for _ in range(reps):
+        run(x)
+    dt = (time.perf_counter() - t0) / reps
+    return {"value": batch / dt, "unit": "images/s", "cores": threads, "kind": kind,
+            "sample": f"{cfg_name}-{size} forward at batch {batch}, 1 warm-up + {reps} timed passes, "
+                      f"-Ofast -fopenmp, OMP_NUM_THREADS={threads}, {dt:.3f} s/pass"}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=10)
+    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--workload", default="yolov3-416", choices=sorted(WORKLOADS))
+    ap.add_argument("--batch", type=int, default=64)
+    ap.add_argument("--per-layer", default="")
+    ap.add_argument("--no-cpu", action="store_true")
+    ap.add_argument("--cpu-kind", default="reference", choices=["reference", "port"])
+    args = ap.parse_args()
+    if args.gpus != 1:
+        log("bench.py: this build runs on one GPU only (the forward path has no exchange step; "
+            "see DESIGN.md for how it shards by batch). Use --gpus 1.")
+        sys.exit(2)
+
+    import numpy as np
+    from darknet_amd import api, cfgs, synth
+
+    cfg_name, size = WORKLOADS[args.workload]
+    text = getattr(cfgs, cfg_name)(args.batch, size)
+    api.set_gpu(0)
+    L = api._lib.load()
+    dev = L.hip_device_name().decode()
+    log("device:", dev)
+    net = api.Network(cfg_text=text)
+    fill_params(net.set_conv, net.layers)
+    x = synth.uniform01(7, net.inputs * net.batch)
+    net.push_input(x)
+    flops_img = net.conv_flops()
+
+    for _ in range(args.warmup):
+        net.forward_device()
+    net.synchronize()
+
+    # ---- timed region: K steps, input resident, per-layer HIP events recorded on the stream
+    layer_ms = np.zeros(net.n)
+    ev0, ev1 = L.hip_event_create(), L.hip_event_create()
+    net.synchronize()
+    t0 = time.perf_counter()
+    L.hip_event_record(ev0)
+    for _ in range(args.steps):
+        _, ms = net.forward_profiled()
+        layer_ms += np.asarray(ms)
+    L.hip_event_record(ev1)
+    total_ms = L.hip_event_elapsed_ms(ev0, ev1)
+    net.synchronize()
+    wall_ms = (time.perf_counter() - t0) * 1e3
+    layer_ms /= args.steps
+    ms_per_step = max(total_ms, 0.0) / args.steps
+    value = args.batch / (ms_per_step / 1e3)
+
+    # ---- PCIe-inclusive figure (network_predict: H2D input + D2H yolo/last outputs), untimed extra
+    t0 = time.perf_counter()
+    for _ in range(2):
+        net.predict(x)
+    pcie_ms = (time.perf_counter() - t0) * 1e3 / 2
+
+    # ---- per-layer accounting, grouped by kernel
+    kernels = {}
+    rows = []
+    for i, Ly in enumerate(net.layers):
+        ms = float(layer_ms[i])
+        row = {"layer": i, "type": Ly["type"], "ms": ms, "bytes": layer_bytes(Ly)}
+        if Ly["type"] == "convolutional":
+            fl = 2.0 * Ly["n"] * Ly["size"] ** 2 * (Ly["c"] // Ly["groups"]) * Ly["out_h"] * Ly["out_w"] * Ly["batch"]
+            name = ("xnor_conv_kernel" if Ly["xnor"] else
+                    L.conv_kernel_name(Ly["n"], Ly["c"], Ly["groups"], Ly["size"]).decode())
+            row.update(flops=fl, kernel=name, tflops=fl / ms / 1e9 if ms > 0 else 0.0,
+                       shape=f'{Ly["size"]}x{Ly["size"]}/{Ly["stride"]} {Ly["c"]}->{Ly["n"]} @{Ly["w"]}x{Ly["h"]}')
+            k = kernels.setdefault(name, {"ms": 0.0, "flops": 0.0, "launches": 0, "bytes": 0.0})
+            k["ms"] += ms
+            k["flops"] += fl
+            k["bytes"] += row["bytes"]
+            k["launches"] += 1
+        row["gbs"] = row["bytes"] / ms / 1e6 if ms > 0 else 0.0
+        rows.append(row)
+    dom_name, dom = max(kernels.items(), key=lambda kv: kv[1]["ms"])
+    achieved = dom["flops"] / dom["ms"] / 1e9  # TFLOP/s
+    conv_ms = sum(k["ms"] for k in kernels.values())
+    conv_tflops = sum(k["flops"] for k in kernels.values()) / conv_ms / 1e9
+    roofline = {"bound": "mfma", "achieved": round(achieved, 3), "peak": PEAK_FP32_MFMA_TFLOPS,
+                "unit": "TFLOP/s", "frac": round(achieved / PEAK_FP32_MFMA_TFLOPS, 4), "traffic": None,
+                "kernel": dom_name, "launches_per_step": dom["launches"],
+                "avg_launch_ms": round(dom["ms"] / dom["launches"], 4),
+                "flops_per_launch": dom["flops"] / dom["launches"],
+                "all_conv_tflops": round(conv_tflops, 3),
+                "all_conv_frac": round(conv_tflops / PEAK_FP32_MFMA_TFLOPS, 4)}
+
+    if args.per_layer:
+        with open(args.per_layer, "w") as f:
+            json.dump({"device": dev, "workload": args.workload, "batch": args.batch,
+                       "ms_per_step": ms_per_step, "layers": rows, "kernels": kernels}, f, indent=1)
+        log("per-layer table written to", args.per_layer)
+    memk = [r for r in rows if r["type"] != "convolutional"]
+    if memk:
+        mb = sum(r["bytes"] for r in memk)
+        mm = sum(r["ms"] for r in memk)
+        log(f"memory-bound layers: {mm:.3f} ms/step, {mb / mm / 1e6:.0f} GB/s "
+            f"({mb / mm / 1e6 / PEAK_HBM_GBS:.1%} of HBM peak); conv layers {conv_ms:.3f} ms/step, "
+            f"{conv_tflops:.1f} TFLOP/s")
+
+    out = {
+        "metric": "images/sec", "value": round(value, 2), "unit": "images/s", "n_gpus": 1,
+        "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(ms_per_step, 4),
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f32",
+        "data": "synthetic",
+        "config": {"workload": f"{args.workload} forward, batch {args.batch}, fp32, input uniform[0,1), "
+                               f"weights uniform(-1,1)*sqrt(2/(k*k*c)), BN mean 0 var 1 scale 1",
+                   "gflop_per_image": round(flops_img / 1e9, 3), "device": dev,
+                   "wall_ms_per_step": round(wall_ms / args.steps, 4),
+                   "pcie_inclusive_ms_per_step": round(pcie_ms, 3),
+                   "pcie_inclusive_images_per_s": round(args.batch / (pcie_ms / 1e3), 2)},
+        "roofline": roofline,
+    }
+    net.free()
+    if not args.no_cpu:
+        try:
+            out["cpu_baseline"] = cpu_baseline(args.cpu_kind, cfg_name, size)
+        except Exception as e:  # the CPU leg must not take the GPU result down with it
+            log("cpu_baseline failed:", repr(e))
+            out["cpu_baseline"] = None
+    print(json.dumps(out), flush=True)
+
+
+if __name__ == "__main__":
+    main()

@@ -160,6 +160,12 @@ class Network:
     def forward_device(self):
         self.L.forward_network_device(self.net)
 
+    def forward_profiled(self):
+        """One device-resident forward with per-layer HIP events -> (total_ms, [layer_ms])."""
+        buf = (C.c_float * self.n)()
+        total = self.L.forward_network_profiled(self.net, buf)
+        return float(total), [float(v) for v in buf]
+
     def synchronize(self):
         self.L.hip_synchronize()
 

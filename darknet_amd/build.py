@@ -55,7 +55,7 @@ def build(verbose: bool = False, jobs: int = 6) -> str:
         for out in ex.map(_run, steps):
             if verbose and out.strip():
                 print(out)
-    out = _run([hipcc, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", LIB] + objs +
+    out = _run([hipcc, "--offload-arch=gfx950", "-shared", "-fPIC", "-Wl,-Bsymbolic", "-o", LIB] + objs +
                ["-L" + os.path.join(ROCM, "lib"), "-lamdhip64", "-lm"])
     if verbose and out.strip():
         print(out)

@@ -20,6 +20,19 @@
  *   them (one barrier per chunk).
  * Weights are pre-packed to [K/16][Mpad][16] (zero padded, Mpad multiple of 128) so the A tile
  * is one contiguous, 16-byte aligned block for any BM.
+ *
+ * Order of K.  The sum over k does not care about the order as long as A and B agree, and the
+ * packing step can permute K for free, so two orders are used:
+ *   - "tap blocked" (1x1, and 3x3 with pad 1, when c % 16 == 0): k' = (cb*taps + tap)*16 + ci,
+ *     channel c = cb*16 + ci.  A 16-wide chunk is then 16 channels of ONE kernel tap: the whole
+ *     chunk shares one border test and one scalar base address (input + (cb*16*H*W + tap shift)),
+ *     each of a thread's loads adds a loop-invariant scalar i*H*W and the thread's fixed 32-bit
+ *     pixel offset, and the nine taps of a channel block follow each other so their input lines
+ *     are still in the L1/L2 when the next tap asks for them.  Lanes whose tap falls outside
+ *     the image read the centre pixel instead (always inside) and are zeroed when the chunk is
+ *     written to LDS.
+ *   - the reference's own (channel, ky, kx) order for everything else (first layer with 3
+ *     channels, 7x7 stems, odd channel counts), with a per-element index split.
  * Workgroup ids are remapped so that the tiles sharing a slice of the input run on the same
  * XCD (ids are dealt round-robin over the 8 XCDs, each with its own L2).
  */
@@ -78,12 +91,15 @@ __device__ __forceinline__ void split_k(int k, int size, int &ci, int &ky, int &
     }
 }
 
-template <int BM, int BN, int WM, int WN, int KS>
+template <int BM, int BN, int WM, int WN, int MODE>
 __global__ __launch_bounds__(DN_THREADS) void conv_mfma_kernel(mfma_args a)
 {
     constexpr int TM = WM / 32, TN = WN / 32;
     constexpr int WAVES_N = BN / WN;
     static_assert((BM / WM) * (BN / WN) == 4, "four waves per workgroup");
+    constexpr bool TAPB = MODE >= 10;             /* tap-blocked K order */
+    constexpr int KS = TAPB ? MODE - 10 : MODE;    /* kernel size known at compile time (0 = runtime) */
+    constexpr int TAPS = KS == 3 ? 9 : 1;
     constexpr int A_F4 = (BM * 4 + DN_THREADS - 1) / DN_THREADS; /* float4 loads of A per thread */
     constexpr int B_G = BN / 64;                                  /* 4-k groups of B per thread */
 
@@ -122,8 +138,10 @@ __global__ __launch_bounds__(DN_THREADS) void conv_mfma_kernel(mfma_args a)
     constexpr int KQ_STEP = DN_THREADS / BN;    /* distance between this thread's groups */
     const long ncol = n0 + bn_local;
     const bool col_ok = ncol < a.Ntotal;
-    int iy0 = 0, ix0 = 0;
-    long pix_base = 0;
+    int iy0 = 0, ix0 = 0, pix = 0;
+    const float *img = a.in;
+    unsigned voff_center = 0; /* tap-blocked: byte offset of (image b, channel 0, oy*stride, ox*stride) */
+    unsigned vmask = 0;       /* tap-blocked: bit ky*3+kx set when that tap lies inside the image */
     {
         const long nn = col_ok ? ncol : 0;
         const int b = (int)(nn / a.P);
@@ -132,11 +150,26 @@ __global__ __launch_bounds__(DN_THREADS) void conv_mfma_kernel(mfma_args a)
         const int ox = p - oy * a.OW;
         iy0 = oy * a.stride - a.pad;
         ix0 = ox * a.stride - a.pad;
-        pix_base = (long)b * a.C * a.H * a.W + (long)iy0 * a.W + ix0;
+        pix = iy0 * a.W + ix0;                       /* may be negative near the border */
+        img = a.in + (long)b * a.C * a.H * a.W;      /* this column's image */
+        if (TAPB) {
+            voff_center = (unsigned)(((long)b * a.C * a.H * a.W + (long)(oy * a.stride) * a.W + ox * a.stride) * 4);
+            if (col_ok) {
+#pragma unroll
+                for (int t = 0; t < TAPS; ++t) {
+                    const int ky = t / 3, kx = t % 3;
+                    if (KS == 1 || ((unsigned)(iy0 + ky) < (unsigned)a.H && (unsigned)(ix0 + kx) < (unsigned)a.W))
+                        vmask |= 1u << t;
+                }
+            }
+        }
     }
     const int HW = a.H * a.W;
+    /* tap-blocked loop state of the chunk being fetched (wave-uniform) */
+    int ld_tap = 0, ld_cb = 0;
+    bool ld_ok = false;      /* validity of the in-flight chunk for this lane */
 
-    float4 a_reg[A_F4];
+    float a_reg[A_F4][4]; /* scalars, not float4: keeps the staging registers out of memory */
     float b_reg[B_G][4];
 
     auto load_chunk = [&](int kc) {
@@ -145,9 +178,37 @@ __global__ __launch_bounds__(DN_THREADS) void conv_mfma_kernel(mfma_args a)
 #pragma unroll
         for (int i = 0; i < A_F4; ++i) {
             const int idx = tid + i * DN_THREADS;
-            if (BM * 4 >= DN_THREADS || idx < BM * 4) a_reg[i] = src[idx];
+            if (BM * 4 >= DN_THREADS || idx < BM * 4) {
+                const float4 t = src[idx];
+                a_reg[i][0] = t.x;
+                a_reg[i][1] = t.y;
+                a_reg[i][2] = t.z;
+                a_reg[i][3] = t.w;
+            }
         }
         /* B: gathered */
+        if (TAPB) {
+            const int ky = (ld_tap * 11) >> 5, kx = ld_tap - 3 * ((ld_tap * 11) >> 5); /* tap/3, tap%3 */
+            const int shift = KS == 1 ? 0 : (ky - 1) * a.W + (kx - 1);       /* pad == 1 for 3x3 */
+            const char *sbase = (const char *)a.in + ((long)ld_cb * 16 * HW + shift) * 4;
+            ld_ok = (vmask >> ld_tap) & 1u;
+            /* outside lanes cancel the tap shift and read the centre pixel; the cancellation is
+             * done in signed 64-bit so that pixel 0 with a positive shift cannot wrap */
+            const long voff = ld_ok ? (long)voff_center : (long)voff_center - (long)shift * 4;
+#pragma unroll
+            for (int g = 0; g < B_G; ++g) {
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                    const int i = (kq0 + g * KQ_STEP) * 4 + j; /* channel inside the block, uniform */
+                    b_reg[g][j] = *(const float *)(sbase + (long)i * HW * 4 + voff);
+                }
+            }
+            if (++ld_tap == TAPS) {
+                ld_tap = 0;
+                ++ld_cb;
+            }
+            return;
+        }
 #pragma unroll
         for (int g = 0; g < B_G; ++g) {
             const int kbase = kc * DN_BK + (kq0 + g * KQ_STEP) * 4;
@@ -156,15 +217,16 @@ __global__ __launch_bounds__(DN_THREADS) void conv_mfma_kernel(mfma_args a)
                 const int k = kbase + j;
                 int ci, ky, kx;
                 split_k<KS>(k, a.size, ci, ky, kx);
-                float v = 0.f;
-                if (KS == 1) {
-                    if (col_ok && k < a.K) v = a.in[pix_base + (long)ci * HW];
-                } else {
-                    const int iy = iy0 + ky, ix = ix0 + kx;
-                    const bool ok = col_ok && k < a.K && (unsigned)iy < (unsigned)a.H &&
-                                    (unsigned)ix < (unsigned)a.W;
-                    if (ok) v = a.in[pix_base + (long)ci * HW + ky * a.W + kx];
+                /* branch-free: an out-of-range tap reads element 0 of the image (always mapped)
+                 * and is replaced by zero afterwards, so a chunk's loads issue back to back */
+                bool ok = col_ok & (k < a.K);
+                int off = ci * HW;
+                if (KS != 1) {
+                    ok = ok & ((unsigned)(iy0 + ky) < (unsigned)a.H) & ((unsigned)(ix0 + kx) < (unsigned)a.W);
+                    off += ky * a.W + kx;
                 }
+                float v = img[ok ? pix + off : 0];
+                v = ok ? v : 0.f;
                 b_reg[g][j] = v;
             }
         }
@@ -176,14 +238,16 @@ __global__ __launch_bounds__(DN_THREADS) void conv_mfma_kernel(mfma_args a)
             const int idx = tid + i * DN_THREADS;
             if (BM * 4 >= DN_THREADS || idx < BM * 4) {
                 const int row = idx >> 2, kq = idx & 3;
-                *(float4 *)&As[buf][row * DN_LDK + kq * 4] = a_reg[i];
+                *(float4 *)&As[buf][row * DN_LDK + kq * 4] =
+                    make_float4(a_reg[i][0], a_reg[i][1], a_reg[i][2], a_reg[i][3]);
             }
         }
 #pragma unroll
         for (int g = 0; g < B_G; ++g) {
             const int kq = kq0 + g * KQ_STEP;
-            *(float4 *)&Bs[buf][bn_local * DN_LDK + kq * 4] =
-                make_float4(b_reg[g][0], b_reg[g][1], b_reg[g][2], b_reg[g][3]);
+            float4 t = make_float4(b_reg[g][0], b_reg[g][1], b_reg[g][2], b_reg[g][3]);
+            if (TAPB && !ld_ok) t = make_float4(0.f, 0.f, 0.f, 0.f);
+            *(float4 *)&Bs[buf][bn_local * DN_LDK + kq * 4] = t;
         }
     };
 
@@ -202,10 +266,7 @@ __global__ __launch_bounds__(DN_THREADS) void conv_mfma_kernel(mfma_args a)
     store_chunk(0);
     __syncthreads();
 
-    for (int kc = 0; kc < a.KCH; ++kc) {
-        const int buf = kc & 1;
-        const bool more = kc + 1 < a.KCH;
-        if (more) load_chunk(kc + 1);
+    auto compute_chunk = [&](int buf) {
 #pragma unroll
         for (int hb = 0; hb < 2; ++hb) {
             float4 av[TM], bv[TN];
@@ -228,9 +289,23 @@ __global__ __launch_bounds__(DN_THREADS) void conv_mfma_kernel(mfma_args a)
                 }
             }
         }
-        if (more) store_chunk(buf ^ 1);
+    };
+
+    /* Steady state: issue the global loads of chunk kc+1, run the MFMAs of chunk kc out of LDS,
+     * then park the prefetched chunk in the other LDS buffer.  The scheduling barriers keep the
+     * three phases in program order (without them the LDS stores are hoisted above the MFMAs
+     * and the wave waits on loads it has just issued).  The last chunk is peeled so that the
+     * loop body carries no condition for the compiler to merge the phases across. */
+    for (int kc = 0; kc + 1 < a.KCH; ++kc) {
+        const int buf = kc & 1;
+        load_chunk(kc + 1);
+        __builtin_amdgcn_sched_barrier(0);
+        compute_chunk(buf);
+        __builtin_amdgcn_sched_barrier(0);
+        store_chunk(buf ^ 1);
         __syncthreads();
     }
+    compute_chunk((a.KCH - 1) & 1);
 
     /* ---- epilogue: accumulator register r of lane l holds row 8*(r/4) + 4*(l/32) + r%4 and
      * column l%32 of its 32x32 block ---- */
@@ -260,16 +335,31 @@ __global__ __launch_bounds__(DN_THREADS) void conv_mfma_kernel(mfma_args a)
 }
 
 /* ---- weight packing ---------------------------------------------------------------------- */
-__global__ void pack_weights_kernel(const float *w, float *packed, int M, int K, int Mpad, long total)
+/* taps > 0 selects the tap-blocked order (taps = size*size, c % 16 == 0): packed row k' holds
+ * channel (k'/16/taps)*16 + k'%16 of tap (k'/16) % taps; taps == 0 keeps the reference order. */
+__global__ void pack_weights_kernel(const float *w, float *packed, int M, int K, int Mpad, long total, int taps)
 {
     for (long i = blockIdx.x * (long)blockDim.x + threadIdx.x; i < total; i += (long)gridDim.x * blockDim.x) {
         const int kk = (int)(i % DN_BK);
         long t = i / DN_BK;
         const int m = (int)(t % Mpad);
         const int kc = (int)(t / Mpad);
-        const int k = kc * DN_BK + kk;
+        int k = kc * DN_BK + kk;
+        if (taps > 0) {
+            const int cb = kc / taps, tap = kc - cb * taps;
+            k = (cb * DN_BK + kk) * taps + tap;
+        }
         packed[i] = (m < M && k < K) ? w[(long)m * K + k] : 0.f;
     }
+}
+
+/* K order of a layer, from the layer geometry alone so that packing and forward agree. */
+static inline int tap_blocked_taps(int c, int groups, int size)
+{
+    if (groups != 1 || (c % DN_BK) != 0) return 0;
+    if (size == 1) return 1;
+    if (size == 3) return 9;
+    return 0;
 }
 
 extern "C" size_t conv_packed_floats(int n, int c, int groups, int size)
@@ -290,7 +380,7 @@ extern "C" void conv_pack_weights_gpu(const float *weights, float *packed, int n
     long blocks = (long)((total + 255) / 256);
     if (blocks > 8192) blocks = 8192;
     hipLaunchKernelGGL(pack_weights_kernel, dim3((int)blocks), dim3(256), 0, dn_stream(), weights, packed, n,
-                       K, mpad, (long)total);
+                       K, mpad, (long)total, tap_blocked_taps(c, groups, size));
     dn_check_launch("conv_pack_weights_gpu");
 }
 
@@ -298,11 +388,27 @@ extern "C" void conv_pack_weights_gpu(const float *weights, float *packed, int n
 static int g_algo = 0;
 extern "C" void conv_set_algo(int algo) { g_algo = algo; }
 
+static int conv_mode(int c, int groups, int size, int stride, int pad, long in_bytes);
+
+extern "C" const char *conv_kernel_name(int n, int c, int groups, int size)
+{
+    static char name[96];
+    const int mode = conv_mode(c, groups, size, 1, size / 2, 0);
+    if (mode < 0) return "conv_direct_kernel";
+    if (n <= 32)
+        snprintf(name, sizeof name, "conv_mfma_kernel<32,256,32,64,%d>", mode);
+    else if (n <= 64)
+        snprintf(name, sizeof name, "conv_mfma_kernel<64,256,64,64,%d>", mode);
+    else
+        snprintf(name, sizeof name, "conv_mfma_kernel<128,128,64,64,%d>", mode);
+    return name;
+}
+
 static float *g_scratch = 0;       /* per-call repack buffer for callers without a packed copy */
 static size_t g_scratch_floats = 0;
 
 template <int BM, int BN, int WM, int WN>
-static void launch_tile(const mfma_args &a0, int ks)
+static void launch_tile(const mfma_args &a0, int mode)
 {
     mfma_args a = a0;
     a.tiles_m = (a.M + BM - 1) / BM;
@@ -310,12 +416,30 @@ static void launch_tile(const mfma_args &a0, int ks)
     const long total = (long)a.tiles_m * a.tiles_n;
     a.per_xcd = (int)((total + 7) / 8);
     const dim3 grid((unsigned)(a.per_xcd * 8));
-    if (ks == 1)
-        hipLaunchKernelGGL((conv_mfma_kernel<BM, BN, WM, WN, 1>), grid, dim3(DN_THREADS), 0, dn_stream(), a);
-    else if (ks == 3)
-        hipLaunchKernelGGL((conv_mfma_kernel<BM, BN, WM, WN, 3>), grid, dim3(DN_THREADS), 0, dn_stream(), a);
-    else
-        hipLaunchKernelGGL((conv_mfma_kernel<BM, BN, WM, WN, 0>), grid, dim3(DN_THREADS), 0, dn_stream(), a);
+    switch (mode) {
+    case 11: hipLaunchKernelGGL((conv_mfma_kernel<BM, BN, WM, WN, 11>), grid, dim3(DN_THREADS), 0, dn_stream(), a); break;
+    case 13: hipLaunchKernelGGL((conv_mfma_kernel<BM, BN, WM, WN, 13>), grid, dim3(DN_THREADS), 0, dn_stream(), a); break;
+    case 1: hipLaunchKernelGGL((conv_mfma_kernel<BM, BN, WM, WN, 1>), grid, dim3(DN_THREADS), 0, dn_stream(), a); break;
+    case 3: hipLaunchKernelGGL((conv_mfma_kernel<BM, BN, WM, WN, 3>), grid, dim3(DN_THREADS), 0, dn_stream(), a); break;
+    default: hipLaunchKernelGGL((conv_mfma_kernel<BM, BN, WM, WN, 0>), grid, dim3(DN_THREADS), 0, dn_stream(), a); break;
+    }
+}
+
+/* Which kernel variant serves a geometry: -1 = direct kernel, else the MODE template value. */
+static int conv_mode(int c, int groups, int size, int stride, int pad, long in_bytes)
+{
+    const long K = (long)(c / (groups > 0 ? groups : 1)) * size * size;
+    if (groups != 1 || g_algo == 1 || (size == 3 && K >= 32768)) return -1;
+    const int taps = tap_blocked_taps(c, groups, size);
+    if (taps) {
+        /* the tap-blocked kernel needs pad 1 for 3x3 and 32-bit byte offsets into the input;
+         * weights of such layers are packed tap-blocked, so the rare misfits go to the direct
+         * kernel rather than to the generic MFMA kernel, which expects the reference K order */
+        if (size == 3 && pad != 1) return -1;
+        if (in_bytes >= (1L << 32)) return -1;
+        return 10 + size;
+    }
+    return size == 1 ? 1 : size == 3 ? 3 : 0;
 }
 
 extern "C" void forward_convolutional_gpu(const float *input, const float *weights, const float *packed,
@@ -341,7 +465,8 @@ extern "C" void forward_convolutional_gpu(const float *input, const float *weigh
         dn_fatal("forward_convolutional_gpu: tensor too large");
 
     const long K = (long)(c / groups) * size * size;
-    if (groups != 1 || g_algo == 1 || (size == 3 && K >= 32768)) {
+    const int mode = conv_mode(c, groups, size, stride, pad, (long)batch * c * h * w * 4);
+    if (mode < 0) {
         conv_direct_forward(input, weights, biases, scales, rolling_mean, rolling_variance, output, batch, c,
                             h, w, n, groups, size, stride, pad, batch_normalize, activation);
         return;
@@ -382,12 +507,11 @@ extern "C" void forward_convolutional_gpu(const float *input, const float *weigh
     a.bn = batch_normalize ? 1 : 0;
     a.act = activation;
     a.tiles_m = a.tiles_n = a.per_xcd = 0;
-    const int ks = size == 1 ? 1 : size == 3 ? 3 : 0;
     if (n <= 32)
-        launch_tile<32, 256, 32, 64>(a, ks);
+        launch_tile<32, 256, 32, 64>(a, mode);
     else if (n <= 64)
-        launch_tile<64, 256, 64, 64>(a, ks);
+        launch_tile<64, 256, 64, 64>(a, mode);
     else
-        launch_tile<128, 128, 64, 64>(a, ks);
+        launch_tile<128, 128, 64, 64>(a, mode);
     dn_check_launch("forward_convolutional_gpu");
 }

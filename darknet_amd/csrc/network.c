@@ -72,6 +72,37 @@ void forward_network_device(network *netp)
     }
 }
 
+/* The same loop with a HIP event between consecutive layers; layer_ms[i] receives layer i's
+ * time on the device.  Returns the total (first event to last) in milliseconds.  Events are
+ * created once per network size and reused. */
+float forward_network_profiled(network *netp, float *layer_ms)
+{
+    static void **ev = 0;
+    static int nev = 0;
+    network net = *netp;
+    int i;
+    float total;
+    if (nev < net.n + 1) {
+        ev = (void **)realloc(ev, sizeof(void *) * (size_t)(net.n + 1));
+        if (!ev) dn_fatal("Malloc error");
+        for (i = nev; i < net.n + 1; ++i) ev[i] = hip_event_create();
+        nev = net.n + 1;
+    }
+    net.train = 0;
+    hip_event_record(ev[0]);
+    for (i = 0; i < net.n; ++i) {
+        layer l = net.layers[i];
+        net.index = i;
+        l.forward_gpu(l, net);
+        net.input_gpu = l.output_gpu;
+        hip_event_record(ev[i + 1]);
+    }
+    total = hip_event_elapsed_ms(ev[0], ev[net.n]);
+    if (layer_ms)
+        for (i = 0; i < net.n; ++i) layer_ms[i] = hip_event_elapsed_ms(ev[i], ev[i + 1]);
+    return total;
+}
+
 /* src/network.c:1123-1127 */
 void pull_network_output(network *net)
 {

@@ -66,7 +66,8 @@ SIGNATURES = {
     "forward_network_gpu": (None, [V]), "network_predict": (F, [V, F]),
     "set_batch_network": (None, [V, i]), "network_output": (F, [V]),
     "pull_network_output": (None, [V]), "network_width": (i, [V]), "network_height": (i, [V]),
-    "forward_network_device": (None, [V]), "layer_output_host": (F, [V, i]),
+    "forward_network_device": (None, [V]), "forward_network_profiled": (f, [V, F]),
+    "conv_kernel_name": (C.c_char_p, [i, i, i, i]), "layer_output_host": (F, [V, i]),
     "layer_indexes_host": (I, [V, i]), "network_set_verbose": (None, [i]),
     "network_set_conv": (None, [V, i, F, F, F, F, F]),
     "network_layer_info": (None, [V, i, I, F]), "network_route_inputs": (i, [V, i, I, I, i]),
@@ -96,7 +97,7 @@ def load() -> C.CDLL:
         raise RuntimeError(
             f"{LIB_PATH} is missing: build it with `python -m darknet_amd.build` "
             "(there is no fallback implementation)")
-    lib = C.CDLL(LIB_PATH, mode=C.RTLD_GLOBAL)
+    lib = C.CDLL(LIB_PATH)  # RTLD_LOCAL: the reference-compatible names stay private to this handle
     for name, (res, args) in SIGNATURES.items():
         fn = getattr(lib, name)  # AttributeError if the symbol is not exported
         fn.restype = res

@@ -207,6 +207,9 @@ int network_height(network *net);                           /* src/network.c:675
  * layer_output_host: pulls layer i's output into a host buffer owned by the layer.
  * network_set_verbose: 0 silences the per-layer table the constructors print to stderr. */
 void forward_network_device(network *net);
+/* forward_network_device with a HIP event after every layer: fills layer_ms[net->n] (may be
+ * NULL) and returns the whole pass in milliseconds; synchronises before returning. */
+float forward_network_profiled(network *net, float *layer_ms);
 float *layer_output_host(network *net, int i);
 int *layer_indexes_host(network *net, int i);
 void network_set_verbose(int on);

@@ -123,6 +123,10 @@ void forward_convolutional_gpu(const float *input, const float *weights, const f
 size_t conv_packed_floats(int n, int c, int groups, int size);
 void conv_pack_weights_gpu(const float *weights, float *packed, int n, int c, int groups, int size);
 
+/* Name of the kernel forward_convolutional_gpu launches for this geometry, as it appears in a
+ * profiler trace (e.g. "conv_mfma_kernel<128,128,64,64,3>"); for reports only. */
+const char *conv_kernel_name(int n, int c, int groups, int size);
+
 /* Selects the convolution kernel: 0 = automatic (default), 1 = always the plain direct
  * kernel.  The direct kernel is the in-library cross-check of the MFMA kernel. */
 void conv_set_algo(int algo);

@@ -40,7 +40,7 @@ def available(variant: str = "o2") -> bool:
 def raw(variant: str = "o2"):
     """The reference library itself (plain-pointer functions such as im2col_cpu, gemm)."""
     name = "libdarknet_ref.so" if variant == "fast" else "libdarknet_ref_o2.so"
-    return C.CDLL(os.path.join(_HERE, "_ref", name), mode=C.RTLD_GLOBAL)
+    return C.CDLL(os.path.join(_HERE, "_ref", name))
 
 
 class RefNet:
