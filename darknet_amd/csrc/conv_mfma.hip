@@ -11,8 +11,8 @@
  *
  * Tiling (64-wide wavefronts, 4 waves per workgroup):
  *   workgroup tile BM x BN x 16; wave tile WM x WN built from 32x32 accumulators of
- *   v_mfma_f32_32x32x2_f32 (TM x TN of them).  LDS holds A as [BM][16+4] and B as [BN][16+4]
- *   floats (k contiguous, 16-byte padded rows), double buffered; one ds_read_b128 per operand
+ *   v_mfma_f32_32x32x2_f32 (TM x TN of them).  LDS holds A as [BM][16] and B as [BN][16] floats
+ *   (k contiguous, 16-byte slots XOR-swizzled by row instead of padded), double buffered; one ds_read_b128 per operand
  *   row feeds four MFMA k-steps.  Within a 16-wide chunk the k index a lane uses at step s of
  *   half hb is hb*8 + (lane/32)*4 + s for A and B alike, a bijection of the chunk, so the
  *   result is the plain sum over k.
@@ -28,9 +28,9 @@
  *     chunk shares one border test and one scalar base address (input + (cb*16*H*W + tap shift)),
  *     each of a thread's loads adds a loop-invariant scalar i*H*W and the thread's fixed 32-bit
  *     pixel offset, and the nine taps of a channel block follow each other so their input lines
- *     are still in the L1/L2 when the next tap asks for them.  Lanes whose tap falls outside
- *     the image read the centre pixel instead (always inside) and are zeroed when the chunk is
- *     written to LDS.
+ *     are still in the L1/L2 when the next tap asks for them.  The loads are buffer loads:
+ *     lanes whose tap falls outside the image carry an out-of-range offset and get their zero
+ *     from the hardware range check, so the gather costs no vector ALU work at all.
  *   - the reference's own (channel, ky, kx) order for everything else (first layer with 3
  *     channels, 7x7 stems, odd channel counts), with a per-element index split.
  * Workgroup ids are remapped so that the tiles sharing a slice of the input run on the same
@@ -46,7 +46,14 @@
 typedef float f32x16 __attribute__((ext_vector_type(16)));
 
 #define DN_BK 16
-#define DN_LDK 20 /* padded LDS row, floats */
+#define DN_LDK 16 /* LDS row, floats: unpadded, the 16-byte slots of a row are XOR-swizzled */
+
+/* LDS address (in floats) of the 16-byte slot `kq` (0..3) of row `row`.  Rows are 64 bytes, so
+ * four rows span the 64 banks; XOR-ing the slot with bits 2..3 of the row spreads any 16
+ * consecutive rows read at the same slot over all 16 four-bank groups (conflict free for
+ * ds_read_b128 / ds_write_b128) without the padding that would cost a fourth resident
+ * workgroup per CU. */
+__device__ __forceinline__ int lds_slot(int row, int kq) { return row * DN_LDK + ((kq ^ (row >> 2)) & 3) * 4; }
 #define DN_MPAD 128
 #define DN_THREADS 256
 
@@ -67,6 +74,7 @@ struct mfma_args {
     int stride, pad, size;
     int bn, act;
     int tiles_m, tiles_n, per_xcd;
+    unsigned in_records; /* bytes the tap-blocked gather may address: input + bias row */
 };
 
 /* k -> (channel, ky, kx) for a size x size kernel in the reference's im2col row order. */
@@ -92,7 +100,7 @@ __device__ __forceinline__ void split_k(int k, int size, int &ci, int &ky, int &
 }
 
 template <int BM, int BN, int WM, int WN, int MODE>
-__global__ __launch_bounds__(DN_THREADS) void conv_mfma_kernel(mfma_args a)
+__global__ __launch_bounds__(DN_THREADS, 4) void conv_mfma_kernel(mfma_args a)
 {
     constexpr int TM = WM / 32, TN = WN / 32;
     constexpr int WAVES_N = BN / WN;
@@ -167,7 +175,15 @@ __global__ __launch_bounds__(DN_THREADS) void conv_mfma_kernel(mfma_args a)
     const int HW = a.H * a.W;
     /* tap-blocked loop state of the chunk being fetched (wave-uniform) */
     int ld_tap = 0, ld_cb = 0;
-    bool ld_ok = false;      /* validity of the in-flight chunk for this lane */
+    /* Buffer view of the input for the tap-blocked gather.  A buffer load adds a per-lane
+     * 32-bit offset and a scalar offset to the descriptor's base and returns 0, without touching
+     * memory, when the sum reaches num_records: lanes whose tap is outside the image get the
+     * offset 0xFFFFFFFC and read their zero for free.  The base sits (W+1) floats below the
+     * tensor so the scalar offset of the top-left tap of channel 0 is still non-negative; no
+     * lane ever resolves to an address below the tensor. */
+    const int bias = KS == 1 ? 0 : a.W + 1;
+    const __amdgpu_buffer_rsrc_t in_rsrc = __builtin_amdgcn_make_buffer_rsrc(
+        (void *)(a.in - bias), 0, (int)a.in_records, 0x00020000);
 
     float a_reg[A_F4][4]; /* scalars, not float4: keeps the staging registers out of memory */
     float b_reg[B_G][4];
@@ -190,17 +206,15 @@ __global__ __launch_bounds__(DN_THREADS) void conv_mfma_kernel(mfma_args a)
         if (TAPB) {
             const int ky = (ld_tap * 11) >> 5, kx = ld_tap - 3 * ((ld_tap * 11) >> 5); /* tap/3, tap%3 */
             const int shift = KS == 1 ? 0 : (ky - 1) * a.W + (kx - 1);       /* pad == 1 for 3x3 */
-            const char *sbase = (const char *)a.in + ((long)ld_cb * 16 * HW + shift) * 4;
-            ld_ok = (vmask >> ld_tap) & 1u;
-            /* outside lanes cancel the tap shift and read the centre pixel; the cancellation is
-             * done in signed 64-bit so that pixel 0 with a positive shift cannot wrap */
-            const long voff = ld_ok ? (long)voff_center : (long)voff_center - (long)shift * 4;
+            const unsigned soff0 = (unsigned)((ld_cb * 16 * HW + shift + bias) * 4); /* wave-uniform */
+            const unsigned voff = ((vmask >> ld_tap) & 1u) ? voff_center : 0xFFFFFFFCu;
 #pragma unroll
             for (int g = 0; g < B_G; ++g) {
 #pragma unroll
                 for (int j = 0; j < 4; ++j) {
                     const int i = (kq0 + g * KQ_STEP) * 4 + j; /* channel inside the block, uniform */
-                    b_reg[g][j] = *(const float *)(sbase + (long)i * HW * 4 + voff);
+                    b_reg[g][j] = __builtin_bit_cast(
+                        float, __builtin_amdgcn_raw_buffer_load_b32(in_rsrc, voff, soff0 + (unsigned)(i * HW * 4), 0));
                 }
             }
             if (++ld_tap == TAPS) {
@@ -238,16 +252,15 @@ __global__ __launch_bounds__(DN_THREADS) void conv_mfma_kernel(mfma_args a)
             const int idx = tid + i * DN_THREADS;
             if (BM * 4 >= DN_THREADS || idx < BM * 4) {
                 const int row = idx >> 2, kq = idx & 3;
-                *(float4 *)&As[buf][row * DN_LDK + kq * 4] =
+                *(float4 *)&As[buf][lds_slot(row, kq)] =
                     make_float4(a_reg[i][0], a_reg[i][1], a_reg[i][2], a_reg[i][3]);
             }
         }
 #pragma unroll
         for (int g = 0; g < B_G; ++g) {
             const int kq = kq0 + g * KQ_STEP;
-            float4 t = make_float4(b_reg[g][0], b_reg[g][1], b_reg[g][2], b_reg[g][3]);
-            if (TAPB && !ld_ok) t = make_float4(0.f, 0.f, 0.f, 0.f);
-            *(float4 *)&Bs[buf][bn_local * DN_LDK + kq * 4] = t;
+            *(float4 *)&Bs[buf][lds_slot(bn_local, kq)] =
+                make_float4(b_reg[g][0], b_reg[g][1], b_reg[g][2], b_reg[g][3]);
         }
     };
 
@@ -266,46 +279,74 @@ __global__ __launch_bounds__(DN_THREADS) void conv_mfma_kernel(mfma_args a)
     store_chunk(0);
     __syncthreads();
 
-    auto compute_chunk = [&](int buf) {
+    float4 av[2][TM], bv[2][TN]; /* MFMA operands of the current chunk: [k half][32-row block] */
+
+    auto read_operands = [&](int buf) {
 #pragma unroll
         for (int hb = 0; hb < 2; ++hb) {
-            float4 av[TM], bv[TN];
 #pragma unroll
             for (int i = 0; i < TM; ++i)
-                av[i] = *(const float4 *)&As[buf][(wm0 + i * 32 + li) * DN_LDK + hb * 8 + kh * 4];
+                av[hb][i] = *(const float4 *)&As[buf][lds_slot(wm0 + i * 32 + li, hb * 2 + kh)];
 #pragma unroll
             for (int j = 0; j < TN; ++j)
-                bv[j] = *(const float4 *)&Bs[buf][(wn0 + j * 32 + li) * DN_LDK + hb * 8 + kh * 4];
+                bv[hb][j] = *(const float4 *)&Bs[buf][lds_slot(wn0 + j * 32 + li, hb * 2 + kh)];
+        }
+    };
+
+    auto mfma_half = [&](int hb) {
 #pragma unroll
-            for (int s = 0; s < 4; ++s) {
+        for (int s = 0; s < 4; ++s) {
 #pragma unroll
-                for (int i = 0; i < TM; ++i) {
-                    const float ae = s == 0 ? av[i].x : s == 1 ? av[i].y : s == 2 ? av[i].z : av[i].w;
+            for (int i = 0; i < TM; ++i) {
+                const float ae = s == 0 ? av[hb][i].x : s == 1 ? av[hb][i].y : s == 2 ? av[hb][i].z : av[hb][i].w;
 #pragma unroll
-                    for (int j = 0; j < TN; ++j) {
-                        const float be = s == 0 ? bv[j].x : s == 1 ? bv[j].y : s == 2 ? bv[j].z : bv[j].w;
-                        acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(ae, be, acc[i][j], 0, 0, 0);
-                    }
+                for (int j = 0; j < TN; ++j) {
+                    const float be = s == 0 ? bv[hb][j].x : s == 1 ? bv[hb][j].y : s == 2 ? bv[hb][j].z : bv[hb][j].w;
+                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(ae, be, acc[i][j], 0, 0, 0);
                 }
             }
         }
     };
 
-    /* Steady state: issue the global loads of chunk kc+1, run the MFMAs of chunk kc out of LDS,
-     * then park the prefetched chunk in the other LDS buffer.  The scheduling barriers keep the
-     * three phases in program order (without them the LDS stores are hoisted above the MFMAs
-     * and the wave waits on loads it has just issued).  The last chunk is peeled so that the
-     * loop body carries no condition for the compiler to merge the phases across. */
-    for (int kc = 0; kc + 1 < a.KCH; ++kc) {
-        const int buf = kc & 1;
-        load_chunk(kc + 1);
+    /* One pipeline step.  Program order, pinned by scheduling barriers (left alone, the compiler
+     * hoists the LDS stores above the MFMAs and waits on loads it has just issued):
+     *   1. global/buffer loads of chunk kc+1 into registers
+     *   2. all LDS operand reads of chunk kc, then the first half of its MFMAs
+     *   3. the prefetched chunk goes to the other LDS buffer - in the middle of the MFMA phase,
+     *      so the store latency hides under the second half instead of sitting in front of
+     *      the barrier
+     *   4. second half of the MFMAs, barrier */
+    auto step = [&](int kc_next, int buf) {
+        load_chunk(kc_next);
         __builtin_amdgcn_sched_barrier(0);
-        compute_chunk(buf);
+        read_operands(buf);
+        __builtin_amdgcn_sched_barrier(0);
+        mfma_half(0);
         __builtin_amdgcn_sched_barrier(0);
         store_chunk(buf ^ 1);
+        __builtin_amdgcn_sched_barrier(0);
+        mfma_half(1);
+        __builtin_amdgcn_sched_barrier(0);
         __syncthreads();
+    };
+    auto last = [&](int buf) {
+        read_operands(buf);
+        mfma_half(0);
+        mfma_half(1);
+    };
+
+    int kc = 0;
+    /* two chunks per trip so the LDS buffer index is a compile-time constant in each half */
+    for (; kc + 2 < a.KCH; kc += 2) {
+        step(kc + 1, 0);
+        step(kc + 2, 1);
     }
-    compute_chunk((a.KCH - 1) & 1);
+    if (kc + 1 < a.KCH) { /* KCH even: one more full step, then the last chunk from buffer 1 */
+        step(kc + 1, 0);
+        last(1);
+    } else {
+        last(0);
+    }
 
     /* ---- epilogue: accumulator register r of lane l holds row 8*(r/4) + 4*(l/32) + r%4 and
      * column l%32 of its 32x32 block ---- */
@@ -416,12 +457,20 @@ static void launch_tile(const mfma_args &a0, int mode)
     const long total = (long)a.tiles_m * a.tiles_n;
     a.per_xcd = (int)((total + 7) / 8);
     const dim3 grid((unsigned)(a.per_xcd * 8));
+    if (BM > 128 && mode != 11 && mode != 13) dn_fatal("conv dispatch: the 256-row tile is only built for the tap-blocked modes");
     switch (mode) {
     case 11: hipLaunchKernelGGL((conv_mfma_kernel<BM, BN, WM, WN, 11>), grid, dim3(DN_THREADS), 0, dn_stream(), a); break;
     case 13: hipLaunchKernelGGL((conv_mfma_kernel<BM, BN, WM, WN, 13>), grid, dim3(DN_THREADS), 0, dn_stream(), a); break;
-    case 1: hipLaunchKernelGGL((conv_mfma_kernel<BM, BN, WM, WN, 1>), grid, dim3(DN_THREADS), 0, dn_stream(), a); break;
-    case 3: hipLaunchKernelGGL((conv_mfma_kernel<BM, BN, WM, WN, 3>), grid, dim3(DN_THREADS), 0, dn_stream(), a); break;
-    default: hipLaunchKernelGGL((conv_mfma_kernel<BM, BN, WM, WN, 0>), grid, dim3(DN_THREADS), 0, dn_stream(), a); break;
+    default:
+        if constexpr (BM <= 128) {
+            if (mode == 1)
+                hipLaunchKernelGGL((conv_mfma_kernel<BM, BN, WM, WN, 1>), grid, dim3(DN_THREADS), 0, dn_stream(), a);
+            else if (mode == 3)
+                hipLaunchKernelGGL((conv_mfma_kernel<BM, BN, WM, WN, 3>), grid, dim3(DN_THREADS), 0, dn_stream(), a);
+            else
+                hipLaunchKernelGGL((conv_mfma_kernel<BM, BN, WM, WN, 0>), grid, dim3(DN_THREADS), 0, dn_stream(), a);
+        }
+        break;
     }
 }
 
@@ -436,7 +485,7 @@ static int conv_mode(int c, int groups, int size, int stride, int pad, long in_b
          * weights of such layers are packed tap-blocked, so the rare misfits go to the direct
          * kernel rather than to the generic MFMA kernel, which expects the reference K order */
         if (size == 3 && pad != 1) return -1;
-        if (in_bytes >= (1L << 32)) return -1;
+        if (in_bytes + (1L << 20) >= (1L << 32)) return -1; /* 32-bit buffer offsets */
         return 10 + size;
     }
     return size == 1 ? 1 : size == 3 ? 3 : 0;
@@ -507,6 +556,7 @@ extern "C" void forward_convolutional_gpu(const float *input, const float *weigh
     a.bn = batch_normalize ? 1 : 0;
     a.act = activation;
     a.tiles_m = a.tiles_n = a.per_xcd = 0;
+    a.in_records = (unsigned)((long)batch * c * h * w * 4 + (long)(w + 1) * 4);
     if (n <= 32)
         launch_tile<32, 256, 32, 64>(a, mode);
     else if (n <= 64)

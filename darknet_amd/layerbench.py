@@ -66,8 +66,10 @@ def main():
     ap.add_argument("--groups", type=int, default=1)
     ap.add_argument("--iters", type=int, default=20)
     ap.add_argument("--sweep", action="store_true")
+    ap.add_argument("--algo", type=int, default=0)
     a = ap.parse_args()
     api.set_gpu(0)
+    _lib.load().conv_set_algo(a.algo)
     if a.sweep:
         for name, (c, h, w, n, size, stride) in cfgs.SWEEP.items():
             for batch in (1, 64):
