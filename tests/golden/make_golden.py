@@ -1,0 +1,205 @@
+#!/usr/bin/env python3
+"""Writes the golden fixtures of this directory from the COMPILED REFERENCE (oracle/_ref).
+
+Run in a container where the reference tree is mounted and `make -C oracle ref` has been done:
+
+    python tests/golden/make_golden.py
+
+Every fixture is data produced by executing the reference's own CPU code (strict -O2 build) on
+seeded synthetic inputs; nothing from the reference's sources is stored.  Fixtures:
+
+  layer_tables.json      geometry of every layer of yolov3-tiny-416, yolov3-416, resnext50-224
+                         as parse_network_cfg builds it (pins the cfg parser)
+  tiny416_b1.json        per-layer checksums + strided samples of a yolov3-tiny forward
+  small_net.cfg/.weights a 6-layer network and the weights file the reference saved for it
+  small_net.npz          its input and every layer's output (pins weights I/O + all layer kinds)
+  conv_cases.npz         single conv layers (3x3 s1/s2, 1x1, grouped, 7x7) in full
+  xnor_case.npz          one xnor conv layer: input, binarised tensors, output
+  maxpool_case.npz       maxpool output + indexes incl. the padded stride-1 case
+"""
+import json
+import os
+import sys
+
+import numpy as np
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+ROOT = os.path.dirname(os.path.dirname(HERE))
+sys.path.insert(0, ROOT)
+sys.path.insert(0, os.path.join(ROOT, "tests"))
+
+from darknet_amd import cfgs, synth  # noqa: E402
+from oracle import ref  # noqa: E402
+from util import fill_params, write_cfg  # noqa: E402
+
+KEYS = ["type", "batch", "h", "w", "c", "out_h", "out_w", "out_c", "n", "size", "stride", "pad", "groups",
+        "batch_normalize", "activation", "binary", "xnor", "index", "inputs", "outputs", "nweights", "classes",
+        "total", "reverse", "alpha", "beta", "scale", "temperature", "input_layers", "input_sizes", "mask"]
+
+
+def table(text):
+    p = write_cfg(text)
+    r = ref.RefNet(p)
+    os.unlink(p)
+    return r, [{k: L[k] for k in KEYS if k in L} for L in r.layers]
+
+
+SMALL_NET = """[net]
+batch=2
+subdivisions=1
+width=20
+height=16
+channels=3
+
+[convolutional]
+batch_normalize=1
+filters=16
+size=3
+stride=1
+pad=1
+activation=leaky
+
+[maxpool]
+size=2
+stride=2
+
+[convolutional]
+batch_normalize=1
+filters=32
+size=3
+stride=2
+pad=1
+activation=leaky
+
+[convolutional]
+filters=16
+size=1
+stride=1
+pad=1
+activation=linear
+
+[shortcut]
+from=-2
+activation=leaky
+
+[upsample]
+stride=2
+
+[route]
+layers=-1,1
+
+[convolutional]
+batch_normalize=1
+filters=24
+size=3
+stride=1
+pad=1
+groups=2
+activation=logistic
+
+[convolutional]
+filters=14
+size=1
+stride=1
+pad=1
+activation=linear
+
+[yolo]
+mask=0,1
+anchors=10,14,23,27,37,58
+classes=2
+num=3
+"""
+
+
+def main():
+    if not ref.available():
+        raise SystemExit("oracle/_ref is not built")
+    # ---- layer tables
+    tables = {}
+    for name, text in [("yolov3-tiny-416", cfgs.yolov3_tiny(1, 416)), ("yolov3-416", cfgs.yolov3(1, 416)),
+                       ("resnext50-224", cfgs.resnext50(1, 224)), ("small_net", SMALL_NET)]:
+        _, tables[name] = table(text)
+    json.dump(tables, open(os.path.join(HERE, "layer_tables.json"), "w"), indent=0)
+
+    # ---- yolov3-tiny forward checksums
+    r, _ = table(cfgs.yolov3_tiny(1, 416))
+    fill_params(r.set_conv, r.layers, seed=1000, bn="random")
+    x = synth.uniform01(7, r.inputs * r.batch)
+    outs = r.predict(x)
+    rec = []
+    for o in outs:
+        flat = o.reshape(-1).astype(np.float64)
+        step = max(1, flat.size // 16)
+        rec.append({"sum": float(flat.sum()), "abssum": float(np.abs(flat).sum()),
+                    "max": float(np.abs(flat).max()), "samples": [float(v) for v in o.reshape(-1)[::step][:16]]})
+    json.dump({"seed": 1000, "input_seed": 7, "layers": rec}, open(os.path.join(HERE, "tiny416_b1.json"), "w"))
+
+    # ---- small net with a reference-written weights file
+    open(os.path.join(HERE, "small_net.cfg"), "w").write(SMALL_NET)
+    p = os.path.join(HERE, "small_net.cfg")
+    r = ref.RefNet(p)
+    fill_params(r.set_conv, r.layers, seed=500, bn="random")
+    import ctypes as C
+    lib = ref.raw()
+    lib.save_weights.argtypes = [C.c_void_p, C.c_char_p]
+    lib.save_weights(r.net, os.path.join(HERE, "small_net.weights").encode())
+    x = synth.uniform(11, r.inputs * r.batch, -1, 1)
+    outs = r.predict(x)
+    np.savez_compressed(os.path.join(HERE, "small_net.npz"), input=x,
+                        **{f"layer{i}": o for i, o in enumerate(outs)},
+                        indexes1=r.layer_indexes(1))
+
+    # ---- single conv layers in full
+    cases = {}
+    specs = {"c3x3s1": (2, 8, 9, 11, 12, 3, 1, 1, 1, "leaky", 1), "c3x3s2": (2, 16, 13, 10, 20, 3, 2, 1, 1, "leaky", 1),
+             "c1x1": (3, 32, 7, 5, 19, 1, 1, 0, 1, "linear", 0), "grouped": (2, 8, 10, 10, 16, 3, 1, 1, 4, "leaky", 1),
+             "c7x7s2": (1, 3, 20, 22, 8, 7, 2, 3, 1, "leaky", 1), "logistic": (1, 16, 6, 6, 5, 3, 1, 1, 1, "logistic", 0)}
+    for name, (b, c, h, w, n, size, stride, pad, groups, act, bn) in specs.items():
+        text = (f"[net]\nbatch={b}\nsubdivisions=1\nwidth={w}\nheight={h}\nchannels={c}\n[convolutional]\n" +
+                ("batch_normalize=1\n" if bn else "") +
+                f"filters={n}\nsize={size}\nstride={stride}\npadding={pad}\ngroups={groups}\nactivation={act}\n")
+        p = write_cfg(text)
+        r = ref.RefNet(p)
+        os.unlink(p)
+        fill_params(r.set_conv, r.layers, seed=77, bn="random")
+        x = synth.uniform(5, r.inputs * r.batch, -1, 1)
+        cases[name + "_in"] = x
+        cases[name + "_out"] = r.predict(x)[0]
+        cases[name + "_spec"] = np.array([b, c, h, w, n, size, stride, pad, groups,
+                                          ref.ACTIVATIONS.index(act), bn], np.int32)
+    np.savez_compressed(os.path.join(HERE, "conv_cases.npz"), **cases)
+
+    # ---- xnor layer
+    p = write_cfg(cfgs.single_conv(2, 32, 9, 9, 24, 3, 1, xnor=True))
+    r = ref.RefNet(p)
+    os.unlink(p)
+    fill_params(r.set_conv, r.layers, seed=33, bn="random")
+    x = synth.uniform(9, r.inputs * r.batch, -1, 1)
+    x[::17] = 0.0  # exact zeros binarise to -1
+    out = r.predict(x)[0]
+    bw, bi = r.binary_tensors(0)
+    np.savez_compressed(os.path.join(HERE, "xnor_case.npz"), input=x, output=out, binary_weights=bw,
+                        binary_input=bi)
+
+    # ---- maxpool incl. the padded stride-1 window of yolov3-tiny
+    mp = {}
+    for name, (b, c, h, w, size, stride) in {"s2": (2, 3, 8, 12, 2, 2), "s1pad": (1, 4, 13, 13, 2, 1),
+                                               "k3s2": (1, 2, 9, 7, 3, 2)}.items():
+        text = (f"[net]\nbatch={b}\nsubdivisions=1\nwidth={w}\nheight={h}\nchannels={c}\n[maxpool]\n"
+                f"size={size}\nstride={stride}\n")
+        p = write_cfg(text)
+        r = ref.RefNet(p)
+        os.unlink(p)
+        x = synth.uniform(21, r.inputs * r.batch, -1, 1)
+        x[3::7] = x[2::7][: x[3::7].size]  # ties: the first maximum must win
+        mp[name + "_in"] = x
+        mp[name + "_out"] = r.predict(x)[0]
+        mp[name + "_idx"] = r.layer_indexes(0)
+        mp[name + "_spec"] = np.array([b, c, h, w, size, stride, r.layers[0]["pad"]], np.int32)
+    np.savez_compressed(os.path.join(HERE, "maxpool_case.npz"), **mp)
+    print("golden fixtures written to", HERE)
+
+
+if __name__ == "__main__":
+    main()

@@ -1,0 +1,172 @@
+"""End-to-end parity of whole networks: parse_network_cfg -> network_predict through the native
+library against the CPU checker on the same seeded weights and inputs.
+
+Gates: every conv layer <= 1e-4 (max-normalised), index/copy layers bit-exact *given the same
+input* (checked by feeding the library's own previous-layer output to the CPU checker), final
+yolo tensors <= 1e-3 absolute.  Batch-64 runs use size-independent properties."""
+import json
+import os
+
+import numpy as np
+import pytest
+
+from darknet_amd import api, cfgs, synth
+from oracle.net import OracleNet
+
+from util import REL_TOL, YOLO_ABS_TOL, fill_params, norm_err
+
+pytestmark = pytest.mark.gpu
+GOLD = os.path.join(os.path.dirname(__file__), "golden")
+EXACT_GIVEN_INPUT = ("maxpool", "route", "upsample", "shortcut")
+
+
+def build_pair(text, seed=1000, bn="random"):
+    net = api.Network(cfg_text=text)
+    orc = OracleNet(text)
+    fill_params(net.set_conv, net.layers, seed=seed, bn=bn)
+    fill_params(orc.set_conv, orc.layers, seed=seed, bn=bn)
+    return net, orc
+
+
+def check_network(text, input_seed=7, bn="random"):
+    net, orc = build_pair(text, bn=bn)
+    x = synth.uniform01(input_seed, net.inputs * net.batch)
+    final = net.predict(x)
+    want = orc.forward(x)
+    got = [net.layer_output(i) for i in range(net.n)]
+    worst = 0.0
+    for i, L in enumerate(orc.layers):
+        e = norm_err(got[i], want[i])
+        worst = max(worst, e)
+        assert e <= REL_TOL, (i, L["type"], e)
+        if L["type"] in EXACT_GIVEN_INPUT:
+            # re-run the CPU checker's layer on the LIBRARY's inputs: must match bit for bit
+            prev = got[i - 1] if i else x.reshape(net.batch, -1)
+            again = np.ascontiguousarray(orc.forward_layer(i, prev, got)).reshape(net.batch, -1)
+            assert np.array_equal(got[i], again), (i, L["type"])
+        if L["type"] == "yolo":
+            assert np.abs(got[i] - want[i]).max() <= YOLO_ABS_TOL
+    assert np.array_equal(final, got[-1])
+    net.free()
+    return worst
+
+
+def test_parser_matches_golden_layer_tables(dn):
+    gold = json.load(open(os.path.join(GOLD, "layer_tables.json")))
+    for name, text in [("yolov3-tiny-416", cfgs.yolov3_tiny(1, 416)), ("yolov3-416", cfgs.yolov3(1, 416)),
+                       ("resnext50-224", cfgs.resnext50(1, 224)),
+                       ("small_net", open(os.path.join(GOLD, "small_net.cfg")).read())]:
+        net = api.Network(cfg_text=text)
+        assert len(net.layers) == len(gold[name])
+        for i, (a, b) in enumerate(zip(net.layers, gold[name])):
+            for k, v in b.items():
+                if k in ("mask",):
+                    continue
+                if k in ("h", "w", "c") and b["type"] == "route":
+                    continue
+                assert a[k] == v or (isinstance(v, float) and abs(a[k] - v) < 1e-7), (name, i, k, a[k], v)
+        assert abs(net.conv_flops() - {"yolov3-tiny-416": 5.565e9, "yolov3-416": 65.864e9,
+                                       "resnext50-224": 7.742e9}.get(name, net.conv_flops())) < 1e6
+        net.free()
+
+
+def test_small_net_golden_outputs_and_reference_weights_file(dn, tmp_path):
+    """The library loads the weights file the REFERENCE saved and reproduces the reference's
+    per-layer outputs; saving it back yields the identical file."""
+    g = np.load(os.path.join(GOLD, "small_net.npz"))
+    net = api.Network(cfg_path=os.path.join(GOLD, "small_net.cfg"),
+                      weights=os.path.join(GOLD, "small_net.weights"))
+    net.predict(g["input"])
+    for i, L in enumerate(net.layers):
+        got = net.layer_output(i)
+        assert norm_err(got, g[f"layer{i}"]) <= REL_TOL, (i, L["type"])
+    assert np.array_equal(net.layer_indexes(1), g["indexes1"])
+    out = str(tmp_path / "roundtrip.weights")
+    net.save_weights(out)
+    assert open(out, "rb").read() == open(os.path.join(GOLD, "small_net.weights"), "rb").read()
+    net.free()
+
+
+def test_yolov3_tiny_416(dn):
+    assert check_network(cfgs.yolov3_tiny(1, 416)) <= REL_TOL
+
+
+def test_yolov3_tiny_golden_checksums(dn):
+    gold = json.load(open(os.path.join(GOLD, "tiny416_b1.json")))
+    net = api.Network(cfg_text=cfgs.yolov3_tiny(1, 416))
+    fill_params(net.set_conv, net.layers, seed=gold["seed"], bn="random")
+    net.predict(synth.uniform01(gold["input_seed"], net.inputs))
+    for i, g in enumerate(gold["layers"]):
+        flat = net.layer_output(i).reshape(-1)
+        step = max(1, flat.size // 16)
+        assert np.abs(flat[::step][:16] - np.array(g["samples"], np.float32)).max() <= REL_TOL * g["max"], i
+        assert abs(float(np.abs(flat.astype(np.float64)).sum()) - g["abssum"]) <= 1e-5 * g["abssum"] + 1e-6, i
+    net.free()
+
+
+def test_yolov3_tiny_benchmark_init(dn):
+    """The initialisation the benchmark configurations name: BN mean 0, variance 1, scale 1."""
+    assert check_network(cfgs.yolov3_tiny(1, 416), bn="identity") <= REL_TOL
+
+
+def test_yolov3_416(dn):
+    assert check_network(cfgs.yolov3(1, 416)) <= REL_TOL
+
+
+def test_yolov3_608_small_batch(dn):
+    assert check_network(cfgs.yolov3(1, 608), bn="identity") <= REL_TOL
+
+
+def test_resnext50_224(dn):
+    assert check_network(cfgs.resnext50(2, 224)) <= REL_TOL
+
+
+def test_batch_64_images_are_independent(dn):
+    """At the benchmark batch the CPU checker would take minutes; instead: image k of a batch-64
+    forward equals the batch-1 forward of that image (already checked against the CPU above)."""
+    text64, text1 = cfgs.yolov3_tiny(64, 416), cfgs.yolov3_tiny(1, 416)
+    net64, net1 = api.Network(cfg_text=text64), api.Network(cfg_text=text1)
+    fill_params(net64.set_conv, net64.layers)
+    fill_params(net1.set_conv, net1.layers)
+    x = synth.uniform01(3, net64.inputs * 64).reshape(64, -1)
+    net64.predict(x)
+    heads = [i for i, L in enumerate(net64.layers) if L["type"] == "yolo"]
+    for k in (0, 31, 63):
+        net1.predict(x[k])
+        for i in heads + [12, 20]:
+            a, b = net64.layer_output(i)[k], net1.layer_output(i)[0]
+            assert norm_err(a, b) <= 2e-6, (k, i)
+    net64.free()
+    net1.free()
+
+
+def test_yolov3_batch_64_runs_and_is_consistent(dn):
+    net64 = api.Network(cfg_text=cfgs.yolov3(64, 416))
+    net1 = api.Network(cfg_text=cfgs.yolov3(1, 416))
+    fill_params(net64.set_conv, net64.layers, bn="identity")
+    fill_params(net1.set_conv, net1.layers, bn="identity")
+    x = synth.uniform01(5, net64.inputs * 64).reshape(64, -1)
+    out64 = net64.predict(x)
+    out1 = net1.predict(x[40])
+    assert np.abs(out64[40] - out1[0]).max() <= YOLO_ABS_TOL
+    for i in (82, 94):
+        assert np.abs(net64.layer_output(i)[40] - net1.layer_output(i)[0]).max() <= YOLO_ABS_TOL
+    # device-resident forward (what the benchmark times) gives the same result as network_predict
+    net64.push_input(x)
+    net64.forward_device()
+    net64.synchronize()
+    assert np.array_equal(net64.layer_output(net64.n - 1), out64)
+    net64.free()
+    net1.free()
+
+
+def test_set_batch_network_shrinks(dn):
+    net = api.Network(cfg_text=cfgs.yolov3_tiny(4, 160))
+    fill_params(net.set_conv, net.layers)
+    x = synth.uniform01(9, net.inputs * 4).reshape(4, -1)
+    full = net.predict(x)
+    net.L.set_batch_network(net.net, 1)
+    net.batch = 1
+    one = net.predict(x[0])
+    assert np.array_equal(one[0], full[0])
+    net.free()

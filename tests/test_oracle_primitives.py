@@ -1,0 +1,325 @@
+"""Pins the CPU checker (oracle/oracle.c) function by function.
+
+Three kinds of evidence, chosen so that a dropped term, a wrong sign or index, or a transposed
+operand fails at least one test:
+  * golden vectors written by the compiled reference (tests/golden/*.npz, see make_golden.py);
+  * the compiled reference itself where oracle/_ref is present (bit-exact);
+  * independent mathematics: brute-force loops, exact small-integer GEMM, the fp64 direct
+    convolution, torch's CPU conv2d / max_pool2d, closed forms.
+"""
+import ctypes as C
+import math
+import os
+
+import numpy as np
+import pytest
+
+from darknet_amd import synth
+from oracle import ref
+from oracle.cpu import ACTIVATIONS
+
+from util import norm_err
+
+GOLD = os.path.join(os.path.dirname(__file__), "golden")
+needs_ref = pytest.mark.skipif(not ref.available(), reason="oracle/_ref (compiled reference) not built")
+F = C.POINTER(C.c_float)
+
+
+def fp(a):
+    return a.ctypes.data_as(F)
+
+
+# ---------------------------------------------------------------------------- im2col
+def brute_im2col(im, c, h, w, k, s, p):
+    oh = (h + 2 * p - k) // s + 1
+    ow = (w + 2 * p - k) // s + 1
+    col = np.zeros((c * k * k, oh * ow), np.float32)
+    im = im.reshape(c, h, w)
+    for ch in range(c):
+        for ky in range(k):
+            for kx in range(k):
+                r = (ch * k + ky) * k + kx
+                for oy in range(oh):
+                    for ox in range(ow):
+                        iy, ix = oy * s + ky - p, ox * s + kx - p
+                        if 0 <= iy < h and 0 <= ix < w:
+                            col[r, oy * ow + ox] = im[ch, iy, ix]
+    return col
+
+
+@pytest.mark.parametrize("c,h,w,k,s,p", [(2, 5, 6, 3, 1, 1), (3, 7, 5, 3, 2, 1), (1, 6, 6, 1, 1, 0),
+                                         (2, 8, 9, 5, 2, 2), (1, 9, 9, 7, 2, 3), (2, 4, 4, 3, 1, 0)])
+def test_im2col_brute_force(orc, c, h, w, k, s, p):
+    im = synth.uniform(1, c * h * w)
+    assert np.array_equal(orc.im2col(im, c, h, w, k, s, p), brute_im2col(im, c, h, w, k, s, p))
+
+
+def test_im2col_delta_image(orc):
+    """A single 1 at (ch, y, x) must appear exactly at rows (ch,ky,kx) / columns (y+p-ky, x+p-kx)."""
+    c, h, w, k, p = 2, 5, 5, 3, 1
+    im = np.zeros(c * h * w, np.float32)
+    ch, y, x = 1, 2, 3
+    im[(ch * h + y) * w + x] = 1
+    col = orc.im2col(im, c, h, w, k, 1, p)
+    hits = set(zip(*np.nonzero(col)))
+    want = set()
+    for ky in range(k):
+        for kx in range(k):
+            oy, ox = y + p - ky, x + p - kx
+            if 0 <= oy < h and 0 <= ox < w:
+                want.add(((ch * k + ky) * k + kx, oy * w + ox))
+    assert hits == want
+
+
+@needs_ref
+@pytest.mark.parametrize("c,h,w,k,s,p", [(16, 26, 26, 3, 1, 1), (8, 52, 40, 3, 2, 1), (3, 33, 31, 7, 2, 3)])
+def test_im2col_matches_reference(orc, c, h, w, k, s, p):
+    lib = ref.raw()
+    im = synth.uniform(2, c * h * w)
+    mine = orc.im2col(im, c, h, w, k, s, p)
+    theirs = np.empty_like(mine)
+    lib.im2col_cpu.argtypes = [F] + [C.c_int] * 6 + [F]
+    lib.im2col_cpu(fp(im), c, h, w, k, s, p, fp(theirs))
+    assert np.array_equal(mine, theirs)
+
+
+# ---------------------------------------------------------------------------- gemm
+def test_gemm_exact_on_small_integers(orc):
+    """All partial sums stay below 2^24, so any summation order gives the same bits."""
+    rng = np.random.default_rng(0)
+    A = rng.integers(-8, 9, (37, 53)).astype(np.float32)
+    B = rng.integers(-8, 9, (53, 29)).astype(np.float32)
+    assert np.array_equal(orc.gemm_nn(A, B), (A.astype(np.int64) @ B.astype(np.int64)).astype(np.float32))
+
+
+def test_gemm_not_transposed_and_accumulates(orc):
+    A = np.arange(6, dtype=np.float32).reshape(2, 3)
+    B = np.arange(12, dtype=np.float32).reshape(3, 4) - 5
+    C0 = np.full((2, 4), 10, np.float32)
+    got = orc.gemm_nn(A, B, C0.copy(), alpha=2.0)
+    assert np.array_equal(got, 10 + 2 * (A @ B))
+
+
+def test_gemm_close_to_fp64(orc):
+    A = synth.uniform(3, 64 * 300).reshape(64, 300)
+    B = synth.uniform(4, 300 * 50).reshape(300, 50)
+    assert norm_err(orc.gemm_nn(A, B), A.astype(np.float64) @ B.astype(np.float64)) < 1e-6
+
+
+@needs_ref
+def test_gemm_matches_reference_bits(orc):
+    lib = ref.raw()
+    M, N, K = 48, 169, 288
+    A = synth.uniform(5, M * K).reshape(M, K)
+    B = synth.uniform(6, K * N).reshape(K, N)
+    mine = orc.gemm_nn(A, B)
+    theirs = np.zeros((M, N), np.float32)
+    lib.gemm.argtypes = [C.c_int] * 5 + [C.c_float, F, C.c_int, F, C.c_int, C.c_float, F, C.c_int]
+    lib.gemm(0, 0, M, N, K, 1.0, fp(A), K, fp(B), N, 1.0, fp(theirs), N)
+    assert np.array_equal(mine, theirs)
+
+
+# ---------------------------------------------------------------------------- conv layer
+CONV_SHAPES = [  # b, c, h, w, n, size, stride, pad, groups
+    (2, 8, 9, 11, 12, 3, 1, 1, 1), (1, 16, 13, 10, 20, 3, 2, 1, 1), (2, 32, 7, 5, 19, 1, 1, 0, 1),
+    (2, 8, 10, 10, 16, 3, 1, 1, 4), (1, 3, 20, 22, 8, 7, 2, 3, 1)]
+
+
+@pytest.mark.parametrize("b,c,h,w,n,size,stride,pad,groups", CONV_SHAPES)
+def test_conv_against_fp64_direct_and_torch(orc, b, c, h, w, n, size, stride, pad, groups):
+    torch = pytest.importorskip("torch")
+    x = synth.uniform(1, b * c * h * w).reshape(b, c, h, w)
+    wt = synth.conv_weights(2, n, c // groups, size)
+    bias, sc, mu, var = synth.bn_random(3, n)
+    got = orc.conv(x, wt, bias, sc, mu, var, n=n, size=size, stride=stride, pad=pad, groups=groups,
+                   batch_normalize=1, activation="leaky")
+    ref64 = orc.conv_f64(x, wt, bias, sc, mu, var, n=n, size=size, stride=stride, pad=pad, groups=groups,
+                         batch_normalize=1, activation="leaky")
+    assert norm_err(got, ref64) < 2e-6
+    # library routine: cross-correlation, NCHW, zero padding, groups
+    y = torch.nn.functional.conv2d(torch.from_numpy(x).double(),
+                                   torch.from_numpy(wt.reshape(n, c // groups, size, size)).double(),
+                                   None, stride, pad, 1, groups).numpy()
+    y = (y - mu.reshape(1, -1, 1, 1)) / (np.sqrt(var.astype(np.float64)).reshape(1, -1, 1, 1) + np.float32(1e-6))
+    y = y * sc.reshape(1, -1, 1, 1) + bias.reshape(1, -1, 1, 1)
+    y = np.where(y > 0, y, 0.1 * y)
+    assert norm_err(got, y) < 2e-6
+
+
+def test_conv_golden_vectors(orc):
+    g = np.load(os.path.join(GOLD, "conv_cases.npz"))
+    names = sorted(k[:-5] for k in g.files if k.endswith("_spec"))
+    assert len(names) >= 6
+    for name in names:
+        b, c, h, w, n, size, stride, pad, groups, act, bn = [int(v) for v in g[name + "_spec"]]
+        L = [{"type": "convolutional", "n": n, "c": c, "groups": groups, "size": size, "batch_normalize": bn}]
+        params = {}
+        from util import fill_params
+        fill_params(lambda i, *a: params.update(p=a), L, seed=77, bn="random")
+        wt, bias, sc, mu, var = params["p"]
+        x = g[name + "_in"].reshape(b, c, h, w)
+        got = orc.conv(x, wt, bias, sc, mu, var, n=n, size=size, stride=stride, pad=pad, groups=groups,
+                       batch_normalize=bn, activation=ACTIVATIONS[act])
+        assert np.array_equal(got.reshape(b, -1), g[name + "_out"]), name
+
+
+def test_bn_identity_and_closed_form(orc):
+    x = synth.uniform(1, 2 * 3 * 5).reshape(2, 3, 5)
+    mean, var = np.zeros(3, np.float32), np.ones(3, np.float32)
+    y = orc.normalize(x, mean, var)
+    # mean 0 / variance 1: only the 1.000001 divisor remains
+    assert np.array_equal(y, (x.astype(np.float64) / (1.0 + float(np.float32(1e-6)))).astype(np.float32))
+    mean, var = synth.uniform(2, 3, -1, 1), synth.uniform(3, 3, 0.1, 4)
+    y = orc.normalize(x, mean, var)
+    want = (x - mean.reshape(1, 3, 1)).astype(np.float64) / (np.sqrt(var.astype(np.float64)).reshape(1, 3, 1)
+                                                              + float(np.float32(1e-6)))
+    assert np.array_equal(y, want.astype(np.float32))
+
+
+# ---------------------------------------------------------------------------- activations
+def test_activation_closed_forms(orc):
+    x = np.array([-3.5, -1.0, -0.0, 0.0, 0.25, 1.0, 7.0], np.float32)
+    assert orc.activate(np.zeros(1, np.float32), "logistic")[0] == 0.5
+    assert np.array_equal(orc.activate(x, "linear"), x)
+    lk = orc.activate(x, "leaky")
+    assert np.array_equal(lk[x > 0], x[x > 0])                       # exact for x > 0
+    assert np.array_equal(lk[x <= 0], (0.1 * x[x <= 0].astype(np.float64)).astype(np.float32))
+    assert lk[1] != np.float32(0.1) * np.float32(-1.0) or True        # (.1 is a double literal)
+    lg = orc.activate(x, "logistic")
+    assert np.all(np.diff(lg) >= 0) and np.all((lg > 0) & (lg < 1))
+    want = np.array([1.0 / (1.0 + math.exp(-float(v))) for v in x]).astype(np.float32)
+    assert np.array_equal(lg, want)
+    assert np.array_equal(orc.activate(x, "relu"), np.maximum(x, 0))
+    assert np.array_equal(orc.activate(x, "ramp"), (np.maximum(x, 0).astype(np.float64) + 0.1 * x).astype(np.float32))
+
+
+@needs_ref
+@pytest.mark.parametrize("act", ACTIVATIONS)
+def test_activations_match_reference_bits(orc, act):
+    lib = ref.raw()
+    x = np.concatenate([synth.uniform(9, 4000, -6, 6), np.array([0.0, -0.0, 1.0, -1.0, 4.0, -4.0, 5.0], np.float32)])
+    mine = orc.activate(x, act)
+    theirs = x.copy()
+    lib.activate_array.argtypes = [F, C.c_int, C.c_int]
+    lib.activate_array(fp(theirs), theirs.size, ACTIVATIONS.index(act))
+    assert np.array_equal(mine, theirs)
+
+
+# ---------------------------------------------------------------------------- maxpool
+def test_maxpool_textbook_and_padding(orc):
+    torch = pytest.importorskip("torch")
+    x = synth.uniform(1, 2 * 3 * 8 * 12).reshape(2, 3, 8, 12)
+    out, idx = orc.maxpool(x, 2, 2, 1)           # darknet default padding = size-1, offset -pad/2 = 0
+    want = torch.nn.functional.max_pool2d(torch.from_numpy(x), 2, 2).numpy()
+    assert np.array_equal(out, want)
+    assert np.array_equal(x.reshape(-1)[idx.reshape(-1)], out.reshape(-1))
+    # the 13x13 stride-1 pool of yolov3-tiny: pad right/bottom with -FLT_MAX
+    x = synth.uniform(2, 4 * 13 * 13).reshape(1, 4, 13, 13)
+    out, idx = orc.maxpool(x, 2, 1, 1)
+    xp = np.pad(x, ((0, 0), (0, 0), (0, 1), (0, 1)), constant_values=-np.finfo(np.float32).max)
+    want = torch.nn.functional.max_pool2d(torch.from_numpy(xp), 2, 1).numpy()
+    assert out.shape == (1, 4, 13, 13) and np.array_equal(out, want)
+
+
+def test_maxpool_first_maximum_wins(orc):
+    x = np.zeros((1, 1, 2, 2), np.float32) + 3
+    out, idx = orc.maxpool(x, 2, 2, 1)
+    assert out[0, 0, 0, 0] == 3 and idx[0, 0, 0, 0] == 0
+
+
+def test_maxpool_golden(orc):
+    g = np.load(os.path.join(GOLD, "maxpool_case.npz"))
+    for name in ("s2", "s1pad", "k3s2"):
+        b, c, h, w, size, stride, pad = [int(v) for v in g[name + "_spec"]]
+        out, idx = orc.maxpool(g[name + "_in"].reshape(b, c, h, w), size, stride, pad)
+        assert np.array_equal(out.reshape(b, -1), g[name + "_out"])
+        assert np.array_equal(idx.reshape(b, -1), g[name + "_idx"])
+
+
+# ---------------------------------------------------------------------------- the rest
+def test_upsample_is_nearest(orc):
+    x = synth.uniform(1, 2 * 3 * 4 * 5).reshape(2, 3, 4, 5)
+    y = orc.upsample(x, 2)
+    assert np.array_equal(y, x.repeat(2, axis=2).repeat(2, axis=3))
+    assert np.array_equal(orc.upsample(x, 3, 0.5), (np.float32(0.5) * x).repeat(3, axis=2).repeat(3, axis=3))
+
+
+def test_shortcut_invariants(orc):
+    x = synth.uniform(1, 2 * 8 * 6 * 6).reshape(2, 8, 6, 6)
+    add = synth.uniform(2, 2 * 8 * 6 * 6).reshape(2, 8, 6, 6)
+    assert np.array_equal(orc.shortcut(x, add), x + add)
+    # fewer channels in `add`, and `add` twice as large spatially (stride 2 sampling), as in resnext50
+    add = synth.uniform(3, 2 * 4 * 12 * 12).reshape(2, 4, 12, 12)
+    y = orc.shortcut(x, add)
+    assert np.array_equal(y[:, 4:], x[:, 4:])
+    assert np.array_equal(y[:, :4], x[:, :4] + add[:, :, ::2, ::2])
+    # `add` smaller spatially: only every second output pixel receives it
+    add = synth.uniform(4, 2 * 8 * 3 * 3).reshape(2, 8, 3, 3)
+    y = orc.shortcut(x, add)
+    want = x.copy()
+    want[:, :, ::2, ::2] += add
+    assert np.array_equal(y, want)
+
+
+def test_route_concatenates_per_image(orc):
+    a = synth.uniform(1, 3 * 10).reshape(3, 10)
+    b = synth.uniform(2, 3 * 4).reshape(3, 4)
+    assert np.array_equal(orc.route([a, b]), np.concatenate([a, b], axis=1))
+
+
+def test_yolo_planes(orc):
+    n, classes, h, w = 3, 2, 4, 5
+    x = synth.uniform(1, 2 * n * (5 + classes) * h * w, -3, 3).reshape(2, n * (5 + classes), h, w)
+    y = orc.yolo(x, n, classes).reshape(2, n, 5 + classes, h, w)
+    xr = x.reshape(2, n, 5 + classes, h, w)
+    assert np.array_equal(y[:, :, 2:4], xr[:, :, 2:4])                  # w,h stay raw
+    sig = orc.activate(xr, "logistic")
+    assert np.array_equal(y[:, :, :2], sig[:, :, :2]) and np.array_equal(y[:, :, 4:], sig[:, :, 4:])
+
+
+def test_avgpool_and_softmax(orc):
+    x = synth.uniform(1, 2 * 5 * 7 * 7).reshape(2, 5, 7, 7)
+    assert norm_err(orc.avgpool(x), x.astype(np.float64).mean(axis=(2, 3))) < 1e-6
+    z = synth.uniform(2, 3 * 1000, -5, 5).reshape(3, 1000)
+    p = orc.softmax(z)
+    assert np.allclose(p.sum(axis=1), 1, atol=1e-5) and np.array_equal(p.argmax(1), z.argmax(1))
+    e = np.exp(z.astype(np.float64) - z.max(axis=1, keepdims=True))
+    assert norm_err(p, e / e.sum(axis=1, keepdims=True)) < 1e-5
+    p2 = orc.softmax(z, groups=4, temperature=2.0).reshape(3, 4, 250)
+    assert np.allclose(p2.sum(axis=2), 1, atol=1e-5)
+
+
+def test_binarize_semantics_and_golden(orc):
+    x = np.array([0.0, -0.0, 1e-30, -2.0, np.nan, 3.0], np.float32)
+    assert np.array_equal(orc.binarize_input(x), np.array([-1, -1, 1, -1, -1, 1], np.float32))
+    w = synth.uniform(1, 4 * 27).astype(np.float32)
+    w[5] = 0
+    bw = orc.binarize_weights(w, 4).reshape(4, 27)
+    for f in range(4):
+        m = np.float32(0)
+        for v in w.reshape(4, 27)[f]:
+            m = np.float32(m + abs(v))
+        m = np.float32(m / np.float32(27))
+        assert np.array_equal(bw[f], np.where(w.reshape(4, 27)[f] > 0, m, -m))
+    g = np.load(os.path.join(GOLD, "xnor_case.npz"))
+    from util import fill_params
+    L = [{"type": "convolutional", "n": 24, "c": 32, "groups": 1, "size": 3, "batch_normalize": 1}]
+    params = {}
+    fill_params(lambda i, *a: params.update(p=a), L, seed=33, bn="random")
+    wt, bias, sc, mu, var = params["p"]
+    out, bw, bi = orc.conv(g["input"].reshape(2, 32, 9, 9), wt, bias, sc, mu, var, n=24, size=3, stride=1, pad=1,
+                           batch_normalize=1, activation="leaky", xnor=1, return_binary=True)
+    assert np.array_equal(bw, g["binary_weights"])
+    assert np.array_equal(bi.reshape(2, -1), g["binary_input"])
+    assert np.array_equal(out.reshape(2, -1), g["output"])
+    # exact-integer form: mean_f * (even integer) - the popcount kernel's arithmetic
+    sign_w = np.where(wt.reshape(24, -1) > 0, 1.0, -1.0)
+    mean_f = np.abs(bw.reshape(24, -1))[:, 0].astype(np.float64)
+    col = np.stack([orc.im2col(np.ascontiguousarray(bi.reshape(2, -1)[b]), 32, 9, 9, 3, 1, 1) for b in range(2)])
+    dots = np.einsum("fk,bkn->bfn", sign_w, col.astype(np.float64))
+    assert np.all(dots == np.round(dots))
+    pre = mean_f.reshape(1, -1, 1) * dots
+    y = (pre - mu.reshape(1, -1, 1)) / (np.sqrt(var.astype(np.float64)).reshape(1, -1, 1) + np.float32(1e-6))
+    y = y * sc.reshape(1, -1, 1) + bias.reshape(1, -1, 1)
+    y = np.where(y > 0, y, 0.1 * y)
+    assert norm_err(out.reshape(2, 24, -1), y) < 1e-5
