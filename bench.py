@@ -75,6 +75,20 @@ def layer_bytes(L):
     return 4 * b * (L["inputs"] + L["outputs"])
 
 
+def profiled_traffic(workload, batch, kernel):
+    """HBM bytes per launch of `kernel`, as measured by the committed rocprofv3 --pmc runs of this
+    very command (profiles/bench_<workload>_b<batch>.md carries the figure and how it was scaled).
+    Counters cannot be read from inside the process, so this is None when no such profile exists."""
+    import re
+    path = os.path.join(ROOT, "profiles", f"bench_{workload.replace('-', '_')}_b{batch}.md")
+    try:
+        text = open(path).read()
+    except OSError:
+        return None
+    m = re.search(r"traffic_bytes_per_launch\(" + re.escape(kernel) + r"\):\s*([0-9.]+)", text)
+    return float(m.group(1)) if m else None
+
+
 def cpu_baseline(kind_pref, cfg_name, size, budget_s=20.0):
     """Time the reference CPU path on a bounded sample: the same network at a small batch."""
     from darknet_amd import cfgs, synth
@@ -163,6 +177,13 @@ def main():
     net.push_input(x)
     flops_img = net.conv_flops()
 
+    # One plain copy of known size (256 MiB read + 256 MiB written): the yardstick that turns a
+    # profiler's FETCH_SIZE / WRITE_SIZE readings for the conv kernel into bytes.
+    cal = api.DeviceArray(n=64 << 20), api.DeviceArray(n=64 << 20)
+    L.copy_gpu(64 << 20, cal[0].ptr, 1, cal[1].ptr, 1)
+    net.synchronize()
+    del cal
+
     for _ in range(args.warmup):
         net.forward_device()
     net.synchronize()
@@ -214,7 +235,8 @@ def main():
     conv_ms = sum(k["ms"] for k in kernels.values())
     conv_tflops = sum(k["flops"] for k in kernels.values()) / conv_ms / 1e9
     roofline = {"bound": "mfma", "achieved": round(achieved, 3), "peak": PEAK_FP32_MFMA_TFLOPS,
-                "unit": "TFLOP/s", "frac": round(achieved / PEAK_FP32_MFMA_TFLOPS, 4), "traffic": None,
+                "unit": "TFLOP/s", "frac": round(achieved / PEAK_FP32_MFMA_TFLOPS, 4),
+                "traffic": profiled_traffic(args.workload, args.batch, dom_name),
                 "kernel": dom_name, "launches_per_step": dom["launches"],
                 "avg_launch_ms": round(dom["ms"] / dom["launches"], 4),
                 "flops_per_launch": dom["flops"] / dom["launches"],

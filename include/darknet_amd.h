@@ -181,10 +181,10 @@ void forward_convolutional_layer_gpu(layer l, network net); /* src/convolutional
 void forward_maxpool_layer_gpu(layer l, network net);       /* src/maxpool_layer_kernels.cu:87 */
 void forward_route_layer_gpu(layer l, network net);         /* src/route_layer.c:105 */
 void forward_shortcut_layer_gpu(layer l, network net);      /* src/shortcut_layer.c:77 */
-void forward_upsample_layer_gpu(layer l, network net);      /* src/upsample_layer.c:91 */
+void forward_upsample_layer_gpu(layer l, network net);      /* src/upsample_layer.c:88 */
 void forward_yolo_layer_gpu(layer l, network net);          /* src/yolo_layer.c:347 */
 void forward_avgpool_layer_gpu(layer l, network net);       /* src/avgpool_layer_kernels.cu:46 */
-void forward_softmax_layer_gpu(layer l, network net);       /* src/softmax_layer.c:82 */
+void forward_softmax_layer_gpu(layer l, network net);       /* src/softmax_layer.c:71 */
 void push_convolutional_layer(layer l);                     /* src/convolutional_kernels.cu:286 */
 void pull_convolutional_layer(layer l);                     /* src/convolutional_kernels.cu:270 */
 
