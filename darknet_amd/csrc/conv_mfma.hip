@@ -75,6 +75,11 @@ struct mfma_args {
     int bn, act;
     int tiles_m, tiles_n, per_xcd;
     unsigned in_records; /* bytes the tap-blocked gather may address: input + bias row */
+    /* K-split tail: tiles [0, whole_tiles) are computed in one piece by workgroups
+     * [0, 8*per_xcd); every later workgroup j computes K-slice j % split of tile
+     * whole_tiles + j / split and leaves raw accumulators in `partial` for the reduce kernel */
+    int whole_tiles, split;
+    float *partial;
 };
 
 /* k -> (channel, ky, kx) for a size x size kernel in the reference's im2col row order. */
@@ -99,8 +104,58 @@ __device__ __forceinline__ void split_k(int k, int size, int &ci, int &ky, int &
     }
 }
 
+/* Activations other than leaky / linear: out of line, so that the 64-element epilogue does not
+ * carry 64 inlined copies of the double-precision exp() expansions (the kernel grew to 45k
+ * instructions and spilled that way). */
+__device__ __attribute__((noinline)) float activate_rare(float x, int a) { return dn_activate(x, a); }
+
+/* Batch-norm / bias / activation and the store.  Accumulator register r of lane l holds row
+ * 8*(r/4) + 4*(l/32) + r%4 and column l%32 of its 32x32 block. */
+template <int TM, int TN>
+__device__ __forceinline__ void conv_epilogue(const mfma_args &a, f32x16 (&acc)[TM][TN], const dn_bn_row *rows,
+                                              int m0, long n0, int wm0, int wn0, int li, int kh)
+{
+#pragma unroll
+    for (int j = 0; j < TN; ++j) {
+        const long n = n0 + wn0 + j * 32 + li;
+        if (n >= a.Ntotal) continue;
+        const int b = (int)(n / a.P);
+        const int p = (int)(n - (long)b * a.P);
+        float *obase = a.out + (long)b * a.M * a.P + p;
+#pragma unroll
+        for (int i = 0; i < TM; ++i) {
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                const int ml = wm0 + i * 32 + 8 * (r >> 2) + 4 * kh + (r & 3);
+                const int m = m0 + ml;
+                if (m >= a.M) continue;
+                const float y = dn_bn_apply(acc[i][j][r], rows[ml], a.bn);
+                float z;
+                if (a.act == DN_LEAKY) z = (y > 0) ? y : (float)(.1 * (double)y);
+                else if (a.act == DN_LINEAR) z = y;
+                else z = activate_rare(y, a.act);
+                obase[(long)m * a.P] = z;
+            }
+        }
+    }
+}
+
+/* Per-filter batch-norm constants of a tile into LDS. */
+template <int BM>
+__device__ __forceinline__ void stage_bn_rows(const mfma_args &a, dn_bn_row *rows, int m0, int tid)
+{
+    for (int i = tid; i < BM; i += DN_THREADS) {
+        const int m = m0 + i;
+        dn_bn_row r = dn_bn_make(0, 0.f, 1.f, 0.f, 1.f);
+        if (m < a.M)
+            r = dn_bn_make(a.bn, a.biases[m], a.bn ? a.scales[m] : 1.f, a.bn ? a.mean[m] : 0.f,
+                           a.bn ? a.var[m] : 1.f);
+        rows[i] = r;
+    }
+}
+
 template <int BM, int BN, int WM, int WN, int MODE>
-__global__ __launch_bounds__(DN_THREADS, 4) void conv_mfma_kernel(mfma_args a)
+__global__ __launch_bounds__(DN_THREADS, (BM == 128 ? 3 : 2)) void conv_mfma_kernel(mfma_args a)
 {
     constexpr int TM = WM / 32, TN = WN / 32;
     constexpr int WAVES_N = BN / WN;
@@ -117,8 +172,17 @@ __global__ __launch_bounds__(DN_THREADS, 4) void conv_mfma_kernel(mfma_args a)
 
     /* XCD-aware tile order: workgroup id -> (xcd, slot) -> linear tile with tile_m fastest. */
     const int bid = blockIdx.x;
-    const int lin = (bid & 7) * a.per_xcd + (bid >> 3);
-    if (lin >= a.tiles_m * a.tiles_n) return;
+    int lin, kc_begin = 0, kc_end = a.KCH, slice_id = -1;
+    if (bid < 8 * a.per_xcd) {
+        lin = (bid & 7) * a.per_xcd + (bid >> 3);
+        if (lin >= a.whole_tiles) return;
+    } else {
+        slice_id = bid - 8 * a.per_xcd;
+        const int t = slice_id / a.split, sl = slice_id - t * a.split;
+        lin = a.whole_tiles + t;
+        kc_begin = (int)((long)sl * a.KCH / a.split);
+        kc_end = (int)((long)(sl + 1) * a.KCH / a.split);
+    }
     const int tile_m = lin % a.tiles_m;
     const int tile_n = lin / a.tiles_m;
     const int m0 = tile_m * BM;
@@ -130,15 +194,7 @@ __global__ __launch_bounds__(DN_THREADS, 4) void conv_mfma_kernel(mfma_args a)
     const int wm0 = (wave / WAVES_N) * WM;
     const int wn0 = (wave % WAVES_N) * WN;
 
-    /* per-filter batch-norm constants of this tile */
-    for (int i = tid; i < BM; i += DN_THREADS) {
-        const int m = m0 + i;
-        dn_bn_row r = dn_bn_make(0, 0.f, 1.f, 0.f, 1.f);
-        if (m < a.M)
-            r = dn_bn_make(a.bn, a.biases[m], a.bn ? a.scales[m] : 1.f, a.bn ? a.mean[m] : 0.f,
-                           a.bn ? a.var[m] : 1.f);
-        rows[i] = r;
-    }
+    stage_bn_rows<BM>(a, rows, m0, tid);
 
     /* ---- gather bookkeeping: this thread's output pixel for the B tile ---- */
     const int bn_local = tid % BN;              /* column of the tile this thread gathers */
@@ -174,7 +230,7 @@ __global__ __launch_bounds__(DN_THREADS, 4) void conv_mfma_kernel(mfma_args a)
     }
     const int HW = a.H * a.W;
     /* tap-blocked loop state of the chunk being fetched (wave-uniform) */
-    int ld_tap = 0, ld_cb = 0;
+    int ld_cb = kc_begin / TAPS, ld_tap = kc_begin - (kc_begin / TAPS) * TAPS;
     /* Buffer view of the input for the tap-blocked gather.  A buffer load adds a per-lane
      * 32-bit offset and a scalar offset to the descriptor's base and returns 0, without touching
      * memory, when the sum reaches num_records: lanes whose tap is outside the image get the
@@ -275,7 +331,7 @@ __global__ __launch_bounds__(DN_THREADS, 4) void conv_mfma_kernel(mfma_args a)
     const int li = lane & 31; /* row of A / column of B inside a 32x32 block */
     const int kh = lane >> 5; /* which half of the k pair this lane feeds */
 
-    load_chunk(0);
+    load_chunk(kc_begin);
     store_chunk(0);
     __syncthreads();
 
@@ -335,43 +391,87 @@ __global__ __launch_bounds__(DN_THREADS, 4) void conv_mfma_kernel(mfma_args a)
         mfma_half(1);
     };
 
-    int kc = 0;
+    int kc = kc_begin;
     /* two chunks per trip so the LDS buffer index is a compile-time constant in each half */
-    for (; kc + 2 < a.KCH; kc += 2) {
+    for (; kc + 2 < kc_end; kc += 2) {
         step(kc + 1, 0);
         step(kc + 2, 1);
     }
-    if (kc + 1 < a.KCH) { /* KCH even: one more full step, then the last chunk from buffer 1 */
+    if (kc + 1 < kc_end) { /* even count: one more full step, then the last chunk from buffer 1 */
         step(kc + 1, 0);
         last(1);
     } else {
         last(0);
     }
 
-    /* ---- epilogue: accumulator register r of lane l holds row 8*(r/4) + 4*(l/32) + r%4 and
-     * column l%32 of its 32x32 block ---- */
+    if (slice_id >= 0) {
+        /* K-slice: park the raw accumulators, lane-major so every store is a full 256-byte row */
+        float *ws = a.partial + (long)slice_id * (BM * BN);
 #pragma unroll
-    for (int j = 0; j < TN; ++j) {
-        const long n = n0 + wn0 + j * 32 + li;
-        if (n >= a.Ntotal) continue;
-        const int b = (int)(n / a.P);
-        const int p = (int)(n - (long)b * a.P);
-        float *obase = a.out + (long)b * a.M * a.P + p;
+        for (int i = 0; i < TM; ++i)
 #pragma unroll
-        for (int i = 0; i < TM; ++i) {
+            for (int j = 0; j < TN; ++j)
 #pragma unroll
-            for (int r = 0; r < 16; ++r) {
-                const int ml = wm0 + i * 32 + 8 * (r >> 2) + 4 * kh + (r & 3);
-                const int m = m0 + ml;
-                if (m >= a.M) continue;
-                const float y = dn_bn_apply(acc[i][j][r], rows[ml], a.bn);
-                float z;
-                if (a.act == DN_LEAKY) z = dn_activate_t<DN_LEAKY>(y);
-                else if (a.act == DN_LINEAR) z = y;
-                else z = dn_activate(y, a.act);
-                obase[(long)m * a.P] = z;
-            }
-        }
+                for (int r = 0; r < 16; ++r)
+                    ws[((wave * TM * TN + i * TN + j) * 16 + r) * 64 + lane] = acc[i][j][r];
+        return;
+    }
+
+    conv_epilogue<TM, TN>(a, acc, rows, m0, n0, wm0, wn0, li, kh);
+}
+
+/* Sums the K-slices of the tail tiles in slice order (deterministic) and applies the epilogue.
+ * A thread owns four consecutive lanes' worth of one accumulator register: one 16-byte read per
+ * slice, four consecutive output columns of one filter row.  Many small workgroups, because a
+ * handful of tail tiles must still spread over the whole chip. */
+template <int BM, int BN, int WM, int WN>
+__global__ __launch_bounds__(DN_THREADS) void conv_reduce_kernel(mfma_args a)
+{
+    constexpr int TM = WM / 32, TN = WN / 32;
+    constexpr int WAVES_N = BN / WN;
+    constexpr int GROUPS_PER_TILE = BM * BN / 4 / DN_THREADS; /* workgroups per tile */
+    const int t = blockIdx.x / GROUPS_PER_TILE;
+    const int e = ((blockIdx.x - t * GROUPS_PER_TILE) * DN_THREADS + threadIdx.x) * 4; /* first element */
+    const int lin = a.whole_tiles + t;
+    const int m0 = (lin % a.tiles_m) * BM;
+    const long n0 = (long)(lin / a.tiles_m) * BN;
+    /* e = ((wave*TM*TN + i*TN + j)*16 + r)*64 + lane */
+    const int lane = e & 63;
+    int q = e >> 6;
+    const int r = q & 15;
+    q >>= 4;
+    const int j = q % TN;
+    q /= TN;
+    const int i = q % TM;
+    const int wave = q / TM;
+    const int ml = (wave / WAVES_N) * WM + i * 32 + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
+    const int m = m0 + ml;
+    const long n = n0 + (wave % WAVES_N) * WN + j * 32 + (lane & 31);
+    float4 sum = make_float4(0.f, 0.f, 0.f, 0.f);
+    const float4 *ws = (const float4 *)(a.partial + (long)t * a.split * (BM * BN) + e);
+    for (int sl = 0; sl < a.split; ++sl) {
+        const float4 v = ws[(long)sl * (BM * BN / 4)];
+        sum.x += v.x;
+        sum.y += v.y;
+        sum.z += v.z;
+        sum.w += v.w;
+    }
+    if (m >= a.M) return;
+    const dn_bn_row row = dn_bn_make(a.bn, a.biases[m], a.bn ? a.scales[m] : 1.f, a.bn ? a.mean[m] : 0.f,
+                                     a.bn ? a.var[m] : 1.f);
+    const float vals[4] = {sum.x, sum.y, sum.z, sum.w};
+#pragma unroll
+    for (int c = 0; c < 4; ++c) {
+        const long nc = n + c;
+        if (nc >= a.Ntotal) break;
+        const int b = (int)(nc / a.P);
+        const int p = (int)(nc - (long)b * a.P);
+        const float y = dn_bn_apply(vals[c], row, a.bn);
+        float z;
+        if (a.act == DN_LEAKY) z = (y > 0) ? y : (float)(.1 * (double)y);
+        else if (a.act == DN_LINEAR) z = y;
+        else z = activate_rare(y, a.act);
+        a.out[((long)b * a.M + m) * a.P + p] = z;
     }
 }
 
@@ -448,6 +548,37 @@ extern "C" const char *conv_kernel_name(int n, int c, int groups, int size)
 static float *g_scratch = 0;       /* per-call repack buffer for callers without a packed copy */
 static size_t g_scratch_floats = 0;
 
+static float *g_partial = 0; /* K-slice accumulators of tail tiles, grown on demand */
+static size_t g_partial_floats = 0;
+static int g_cus = 0;
+
+/* How to cover `tiles` equal tiles on `cus` compute units.  Whole tiles are dealt out in rounds;
+ * a remainder that would leave most CUs idle for a whole tile time (or, at batch 1, a grid far
+ * smaller than the chip) is cut along K into `split` slices each, reduced afterwards.
+ * Returns the number of whole tiles; *split = 1 means no tail. */
+static long plan_split(long tiles, int kch, int cus, int *split)
+{
+    *split = 1;
+    if (g_algo == 3 || cus <= 0) return tiles;
+    const long whole = tiles / cus * cus;
+    const long tail = tiles - whole;
+    if (tail == 0 || tail * 10 >= (long)cus * 9) return tiles; /* a nearly full round: leave it */
+    /* Time in units of one 16-wide K chunk.  A workgroup costs its chunks plus a fixed part
+     * (first load latency, epilogue or partial store); the reduce pass costs a little more. */
+    const double fixed_whole = 5.0, fixed_slice = 8.0, reduce = 4.0;
+    double best = (double)kch + fixed_whole;                   /* the tail as whole tiles */
+    const int max_s = kch / 4 < 32 ? kch / 4 : 32;             /* at least 4 chunks per slice */
+    for (int s = 2; s <= max_s; ++s) {
+        const long rounds = (tail * s + cus - 1) / cus;
+        const double cost = rounds * ((double)kch / s + fixed_slice) + reduce;
+        if (cost < 0.9 * best) {
+            best = cost / 0.9;                                 /* later candidates must beat this one outright */
+            *split = s;
+        }
+    }
+    return *split > 1 ? whole : tiles;
+}
+
 template <int BM, int BN, int WM, int WN>
 static void launch_tile(const mfma_args &a0, int mode)
 {
@@ -455,8 +586,28 @@ static void launch_tile(const mfma_args &a0, int mode)
     a.tiles_m = (a.M + BM - 1) / BM;
     a.tiles_n = (int)((a.Ntotal + BN - 1) / BN);
     const long total = (long)a.tiles_m * a.tiles_n;
-    a.per_xcd = (int)((total + 7) / 8);
-    const dim3 grid((unsigned)(a.per_xcd * 8));
+    if (!g_cus) {
+        hipDeviceProp_t prop;
+        hip_check_error(hipGetDeviceProperties(&prop, hip_get_device()));
+        g_cus = prop.multiProcessorCount;
+    }
+    int split = 1;
+    const long whole = plan_split(total, a.KCH, g_cus, &split);
+    const long tail = total - whole;
+    a.whole_tiles = (int)whole;
+    a.split = split;
+    a.per_xcd = (int)((whole + 7) / 8);
+    a.partial = 0;
+    if (tail > 0) {
+        const size_t need = (size_t)tail * split * BM * BN;
+        if (need > g_partial_floats) {
+            if (g_partial) hip_free(g_partial);
+            g_partial = hip_make_array(0, need);
+            g_partial_floats = need;
+        }
+        a.partial = g_partial;
+    }
+    const dim3 grid((unsigned)(a.per_xcd * 8 + tail * split));
     if (BM > 128 && mode != 11 && mode != 13) dn_fatal("conv dispatch: the 256-row tile is only built for the tap-blocked modes");
     switch (mode) {
     case 11: hipLaunchKernelGGL((conv_mfma_kernel<BM, BN, WM, WN, 11>), grid, dim3(DN_THREADS), 0, dn_stream(), a); break;
@@ -472,6 +623,9 @@ static void launch_tile(const mfma_args &a0, int mode)
         }
         break;
     }
+    if (tail > 0)
+        hipLaunchKernelGGL((conv_reduce_kernel<BM, BN, WM, WN>), dim3((unsigned)(tail * (BM * BN / 4 / DN_THREADS))),
+                           dim3(DN_THREADS), 0, dn_stream(), a);
 }
 
 /* Which kernel variant serves a geometry: -1 = direct kernel, else the MODE template value. */
@@ -556,6 +710,9 @@ extern "C" void forward_convolutional_gpu(const float *input, const float *weigh
     a.bn = batch_normalize ? 1 : 0;
     a.act = activation;
     a.tiles_m = a.tiles_n = a.per_xcd = 0;
+    a.whole_tiles = 0;
+    a.split = 1;
+    a.partial = 0;
     a.in_records = (unsigned)((long)batch * c * h * w * 4 + (long)(w + 1) * 4);
     if (n <= 32)
         launch_tile<32, 256, 32, 64>(a, mode);

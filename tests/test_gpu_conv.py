@@ -130,7 +130,11 @@ def test_conv_linearity_at_full_size(dn):
     zero = np.zeros(n, np.float32)
     kw = dict(n=n, size=3, stride=1, pad=1, groups=1, bn=0, act="linear")
     y = run_conv(dn, x1, wt, zero, None, None, None, **kw)
-    assert all(np.array_equal(y[0], y[i]) for i in (1, 17, 63))
+    # copies agree to rounding: tiles of the last, partial round are summed in K-slices, so an
+    # image that falls there sees a different (fixed) summation order than one that does not
+    assert all(norm_err(y[i], y[0]) <= 1e-5 for i in (1, 17, 63))
+    y_again = run_conv(dn, x1, wt, zero, None, None, None, **kw)
+    assert np.array_equal(y, y_again)                      # run-to-run deterministic
     x2 = synth.uniform(5, b * c * h * w).reshape(b, c, h, w)
     y2 = run_conv(dn, x2, wt, zero, None, None, None, **kw)
     y12 = run_conv(dn, x1 + x2, wt, zero, None, None, None, **kw)

