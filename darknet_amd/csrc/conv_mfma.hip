@@ -46,14 +46,6 @@
 typedef float f32x16 __attribute__((ext_vector_type(16)));
 
 #define DN_BK 16
-#define DN_LDK 16 /* LDS row, floats: unpadded, the 16-byte slots of a row are XOR-swizzled */
-
-/* LDS address (in floats) of the 16-byte slot `kq` (0..3) of row `row`.  Rows are 64 bytes, so
- * four rows span the 64 banks; XOR-ing the slot with bits 2..3 of the row spreads any 16
- * consecutive rows read at the same slot over all 16 four-bank groups (conflict free for
- * ds_read_b128 / ds_write_b128) without the padding that would cost a fourth resident
- * workgroup per CU. */
-__device__ __forceinline__ int lds_slot(int row, int kq) { return row * DN_LDK + ((kq ^ (row >> 2)) & 3) * 4; }
 #define DN_MPAD 128
 #define DN_THREADS 256
 
@@ -74,7 +66,8 @@ struct mfma_args {
     int stride, pad, size;
     int bn, act;
     int tiles_m, tiles_n, per_xcd;
-    unsigned in_records; /* bytes the tap-blocked gather may address: input + bias row */
+    unsigned in_records; /* bytes the gather may address: input + bias row */
+    unsigned wp_records; /* bytes of the packed weights */
     /* K-split tail: tiles [0, whole_tiles) are computed in one piece by workgroups
      * [0, 8*per_xcd); every later workgroup j computes K-slice j % split of tile
      * whole_tiles + j / split and leaves raw accumulators in `partial` for the reduce kernel */
@@ -163,11 +156,12 @@ __global__ __launch_bounds__(DN_THREADS, (BM == 128 ? 3 : 2)) void conv_mfma_ker
     constexpr bool TAPB = MODE >= 10;             /* tap-blocked K order */
     constexpr int KS = TAPB ? MODE - 10 : MODE;    /* kernel size known at compile time (0 = runtime) */
     constexpr int TAPS = KS == 3 ? 9 : 1;
-    constexpr int A_F4 = (BM * 4 + DN_THREADS - 1) / DN_THREADS; /* float4 loads of A per thread */
-    constexpr int B_G = BN / 64;                                  /* 4-k groups of B per thread */
 
-    __shared__ __attribute__((aligned(16))) float As[2][BM * DN_LDK];
-    __shared__ __attribute__((aligned(16))) float Bs[2][BN * DN_LDK];
+    /* Four separate LDS objects rather than two [2][...] arrays: the compiler makes every LDS read
+     * wait (vmcnt) for direct-to-LDS loads it cannot prove disjoint from it, and it can only
+     * prove that for distinct objects. */
+    __shared__ __attribute__((aligned(16))) float As0[BM * DN_BK], As1[BM * DN_BK];
+    __shared__ __attribute__((aligned(16))) float Bs0[BN * DN_BK], Bs1[BN * DN_BK];
     __shared__ dn_bn_row rows[BM];
 
     /* XCD-aware tile order: workgroup id -> (xcd, slot) -> linear tile with tile_m fastest. */
@@ -196,127 +190,127 @@ __global__ __launch_bounds__(DN_THREADS, (BM == 128 ? 3 : 2)) void conv_mfma_ker
 
     stage_bn_rows<BM>(a, rows, m0, tid);
 
-    /* ---- gather bookkeeping: this thread's output pixel for the B tile ---- */
-    const int bn_local = tid % BN;              /* column of the tile this thread gathers */
-    const int kq0 = __builtin_amdgcn_readfirstlane(tid / BN); /* first 4-k group (wave-uniform) */
-    constexpr int KQ_STEP = DN_THREADS / BN;    /* distance between this thread's groups */
-    const long ncol = n0 + bn_local;
-    const bool col_ok = ncol < a.Ntotal;
-    int iy0 = 0, ix0 = 0, pix = 0;
-    const float *img = a.in;
-    unsigned voff_center = 0; /* tap-blocked: byte offset of (image b, channel 0, oy*stride, ox*stride) */
-    unsigned vmask = 0;       /* tap-blocked: bit ky*3+kx set when that tap lies inside the image */
-    {
-        const long nn = col_ok ? ncol : 0;
+    /* ---- global -> LDS without passing through registers ------------------------------------
+     * A buffer load with the LDS modifier writes lane i's dword (or 16 bytes) to
+     * lds_base + i*4 (i*16); lanes whose offset is out of range write zeros.  The layouts are
+     * chosen so that those wave-contiguous images are exactly what the MFMA operand reads want:
+     *   LDS   A: [slot q = 0..3][row m][4 floats],  B: [slot q][column n][4 floats]  (k = 4q + j)
+     *   A wave-load: 64 rows of one slot, 16 bytes per lane - the packed weights are stored
+     *                [chunk][slot][Mpad][4] so this is one contiguous kilobyte;
+     *   B wave-load: 16 consecutive columns x the 4 k of one slot, lane = 4*column + j.
+     * No ds_write, no staging registers; completion is tracked by vmcnt. */
+    constexpr int A_WAVE_LOADS = BM * 4 / 64;            /* wave-loads of A per chunk (8, 4 or 2) */
+    constexpr int A_PER_WAVE = (A_WAVE_LOADS + 3) / 4;   /* 2, 1, 1 */
+    constexpr int NG = BN / 16;                          /* 16-column groups per tile */
+    constexpr int NG_PER_WAVE = NG / 4;                  /* 2 (BN=128) or 4 (BN=256) */
+    const int nl = lane >> 2;                            /* column inside a 16-group */
+    const int kk = lane & 3;                             /* k inside a slot */
+    const int HW = a.H * a.W;
+
+    const __amdgpu_buffer_rsrc_t w_rsrc = __builtin_amdgcn_make_buffer_rsrc(
+        (void *)a.wp, 0, (int)a.wp_records, 0x00020000);
+    const int bias = (TAPB && KS == 3) ? a.W + 1 : 0;
+    const __amdgpu_buffer_rsrc_t in_rsrc = __builtin_amdgcn_make_buffer_rsrc(
+        (void *)(a.in - bias), 0, (int)a.in_records, 0x00020000);
+
+    /* per column group handled by this wave: the lane's pixel */
+    unsigned voff_px[NG_PER_WAVE]; /* tap-blocked: byte offset of (image, channel kk, oy*s, ox*s) */
+    unsigned vmask[NG_PER_WAVE];   /* tap-blocked: bit t set when tap t lies inside the image */
+    int iy0[NG_PER_WAVE], ix0[NG_PER_WAVE];
+    long img_off[NG_PER_WAVE];     /* reference order: float offset of the lane's image */
+    bool col_ok[NG_PER_WAVE];
+#pragma unroll
+    for (int g = 0; g < NG_PER_WAVE; ++g) {
+        const long ncol = n0 + (wave * NG_PER_WAVE + g) * 16 + nl;
+        col_ok[g] = ncol < a.Ntotal;
+        const long nn = col_ok[g] ? ncol : 0;
         const int b = (int)(nn / a.P);
         const int p = (int)(nn - (long)b * a.P);
         const int oy = p / a.OW;
         const int ox = p - oy * a.OW;
-        iy0 = oy * a.stride - a.pad;
-        ix0 = ox * a.stride - a.pad;
-        pix = iy0 * a.W + ix0;                       /* may be negative near the border */
-        img = a.in + (long)b * a.C * a.H * a.W;      /* this column's image */
-        if (TAPB) {
-            voff_center = (unsigned)(((long)b * a.C * a.H * a.W + (long)(oy * a.stride) * a.W + ox * a.stride) * 4);
-            if (col_ok) {
+        iy0[g] = oy * a.stride - a.pad;
+        ix0[g] = ox * a.stride - a.pad;
+        img_off[g] = (long)b * a.C * HW;
+        voff_px[g] = (unsigned)((img_off[g] + (long)kk * HW + (long)(oy * a.stride) * a.W + ox * a.stride) * 4);
+        vmask[g] = 0;
+        if (TAPB && col_ok[g]) {
 #pragma unroll
-                for (int t = 0; t < TAPS; ++t) {
-                    const int ky = t / 3, kx = t % 3;
-                    if (KS == 1 || ((unsigned)(iy0 + ky) < (unsigned)a.H && (unsigned)(ix0 + kx) < (unsigned)a.W))
-                        vmask |= 1u << t;
-                }
+            for (int t = 0; t < TAPS; ++t) {
+                const int ky = t / 3, kx = t % 3;
+                if (KS == 1 || ((unsigned)(iy0[g] + ky) < (unsigned)a.H && (unsigned)(ix0[g] + kx) < (unsigned)a.W))
+                    vmask[g] |= 1u << t;
             }
         }
     }
-    const int HW = a.H * a.W;
     /* tap-blocked loop state of the chunk being fetched (wave-uniform) */
     int ld_cb = kc_begin / TAPS, ld_tap = kc_begin - (kc_begin / TAPS) * TAPS;
-    /* Buffer view of the input for the tap-blocked gather.  A buffer load adds a per-lane
-     * 32-bit offset and a scalar offset to the descriptor's base and returns 0, without touching
-     * memory, when the sum reaches num_records: lanes whose tap is outside the image get the
-     * offset 0xFFFFFFFC and read their zero for free.  The base sits (W+1) floats below the
-     * tensor so the scalar offset of the top-left tap of channel 0 is still non-negative; no
-     * lane ever resolves to an address below the tensor. */
-    const int bias = KS == 1 ? 0 : a.W + 1;
-    const __amdgpu_buffer_rsrc_t in_rsrc = __builtin_amdgcn_make_buffer_rsrc(
-        (void *)(a.in - bias), 0, (int)a.in_records, 0x00020000);
 
-    float a_reg[A_F4][4]; /* scalars, not float4: keeps the staging registers out of memory */
-    float b_reg[B_G][4];
+    typedef __attribute__((address_space(3))) void *lds_ptr;
 
-    auto load_chunk = [&](int kc) {
-        /* A: contiguous block of BM*16 floats */
-        const float4 *src = (const float4 *)(a.wp + ((long)kc * a.Mpad + m0) * DN_BK);
+    auto load_chunk = [&](int kc, int buf) {
+        /* A */
 #pragma unroll
-        for (int i = 0; i < A_F4; ++i) {
-            const int idx = tid + i * DN_THREADS;
-            if (BM * 4 >= DN_THREADS || idx < BM * 4) {
-                const float4 t = src[idx];
-                a_reg[i][0] = t.x;
-                a_reg[i][1] = t.y;
-                a_reg[i][2] = t.z;
-                a_reg[i][3] = t.w;
+        for (int i = 0; i < A_PER_WAVE; ++i) {
+            const int wl = wave * A_PER_WAVE + i;        /* wave-load index: slot q, 64-row block rb */
+            if (A_WAVE_LOADS >= 4 || wl < A_WAVE_LOADS) {
+                constexpr int RB = BM / 64 > 0 ? BM / 64 : 1; /* 64-row blocks per slot (BM >= 64) */
+                const int q = BM >= 64 ? wl / RB : wl / 1;
+                const int rb = BM >= 64 ? wl - q * RB : 0;
+                if (BM >= 64) {
+                    const unsigned soff = (unsigned)((((long)kc * 4 + q) * a.Mpad + m0 + rb * 64) * 16);
+                    __builtin_amdgcn_raw_ptr_buffer_load_lds(w_rsrc, (lds_ptr)&(buf ? As1 : As0)[(q * BM + rb * 64) * 4], 16,
+                                                             lane * 16, soff, 0, 0);
+                } else {
+                    /* BM == 32: one wave-load covers two slots of 32 rows each */
+                    const int q2 = wl * 2 + (lane >> 5);
+                    const unsigned voff = (unsigned)((((long)q2 * a.Mpad) + (lane & 31)) * 16);
+                    const unsigned soff = (unsigned)(((long)kc * 4 * a.Mpad + m0) * 16);
+                    __builtin_amdgcn_raw_ptr_buffer_load_lds(w_rsrc, (lds_ptr)&(buf ? As1 : As0)[(wl * 2 * BM) * 4], 16, voff,
+                                                             soff, 0, 0);
+                }
             }
         }
-        /* B: gathered */
+        /* B */
         if (TAPB) {
             const int ky = (ld_tap * 11) >> 5, kx = ld_tap - 3 * ((ld_tap * 11) >> 5); /* tap/3, tap%3 */
             const int shift = KS == 1 ? 0 : (ky - 1) * a.W + (kx - 1);       /* pad == 1 for 3x3 */
             const unsigned soff0 = (unsigned)((ld_cb * 16 * HW + shift + bias) * 4); /* wave-uniform */
-            const unsigned voff = ((vmask >> ld_tap) & 1u) ? voff_center : 0xFFFFFFFCu;
 #pragma unroll
-            for (int g = 0; g < B_G; ++g) {
+            for (int g = 0; g < NG_PER_WAVE; ++g) {
+                const unsigned voff = ((vmask[g] >> ld_tap) & 1u) ? voff_px[g] : 0xFFFFFFFCu;
+                const int ng = wave * NG_PER_WAVE + g;
 #pragma unroll
-                for (int j = 0; j < 4; ++j) {
-                    const int i = (kq0 + g * KQ_STEP) * 4 + j; /* channel inside the block, uniform */
-                    b_reg[g][j] = __builtin_bit_cast(
-                        float, __builtin_amdgcn_raw_buffer_load_b32(in_rsrc, voff, soff0 + (unsigned)(i * HW * 4), 0));
-                }
+                for (int q = 0; q < 4; ++q)
+                    __builtin_amdgcn_raw_ptr_buffer_load_lds(in_rsrc, (lds_ptr)&(buf ? Bs1 : Bs0)[(q * BN + ng * 16) * 4], 4,
+                                                             voff, soff0 + (unsigned)(q * 4 * HW * 4), 0, 0);
             }
             if (++ld_tap == TAPS) {
                 ld_tap = 0;
                 ++ld_cb;
             }
-            return;
-        }
+        } else {
+            /* reference K order: every lane splits its own k */
 #pragma unroll
-        for (int g = 0; g < B_G; ++g) {
-            const int kbase = kc * DN_BK + (kq0 + g * KQ_STEP) * 4;
+            for (int g = 0; g < NG_PER_WAVE; ++g) {
+                const int ng = wave * NG_PER_WAVE + g;
 #pragma unroll
-            for (int j = 0; j < 4; ++j) {
-                const int k = kbase + j;
-                int ci, ky, kx;
-                split_k<KS>(k, a.size, ci, ky, kx);
-                /* branch-free: an out-of-range tap reads element 0 of the image (always mapped)
-                 * and is replaced by zero afterwards, so a chunk's loads issue back to back */
-                bool ok = col_ok & (k < a.K);
-                int off = ci * HW;
-                if (KS != 1) {
-                    ok = ok & ((unsigned)(iy0 + ky) < (unsigned)a.H) & ((unsigned)(ix0 + kx) < (unsigned)a.W);
-                    off += ky * a.W + kx;
+                for (int q = 0; q < 4; ++q) {
+                    const int k = kc * DN_BK + q * 4 + kk;
+                    int ci, ky, kx;
+                    split_k<KS>(k, a.size, ci, ky, kx);
+                    bool ok = col_ok[g] & (k < a.K);
+                    long off = img_off[g] + (long)ci * HW;
+                    if (KS != 1) {
+                        ok = ok & ((unsigned)(iy0[g] + ky) < (unsigned)a.H) & ((unsigned)(ix0[g] + kx) < (unsigned)a.W);
+                        off += (long)(iy0[g] + ky) * a.W + ix0[g] + kx;
+                    } else {
+                        off += (long)iy0[g] * a.W + ix0[g];
+                    }
+                    const unsigned voff = ok ? (unsigned)(off * 4) : 0xFFFFFFFCu;
+                    __builtin_amdgcn_raw_ptr_buffer_load_lds(in_rsrc, (lds_ptr)&(buf ? Bs1 : Bs0)[(q * BN + ng * 16) * 4], 4,
+                                                             voff, 0, 0, 0);
                 }
-                float v = img[ok ? pix + off : 0];
-                v = ok ? v : 0.f;
-                b_reg[g][j] = v;
             }
-        }
-    };
-
-    auto store_chunk = [&](int buf) {
-#pragma unroll
-        for (int i = 0; i < A_F4; ++i) {
-            const int idx = tid + i * DN_THREADS;
-            if (BM * 4 >= DN_THREADS || idx < BM * 4) {
-                const int row = idx >> 2, kq = idx & 3;
-                *(float4 *)&As[buf][lds_slot(row, kq)] =
-                    make_float4(a_reg[i][0], a_reg[i][1], a_reg[i][2], a_reg[i][3]);
-            }
-        }
-#pragma unroll
-        for (int g = 0; g < B_G; ++g) {
-            const int kq = kq0 + g * KQ_STEP;
-            *(float4 *)&Bs[buf][lds_slot(bn_local, kq)] =
-                make_float4(b_reg[g][0], b_reg[g][1], b_reg[g][2], b_reg[g][3]);
         }
     };
 
@@ -331,8 +325,8 @@ __global__ __launch_bounds__(DN_THREADS, (BM == 128 ? 3 : 2)) void conv_mfma_ker
     const int li = lane & 31; /* row of A / column of B inside a 32x32 block */
     const int kh = lane >> 5; /* which half of the k pair this lane feeds */
 
-    load_chunk(kc_begin);
-    store_chunk(0);
+    load_chunk(kc_begin, 0);
+    __builtin_amdgcn_s_waitcnt(0);
     __syncthreads();
 
     float4 av[2][TM], bv[2][TN]; /* MFMA operands of the current chunk: [k half][32-row block] */
@@ -342,10 +336,10 @@ __global__ __launch_bounds__(DN_THREADS, (BM == 128 ? 3 : 2)) void conv_mfma_ker
         for (int hb = 0; hb < 2; ++hb) {
 #pragma unroll
             for (int i = 0; i < TM; ++i)
-                av[hb][i] = *(const float4 *)&As[buf][lds_slot(wm0 + i * 32 + li, hb * 2 + kh)];
+                av[hb][i] = *(const float4 *)&(buf ? As1 : As0)[((hb * 2 + kh) * BM + wm0 + i * 32 + li) * 4];
 #pragma unroll
             for (int j = 0; j < TN; ++j)
-                bv[hb][j] = *(const float4 *)&Bs[buf][lds_slot(wn0 + j * 32 + li, hb * 2 + kh)];
+                bv[hb][j] = *(const float4 *)&(buf ? Bs1 : Bs0)[((hb * 2 + kh) * BN + wn0 + j * 32 + li) * 4];
         }
     };
 
@@ -364,25 +358,20 @@ __global__ __launch_bounds__(DN_THREADS, (BM == 128 ? 3 : 2)) void conv_mfma_ker
         }
     };
 
-    /* One pipeline step.  Program order, pinned by scheduling barriers (left alone, the compiler
-     * hoists the LDS stores above the MFMAs and waits on loads it has just issued):
-     *   1. global/buffer loads of chunk kc+1 into registers
-     *   2. all LDS operand reads of chunk kc, then the first half of its MFMAs
-     *   3. the prefetched chunk goes to the other LDS buffer - in the middle of the MFMA phase,
-     *      so the store latency hides under the second half instead of sitting in front of
-     *      the barrier
-     *   4. second half of the MFMAs, barrier */
+    /* One pipeline step, in program order (pinned by scheduling barriers):
+     *   1. direct-to-LDS loads of chunk kc+1 into the other buffer (nobody reads it: every wave
+     *      passed the previous barrier only after its MFMAs had consumed that buffer)
+     *   2. LDS operand reads of chunk kc, 32 MFMAs
+     *   3. wait for this wave's loads (vmcnt), barrier: chunk kc+1 is now visible to all waves */
     auto step = [&](int kc_next, int buf) {
-        load_chunk(kc_next);
+        load_chunk(kc_next, buf ^ 1);
         __builtin_amdgcn_sched_barrier(0);
         read_operands(buf);
         __builtin_amdgcn_sched_barrier(0);
         mfma_half(0);
-        __builtin_amdgcn_sched_barrier(0);
-        store_chunk(buf ^ 1);
-        __builtin_amdgcn_sched_barrier(0);
         mfma_half(1);
         __builtin_amdgcn_sched_barrier(0);
+        __builtin_amdgcn_s_waitcnt(0);
         __syncthreads();
     };
     auto last = [&](int buf) {
@@ -481,10 +470,14 @@ __global__ __launch_bounds__(DN_THREADS) void conv_reduce_kernel(mfma_args a)
 __global__ void pack_weights_kernel(const float *w, float *packed, int M, int K, int Mpad, long total, int taps)
 {
     for (long i = blockIdx.x * (long)blockDim.x + threadIdx.x; i < total; i += (long)gridDim.x * blockDim.x) {
-        const int kk = (int)(i % DN_BK);
-        long t = i / DN_BK;
+        /* packed index = ((chunk*4 + slot)*Mpad + m)*4 + j,  position in chunk kk = 4*slot + j */
+        const int j = (int)(i & 3);
+        long t = i >> 2;
         const int m = (int)(t % Mpad);
-        const int kc = (int)(t / Mpad);
+        t /= Mpad;
+        const int q = (int)(t & 3);
+        const int kc = (int)(t >> 2);
+        const int kk = q * 4 + j;
         int k = kc * DN_BK + kk;
         if (taps > 0) {
             const int cb = kc / taps, tap = kc - cb * taps;
@@ -633,13 +626,14 @@ static int conv_mode(int c, int groups, int size, int stride, int pad, long in_b
 {
     const long K = (long)(c / (groups > 0 ? groups : 1)) * size * size;
     if (groups != 1 || g_algo == 1 || (size == 3 && K >= 32768)) return -1;
+    /* the gather addresses the input through 32-bit buffer offsets */
+    if (in_bytes + (1L << 20) >= (1L << 32)) return -1;
     const int taps = tap_blocked_taps(c, groups, size);
     if (taps) {
-        /* the tap-blocked kernel needs pad 1 for 3x3 and 32-bit byte offsets into the input;
-         * weights of such layers are packed tap-blocked, so the rare misfits go to the direct
-         * kernel rather than to the generic MFMA kernel, which expects the reference K order */
+        /* the tap-blocked kernel needs pad 1 for 3x3; weights of such layers are packed
+         * tap-blocked, so the rare misfit goes to the direct kernel rather than to the generic
+         * MFMA kernel, which expects the reference K order */
         if (size == 3 && pad != 1) return -1;
-        if (in_bytes + (1L << 20) >= (1L << 32)) return -1; /* 32-bit buffer offsets */
         return 10 + size;
     }
     return size == 1 ? 1 : size == 3 ? 3 : 0;
@@ -714,6 +708,7 @@ extern "C" void forward_convolutional_gpu(const float *input, const float *weigh
     a.split = 1;
     a.partial = 0;
     a.in_records = (unsigned)((long)batch * c * h * w * 4 + (long)(w + 1) * 4);
+    a.wp_records = (unsigned)(conv_packed_floats(n, c, groups, size) * 4);
     if (n <= 32)
         launch_tile<32, 256, 32, 64>(a, mode);
     else if (n <= 64)
