@@ -214,32 +214,37 @@ __global__ __launch_bounds__(DN_THREADS, (BM == 128 ? 3 : 2)) void conv_mfma_ker
         (void *)(a.in - bias), 0, (int)a.in_records, 0x00020000);
 
     /* per column group handled by this wave: the lane's pixel */
-    unsigned voff_px[NG_PER_WAVE]; /* tap-blocked: byte offset of (image, channel kk, oy*s, ox*s) */
+    unsigned voff_px[NG_PER_WAVE]; /* byte offset of (image, channel kk [tap-blocked] or 0, oy*s, ox*s) */
     unsigned vmask[NG_PER_WAVE];   /* tap-blocked: bit t set when tap t lies inside the image */
-    int iy0[NG_PER_WAVE], ix0[NG_PER_WAVE];
-    long img_off[NG_PER_WAVE];     /* reference order: float offset of the lane's image */
-    bool col_ok[NG_PER_WAVE];
+    int iy0[NG_PER_WAVE], ix0[NG_PER_WAVE]; /* reference order: top-left input pixel of the window;
+                                             * a column beyond N gets iy0 far outside the image */
 #pragma unroll
     for (int g = 0; g < NG_PER_WAVE; ++g) {
         const long ncol = n0 + (wave * NG_PER_WAVE + g) * 16 + nl;
-        col_ok[g] = ncol < a.Ntotal;
-        const long nn = col_ok[g] ? ncol : 0;
+        const bool col_ok = ncol < a.Ntotal;
+        const long nn = col_ok ? ncol : 0;
         const int b = (int)(nn / a.P);
         const int p = (int)(nn - (long)b * a.P);
         const int oy = p / a.OW;
         const int ox = p - oy * a.OW;
-        iy0[g] = oy * a.stride - a.pad;
+        iy0[g] = col_ok ? oy * a.stride - a.pad : -0x1000000;
         ix0[g] = ox * a.stride - a.pad;
-        img_off[g] = (long)b * a.C * HW;
-        voff_px[g] = (unsigned)((img_off[g] + (long)kk * HW + (long)(oy * a.stride) * a.W + ox * a.stride) * 4);
+        const long img = (long)b * a.C * HW;
         vmask[g] = 0;
-        if (TAPB && col_ok[g]) {
+        if (TAPB) {
+            voff_px[g] = (unsigned)((img + (long)kk * HW + (long)(oy * a.stride) * a.W + ox * a.stride) * 4);
+            if (col_ok) {
 #pragma unroll
-            for (int t = 0; t < TAPS; ++t) {
-                const int ky = t / 3, kx = t % 3;
-                if (KS == 1 || ((unsigned)(iy0[g] + ky) < (unsigned)a.H && (unsigned)(ix0[g] + kx) < (unsigned)a.W))
-                    vmask[g] |= 1u << t;
+                for (int t = 0; t < TAPS; ++t) {
+                    const int ky = t / 3, kx = t % 3;
+                    if (KS == 1 || ((unsigned)(iy0[g] + ky) < (unsigned)a.H && (unsigned)(ix0[g] + kx) < (unsigned)a.W))
+                        vmask[g] |= 1u << t;
+                }
             }
+        } else {
+            /* (image, channel 0, window origin); the origin may lie above/left of the image, the
+             * sum with a valid tap's offset never does */
+            voff_px[g] = (unsigned)((img + (long)(oy * a.stride - a.pad) * a.W + (ox * a.stride - a.pad)) * 4);
         }
     }
     /* tap-blocked loop state of the chunk being fetched (wave-uniform) */
@@ -289,24 +294,25 @@ __global__ __launch_bounds__(DN_THREADS, (BM == 128 ? 3 : 2)) void conv_mfma_ker
                 ++ld_cb;
             }
         } else {
-            /* reference K order: every lane splits its own k */
+            /* reference K order: every lane splits its own k (4 per chunk, one per slot) */
+            int koff[4];
+            int kyx[4];
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+                const int k = kc * DN_BK + q * 4 + kk;
+                int ci, ky, kx;
+                split_k<KS>(k, a.size, ci, ky, kx);
+                koff[q] = (ci * HW + ky * a.W + kx) * 4;
+                kyx[q] = k < a.K ? (ky << 16) | kx : 0x7fff0000; /* k beyond K: fails the row test */
+            }
 #pragma unroll
             for (int g = 0; g < NG_PER_WAVE; ++g) {
                 const int ng = wave * NG_PER_WAVE + g;
 #pragma unroll
                 for (int q = 0; q < 4; ++q) {
-                    const int k = kc * DN_BK + q * 4 + kk;
-                    int ci, ky, kx;
-                    split_k<KS>(k, a.size, ci, ky, kx);
-                    bool ok = col_ok[g] & (k < a.K);
-                    long off = img_off[g] + (long)ci * HW;
-                    if (KS != 1) {
-                        ok = ok & ((unsigned)(iy0[g] + ky) < (unsigned)a.H) & ((unsigned)(ix0[g] + kx) < (unsigned)a.W);
-                        off += (long)(iy0[g] + ky) * a.W + ix0[g] + kx;
-                    } else {
-                        off += (long)iy0[g] * a.W + ix0[g];
-                    }
-                    const unsigned voff = ok ? (unsigned)(off * 4) : 0xFFFFFFFCu;
+                    const int ky = kyx[q] >> 16, kx = kyx[q] & 0xffff;
+                    const bool ok = ((unsigned)(iy0[g] + ky) < (unsigned)a.H) & ((unsigned)(ix0[g] + kx) < (unsigned)a.W);
+                    const unsigned voff = ok ? voff_px[g] + (unsigned)koff[q] : 0xFFFFFFFCu;
                     __builtin_amdgcn_raw_ptr_buffer_load_lds(in_rsrc, (lds_ptr)&(buf ? Bs1 : Bs0)[(q * BN + ng * 16) * 4], 4,
                                                              voff, 0, 0, 0);
                 }
