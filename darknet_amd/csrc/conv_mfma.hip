@@ -102,48 +102,69 @@ __device__ __forceinline__ void split_k(int k, int size, int &ci, int &ky, int &
  * instructions and spilled that way). */
 __device__ __attribute__((noinline)) float activate_rare(float x, int a) { return dn_activate(x, a); }
 
-/* Batch-norm / bias / activation and the store.  Accumulator register r of lane l holds row
- * 8*(r/4) + 4*(l/32) + r%4 and column l%32 of its 32x32 block. */
-template <int TM, int TN>
-__device__ __forceinline__ void conv_epilogue(const mfma_args &a, f32x16 (&acc)[TM][TN], const dn_bn_row *rows,
-                                              int m0, long n0, int wm0, int wn0, int li, int kh)
+typedef float float4u __attribute__((ext_vector_type(4), aligned(4)));
+
+__device__ __forceinline__ float conv_tail_one(float acc, const dn_bn_row &row, int bn, int act)
 {
+    const float y = dn_bn_apply(acc, row, bn);
+    if (act == DN_LEAKY) return (y > 0) ? y : (float)(.1 * (double)y);
+    if (act == DN_LINEAR) return y;
+    return activate_rare(y, act);
+}
+
+/* Stores four consecutive output columns n..n+3 of filter row m (one 16-byte store when they
+ * lie in one image, element by element across an image boundary or the end of N). */
+__device__ __forceinline__ void conv_store4(const mfma_args &a, int m, long n, const float v[4],
+                                            const dn_bn_row &row)
+{
+    if (n >= a.Ntotal) return;
+    const int b = (int)(n / a.P);
+    const int p = (int)(n - (long)b * a.P);
+    float *dst = a.out + ((long)b * a.M + m) * a.P + p;
+    if (p + 3 < a.P) { /* implies n + 3 < Ntotal */
+        float4u o;
+        o.x = conv_tail_one(v[0], row, a.bn, a.act);
+        o.y = conv_tail_one(v[1], row, a.bn, a.act);
+        o.z = conv_tail_one(v[2], row, a.bn, a.act);
+        o.w = conv_tail_one(v[3], row, a.bn, a.act);
+        *(float4u *)dst = o;
+        return;
+    }
 #pragma unroll
-    for (int j = 0; j < TN; ++j) {
-        const long n = n0 + wn0 + j * 32 + li;
-        if (n >= a.Ntotal) continue;
-        const int b = (int)(n / a.P);
-        const int p = (int)(n - (long)b * a.P);
-        float *obase = a.out + (long)b * a.M * a.P + p;
-#pragma unroll
-        for (int i = 0; i < TM; ++i) {
-#pragma unroll
-            for (int r = 0; r < 16; ++r) {
-                const int ml = wm0 + i * 32 + 8 * (r >> 2) + 4 * kh + (r & 3);
-                const int m = m0 + ml;
-                if (m >= a.M) continue;
-                const float y = dn_bn_apply(acc[i][j][r], rows[ml], a.bn);
-                float z;
-                if (a.act == DN_LEAKY) z = (y > 0) ? y : (float)(.1 * (double)y);
-                else if (a.act == DN_LINEAR) z = y;
-                else z = activate_rare(y, a.act);
-                obase[(long)m * a.P] = z;
-            }
-        }
+    for (int c = 0; c < 4; ++c) {
+        const long nc = n + c;
+        if (nc >= a.Ntotal) break;
+        const int bc = (int)(nc / a.P);
+        const int pc = (int)(nc - (long)bc * a.P);
+        a.out[((long)bc * a.M + m) * a.P + pc] = conv_tail_one(v[c], row, a.bn, a.act);
     }
 }
 
-/* Per-filter batch-norm constants of a tile into LDS. */
-template <int BM>
-__device__ __forceinline__ void stage_bn_rows(const mfma_args &a, dn_bn_row *rows, int m0, int tid)
+/* Batch-norm / bias / activation and the store.  The MFMAs are issued with the pixel tile as
+ * the row operand and the filter tile as the column operand, so accumulator register r of lane l
+ * holds filter (l % 32) and pixel 8*(r/4) + 4*(l/32) + r%4 of its 32x32 block: a lane owns one
+ * filter (its batch-norm constants are loaded once) and four consecutive pixels per register
+ * quad, which go out as one 16-byte store. */
+template <int TM, int TN>
+__device__ __forceinline__ void conv_epilogue(const mfma_args &a, f32x16 (&acc)[TM][TN], int m0, long n0,
+                                              int wm0, int wn0, int li, int kh)
 {
-    for (int i = tid; i < BM; i += DN_THREADS) {
-        const int m = m0 + i;
-        dn_bn_row r = dn_bn_make(0, 0.f, 1.f, 0.f, 1.f);
-        if (m < a.M)
-            r = dn_bn_make(a.bn, a.biases[m], a.bn ? a.scales[m] : 1.f, a.bn ? a.mean[m] : 0.f,
-                           a.bn ? a.var[m] : 1.f);
-        rows[i] = r;
+#pragma unroll
+    for (int i = 0; i < TM; ++i) {
+        const int m = m0 + wm0 + i * 32 + li;
+        if (m >= a.M) continue;
+        const dn_bn_row row = dn_bn_make(a.bn, a.biases[m], a.bn ? a.scales[m] : 1.f, a.bn ? a.mean[m] : 0.f,
+                                         a.bn ? a.var[m] : 1.f);
+#pragma unroll
+        for (int j = 0; j < TN; ++j) {
+#pragma unroll
+            for (int rg = 0; rg < 4; ++rg) {
+                const long n = n0 + wn0 + j * 32 + 8 * rg + 4 * kh;
+                const float v[4] = {acc[i][j][rg * 4 + 0], acc[i][j][rg * 4 + 1], acc[i][j][rg * 4 + 2],
+                                    acc[i][j][rg * 4 + 3]};
+                conv_store4(a, m, n, v, row);
+            }
+        }
     }
 }
 
@@ -162,7 +183,6 @@ __global__ __launch_bounds__(DN_THREADS, (BM == 128 ? 3 : 2)) void conv_mfma_ker
      * prove that for distinct objects. */
     __shared__ __attribute__((aligned(16))) float As0[BM * DN_BK], As1[BM * DN_BK];
     __shared__ __attribute__((aligned(16))) float Bs0[BN * DN_BK], Bs1[BN * DN_BK];
-    __shared__ dn_bn_row rows[BM];
 
     /* XCD-aware tile order: workgroup id -> (xcd, slot) -> linear tile with tile_m fastest. */
     const int bid = blockIdx.x;
@@ -187,8 +207,6 @@ __global__ __launch_bounds__(DN_THREADS, (BM == 128 ? 3 : 2)) void conv_mfma_ker
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int wm0 = (wave / WAVES_N) * WM;
     const int wn0 = (wave % WAVES_N) * WN;
-
-    stage_bn_rows<BM>(a, rows, m0, tid);
 
     /* ---- global -> LDS without passing through registers ------------------------------------
      * A buffer load with the LDS modifier writes lane i's dword (or 16 bytes) to
@@ -358,7 +376,7 @@ __global__ __launch_bounds__(DN_THREADS, (BM == 128 ? 3 : 2)) void conv_mfma_ker
 #pragma unroll
                 for (int j = 0; j < TN; ++j) {
                     const float be = s == 0 ? bv[hb][j].x : s == 1 ? bv[hb][j].y : s == 2 ? bv[hb][j].z : bv[hb][j].w;
-                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(ae, be, acc[i][j], 0, 0, 0);
+                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(be, ae, acc[i][j], 0, 0, 0);
                 }
             }
         }
@@ -412,7 +430,7 @@ __global__ __launch_bounds__(DN_THREADS, (BM == 128 ? 3 : 2)) void conv_mfma_ker
         return;
     }
 
-    conv_epilogue<TM, TN>(a, acc, rows, m0, n0, wm0, wn0, li, kh);
+    conv_epilogue<TM, TN>(a, acc, m0, n0, wm0, wn0, li, kh);
 }
 
 /* Sums the K-slices of the tail tiles in slice order (deterministic) and applies the epilogue.
@@ -430,7 +448,8 @@ __global__ __launch_bounds__(DN_THREADS) void conv_reduce_kernel(mfma_args a)
     const int lin = a.whole_tiles + t;
     const int m0 = (lin % a.tiles_m) * BM;
     const long n0 = (long)(lin / a.tiles_m) * BN;
-    /* e = ((wave*TM*TN + i*TN + j)*16 + r)*64 + lane */
+    /* e = ((wave*TM*TN + i*TN + j)*16 + r)*64 + lane; four consecutive e are four consecutive
+     * lanes = four consecutive FILTERS at one pixel (see conv_epilogue for the register map) */
     const int lane = e & 63;
     int q = e >> 6;
     const int r = q & 15;
@@ -439,9 +458,8 @@ __global__ __launch_bounds__(DN_THREADS) void conv_reduce_kernel(mfma_args a)
     q /= TN;
     const int i = q % TM;
     const int wave = q / TM;
-    const int ml = (wave / WAVES_N) * WM + i * 32 + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
-    const int m = m0 + ml;
-    const long n = n0 + (wave % WAVES_N) * WN + j * 32 + (lane & 31);
+    const int mbase = m0 + (wave / WAVES_N) * WM + i * 32 + (lane & 31);
+    const long n = n0 + (wave % WAVES_N) * WN + j * 32 + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
     float4 sum = make_float4(0.f, 0.f, 0.f, 0.f);
     const float4 *ws = (const float4 *)(a.partial + (long)t * a.split * (BM * BN) + e);
     for (int sl = 0; sl < a.split; ++sl) {
@@ -451,22 +469,17 @@ __global__ __launch_bounds__(DN_THREADS) void conv_reduce_kernel(mfma_args a)
         sum.z += v.z;
         sum.w += v.w;
     }
-    if (m >= a.M) return;
-    const dn_bn_row row = dn_bn_make(a.bn, a.biases[m], a.bn ? a.scales[m] : 1.f, a.bn ? a.mean[m] : 0.f,
-                                     a.bn ? a.var[m] : 1.f);
+    if (n >= a.Ntotal) return;
+    const int b = (int)(n / a.P);
+    const int p = (int)(n - (long)b * a.P);
     const float vals[4] = {sum.x, sum.y, sum.z, sum.w};
 #pragma unroll
     for (int c = 0; c < 4; ++c) {
-        const long nc = n + c;
-        if (nc >= a.Ntotal) break;
-        const int b = (int)(nc / a.P);
-        const int p = (int)(nc - (long)b * a.P);
-        const float y = dn_bn_apply(vals[c], row, a.bn);
-        float z;
-        if (a.act == DN_LEAKY) z = (y > 0) ? y : (float)(.1 * (double)y);
-        else if (a.act == DN_LINEAR) z = y;
-        else z = activate_rare(y, a.act);
-        a.out[((long)b * a.M + m) * a.P + p] = z;
+        const int m = mbase + c;
+        if (m >= a.M) break;
+        const dn_bn_row row = dn_bn_make(a.bn, a.biases[m], a.bn ? a.scales[m] : 1.f, a.bn ? a.mean[m] : 0.f,
+                                         a.bn ? a.var[m] : 1.f);
+        a.out[((long)b * a.M + m) * a.P + p] = conv_tail_one(vals[c], row, a.bn, a.act);
     }
 }
 
