@@ -39,6 +39,7 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 #include <stdio.h>
+#include <stdlib.h>
 
 #include "device_math.h"
 #include "hip.h"
@@ -64,7 +65,8 @@ struct mfma_args {
     int P, OW;          /* out_h*out_w, out_w */
     long Ntotal;        /* batch * P */
     int stride, pad, size;
-    int bn, act;
+    int bn;
+    double slope;       /* activation as conv_inline_activation encodes it */
     int tiles_m, tiles_n, per_xcd;
     unsigned in_records; /* bytes the gather may address: input + bias row */
     unsigned wp_records; /* bytes of the packed weights */
@@ -73,6 +75,15 @@ struct mfma_args {
      * whole_tiles + j / split and leaves raw accumulators in `partial` for the reduce kernel */
     int whole_tiles, split;
     float *partial;
+    /* fused residual add (null = none): sum[i] = act2(s1*out[i] + s2*add[i]) over the same
+     * geometry as out, the arithmetic of src/blas.c:36 followed by src/shortcut_layer.c:64 */
+    const float *add;
+    float *sum;
+    float s1, s2;
+    double sum_slope;
+#ifdef DN_TRACE
+    unsigned long long *trace;
+#endif
 };
 
 /* k -> (channel, ky, kx) for a size x size kernel in the reference's im2col row order. */
@@ -97,72 +108,133 @@ __device__ __forceinline__ void split_k(int k, int size, int &ci, int &ky, int &
     }
 }
 
-/* Activations other than leaky / linear: out of line, so that the 64-element epilogue does not
- * carry 64 inlined copies of the double-precision exp() expansions (the kernel grew to 45k
- * instructions and spilled that way). */
-__device__ __attribute__((noinline)) float activate_rare(float x, int a) { return dn_activate(x, a); }
-
 typedef float float4u __attribute__((ext_vector_type(4), aligned(4)));
 
-__device__ __forceinline__ float conv_tail_one(float acc, const dn_bn_row &row, int bn, int act)
+/* The three activations the epilogue applies itself share one branch-free form,
+ *     f(y) = y > 0 ? y : (float)(slope * (double)y),
+ * with slope .1 for leaky (src/activations.h:39), 1 for linear and 0 for relu: for relu the
+ * reference's x*(x>0) (src/activations.h:35) and 0.*x agree on every input including -0, the
+ * infinities and NaN.  Any other activation runs as a second pass over the output. */
+__host__ __device__ inline bool conv_inline_activation(int act, double *slope)
 {
-    const float y = dn_bn_apply(acc, row, bn);
-    if (act == DN_LEAKY) return (y > 0) ? y : (float)(.1 * (double)y);
-    if (act == DN_LINEAR) return y;
-    return activate_rare(y, act);
+    if (act == DN_LEAKY) *slope = .1;
+    else if (act == DN_LINEAR) *slope = 1.;
+    else if (act == DN_RELU) *slope = 0.;
+    else return false;
+    return true;
 }
 
-/* Stores four consecutive output columns n..n+3 of filter row m (one 16-byte store when they
- * lie in one image, element by element across an image boundary or the end of N). */
-__device__ __forceinline__ void conv_store4(const mfma_args &a, int m, long n, const float v[4],
-                                            const dn_bn_row &row)
+__device__ __forceinline__ float conv_slope(float y, double slope)
 {
-    if (n >= a.Ntotal) return;
-    const int b = (int)(n / a.P);
-    const int p = (int)(n - (long)b * a.P);
-    float *dst = a.out + ((long)b * a.M + m) * a.P + p;
-    if (p + 3 < a.P) { /* implies n + 3 < Ntotal */
-        float4u o;
-        o.x = conv_tail_one(v[0], row, a.bn, a.act);
-        o.y = conv_tail_one(v[1], row, a.bn, a.act);
-        o.z = conv_tail_one(v[2], row, a.bn, a.act);
-        o.w = conv_tail_one(v[3], row, a.bn, a.act);
-        *(float4u *)dst = o;
-        return;
-    }
-#pragma unroll
-    for (int c = 0; c < 4; ++c) {
-        const long nc = n + c;
-        if (nc >= a.Ntotal) break;
-        const int bc = (int)(nc / a.P);
-        const int pc = (int)(nc - (long)bc * a.P);
-        a.out[((long)bc * a.M + m) * a.P + pc] = conv_tail_one(v[c], row, a.bn, a.act);
-    }
+    return (y > 0) ? y : (float)(slope * (double)y);
+}
+
+/* batch-norm -> scale -> bias -> activation of one accumulator; without batch-norm the row holds
+ * the neutral constants (mean 0, reciprocal 1, scale 1), which change no bit */
+__device__ __forceinline__ float conv_tail_one(float acc, const dn_bn_row &row, double slope)
+{
+    return conv_slope(dn_bn_apply(acc, row, 1), slope);
+}
+
+__device__ __forceinline__ float conv_residual_one(const mfma_args &a, float y, float r)
+{
+    return conv_slope(__fadd_rn(__fmul_rn(a.s1, y), __fmul_rn(a.s2, r)), a.sum_slope);
+}
+
+__device__ __forceinline__ dn_bn_row conv_row(const mfma_args &a, int m)
+{
+    return dn_bn_make(a.bn, a.biases[m], a.bn ? a.scales[m] : 1.f, a.bn ? a.mean[m] : 0.f,
+                      a.bn ? a.var[m] : 1.f);
 }
 
 /* Batch-norm / bias / activation and the store.  The MFMAs are issued with the pixel tile as
  * the row operand and the filter tile as the column operand, so accumulator register r of lane l
  * holds filter (l % 32) and pixel 8*(r/4) + 4*(l/32) + r%4 of its 32x32 block: a lane owns one
- * filter (its batch-norm constants are loaded once) and four consecutive pixels per register
- * quad, which go out as one 16-byte store. */
+ * filter per 32-row block (its batch-norm constants are loaded once) and, per register quad,
+ * four consecutive pixels, which go out as one 16-byte store.
+ * The lane's quads sit 8 columns apart, so the (image, pixel) split of the column index is
+ * computed once and then stepped: no division inside the loop. */
 template <int TM, int TN>
 __device__ __forceinline__ void conv_epilogue(const mfma_args &a, f32x16 (&acc)[TM][TN], int m0, long n0,
                                               int wm0, int wn0, int li, int kh)
 {
+    dn_bn_row row[TM];
+    long moff[TM];
+    bool mok[TM];
 #pragma unroll
     for (int i = 0; i < TM; ++i) {
         const int m = m0 + wm0 + i * 32 + li;
-        if (m >= a.M) continue;
-        const dn_bn_row row = dn_bn_make(a.bn, a.biases[m], a.bn ? a.scales[m] : 1.f, a.bn ? a.mean[m] : 0.f,
-                                         a.bn ? a.var[m] : 1.f);
+        mok[i] = m < a.M;
+        const int mc = mok[i] ? m : a.M - 1;
+        row[i] = conv_row(a, mc);
+        moff[i] = (long)mc * a.P;
+    }
+    const int P = a.P;
+    int n = (int)n0 + wn0 + 4 * kh;                 /* Ntotal < 2^31 on this path */
+    const int Nt = (int)a.Ntotal;
+    int p;
+    long off;                                        /* image*M*P + pixel */
+    {
+        const int b = (int)((unsigned)n / (unsigned)P);
+        p = n - b * P;
+        off = (long)b * a.M * P + p;
+    }
+    const long wrap = (long)(a.M - 1) * P;           /* what `off` gains when the pixel index wraps */
 #pragma unroll
-        for (int j = 0; j < TN; ++j) {
+    for (int j = 0; j < TN; ++j) {
 #pragma unroll
-            for (int rg = 0; rg < 4; ++rg) {
-                const long n = n0 + wn0 + j * 32 + 8 * rg + 4 * kh;
-                const float v[4] = {acc[i][j][rg * 4 + 0], acc[i][j][rg * 4 + 1], acc[i][j][rg * 4 + 2],
-                                    acc[i][j][rg * 4 + 3]};
-                conv_store4(a, m, n, v, row);
+        for (int rg = 0; rg < 4; ++rg) {
+            if (n < Nt) {
+                if (p + 3 < P) { /* the quad lies in one image (and n + 3 < Ntotal) */
+#pragma unroll
+                    for (int i = 0; i < TM; ++i) {
+                        if (!mok[i]) continue;
+                        float4u o;
+                        o.x = conv_tail_one(acc[i][j][rg * 4 + 0], row[i], a.slope);
+                        o.y = conv_tail_one(acc[i][j][rg * 4 + 1], row[i], a.slope);
+                        o.z = conv_tail_one(acc[i][j][rg * 4 + 2], row[i], a.slope);
+                        o.w = conv_tail_one(acc[i][j][rg * 4 + 3], row[i], a.slope);
+                        const long o_off = off + moff[i];
+                        *(float4u *)(a.out + o_off) = o;
+                        if (a.sum) {
+                            const float4u r = *(const float4u *)(a.add + o_off);
+                            float4u t;
+                            t.x = conv_residual_one(a, o.x, r.x);
+                            t.y = conv_residual_one(a, o.y, r.y);
+                            t.z = conv_residual_one(a, o.z, r.z);
+                            t.w = conv_residual_one(a, o.w, r.w);
+                            *(float4u *)(a.sum + o_off) = t;
+                        }
+                    }
+                } else {         /* image boundary or end of N inside the quad: element by element */
+                    int pc = p;
+                    long offc = off;
+#pragma unroll
+                    for (int c = 0; c < 4; ++c) {
+                        if (n + c < Nt) {
+                            while (pc >= P) {
+                                pc -= P;
+                                offc += wrap;
+                            }
+#pragma unroll
+                            for (int i = 0; i < TM; ++i) {
+                                if (!mok[i]) continue;
+                                const float y = conv_tail_one(acc[i][j][rg * 4 + c], row[i], a.slope);
+                                a.out[offc + moff[i]] = y;
+                                if (a.sum) a.sum[offc + moff[i]] = conv_residual_one(a, y, a.add[offc + moff[i]]);
+                            }
+                        }
+                        ++pc;
+                        ++offc;
+                    }
+                }
+            }
+            n += 8;
+            p += 8;
+            off += 8;
+            while (p >= P) {
+                p -= P;
+                off += wrap;
             }
         }
     }
@@ -186,6 +258,9 @@ __global__ __launch_bounds__(DN_THREADS, (BM == 128 ? 3 : 2)) void conv_mfma_ker
 
     /* XCD-aware tile order: workgroup id -> (xcd, slot) -> linear tile with tile_m fastest. */
     const int bid = blockIdx.x;
+#ifdef DN_TRACE
+    unsigned long long tr0 = __builtin_amdgcn_s_memrealtime(), tr1 = 0, tr2 = 0;
+#endif
     int lin, kc_begin = 0, kc_end = a.KCH, slice_id = -1;
     if (bid < 8 * a.per_xcd) {
         lin = (bid & 7) * a.per_xcd + (bid >> 3);
@@ -352,6 +427,9 @@ __global__ __launch_bounds__(DN_THREADS, (BM == 128 ? 3 : 2)) void conv_mfma_ker
     load_chunk(kc_begin, 0);
     __builtin_amdgcn_s_waitcnt(0);
     __syncthreads();
+#ifdef DN_TRACE
+    tr1 = __builtin_amdgcn_s_memrealtime();
+#endif
 
     float4 av[2][TM], bv[2][TN]; /* MFMA operands of the current chunk: [k half][32-row block] */
 
@@ -417,6 +495,11 @@ __global__ __launch_bounds__(DN_THREADS, (BM == 128 ? 3 : 2)) void conv_mfma_ker
         last(0);
     }
 
+#ifdef DN_TRACE
+    __builtin_amdgcn_sched_barrier(0);
+    tr2 = __builtin_amdgcn_s_memrealtime();
+    __builtin_amdgcn_sched_barrier(0);
+#endif
     if (slice_id >= 0) {
         /* K-slice: park the raw accumulators, lane-major so every store is a full 256-byte row */
         float *ws = a.partial + (long)slice_id * (BM * BN);
@@ -427,10 +510,26 @@ __global__ __launch_bounds__(DN_THREADS, (BM == 128 ? 3 : 2)) void conv_mfma_ker
 #pragma unroll
                 for (int r = 0; r < 16; ++r)
                     ws[((wave * TM * TN + i * TN + j) * 16 + r) * 64 + lane] = acc[i][j][r];
-        return;
+    } else {
+        conv_epilogue<TM, TN>(a, acc, m0, n0, wm0, wn0, li, kh);
     }
-
-    conv_epilogue<TM, TN>(a, acc, m0, n0, wm0, wn0, li, kh);
+#ifdef DN_TRACE
+    if (a.trace) {
+        __builtin_amdgcn_s_waitcnt(0);
+        __syncthreads();
+        if (tid == 0) {
+            const unsigned hw = __builtin_amdgcn_s_getreg(4 | (0 << 6) | (15 << 11));
+            const unsigned xcc = __builtin_amdgcn_s_getreg(20 | (0 << 6) | (3 << 11));
+            unsigned long long *t = a.trace + (long)bid * 6;
+            t[0] = ((unsigned long long)xcc << 32) | hw;
+            t[1] = tr0;
+            t[2] = tr1;
+            t[3] = tr2;
+            t[4] = __builtin_amdgcn_s_memrealtime();
+            t[5] = (unsigned long long)(kc_end - kc_begin) | ((unsigned long long)(slice_id >= 0) << 32);
+        }
+    }
+#endif
 }
 
 /* Sums the K-slices of the tail tiles in slice order (deterministic) and applies the epilogue.
@@ -470,16 +569,18 @@ __global__ __launch_bounds__(DN_THREADS) void conv_reduce_kernel(mfma_args a)
         sum.w += v.w;
     }
     if (n >= a.Ntotal) return;
-    const int b = (int)(n / a.P);
-    const int p = (int)(n - (long)b * a.P);
+    const int b = (int)((unsigned)n / (unsigned)a.P);
+    const int p = (int)n - b * a.P;
     const float vals[4] = {sum.x, sum.y, sum.z, sum.w};
 #pragma unroll
     for (int c = 0; c < 4; ++c) {
         const int m = mbase + c;
         if (m >= a.M) break;
-        const dn_bn_row row = dn_bn_make(a.bn, a.biases[m], a.bn ? a.scales[m] : 1.f, a.bn ? a.mean[m] : 0.f,
-                                         a.bn ? a.var[m] : 1.f);
-        a.out[((long)b * a.M + m) * a.P + p] = conv_tail_one(vals[c], row, a.bn, a.act);
+        const dn_bn_row row = conv_row(a, m);
+        const long off = ((long)b * a.M + m) * a.P + p;
+        const float y = conv_tail_one(vals[c], row, a.slope);
+        a.out[off] = y;
+        if (a.sum) a.sum[off] = conv_residual_one(a, y, a.add[off]);
     }
 }
 
@@ -620,6 +721,13 @@ static void launch_tile(const mfma_args &a0, int mode)
         a.partial = g_partial;
     }
     const dim3 grid((unsigned)(a.per_xcd * 8 + tail * split));
+#ifdef DN_TRACE
+    a.trace = 0;
+    if (getenv("DN_TRACE")) {
+        hip_check_error(hipMalloc((void **)&a.trace, (size_t)grid.x * 48));
+        hip_check_error(hipMemset(a.trace, 0, (size_t)grid.x * 48));
+    }
+#endif
     if (BM > 128 && mode != 11 && mode != 13) dn_fatal("conv dispatch: the 256-row tile is only built for the tap-blocked modes");
     switch (mode) {
     case 11: hipLaunchKernelGGL((conv_mfma_kernel<BM, BN, WM, WN, 11>), grid, dim3(DN_THREADS), 0, dn_stream(), a); break;
@@ -635,6 +743,20 @@ static void launch_tile(const mfma_args &a0, int mode)
         }
         break;
     }
+#ifdef DN_TRACE
+    if (a.trace) {
+        static int seq = 0;
+        unsigned long long *h = (unsigned long long *)malloc((size_t)grid.x * 48);
+        hip_check_error(hipDeviceSynchronize());
+        hip_check_error(hipMemcpy(h, a.trace, (size_t)grid.x * 48, hipMemcpyDeviceToHost));
+        char name[256];
+        snprintf(name, sizeof name, "%s/trace_%03d.bin", getenv("DN_TRACE"), seq++);
+        FILE *f = fopen(name, "wb");
+        if (f) { fwrite(h, 48, grid.x, f); fclose(f); }
+        free(h);
+        hip_check_error(hipFree(a.trace));
+    }
+#endif
     if (tail > 0)
         hipLaunchKernelGGL((conv_reduce_kernel<BM, BN, WM, WN>), dim3((unsigned)(tail * (BM * BN / 4 / DN_THREADS))),
                            dim3(DN_THREADS), 0, dn_stream(), a);
@@ -658,12 +780,15 @@ static int conv_mode(int c, int groups, int size, int stride, int pad, long in_b
     return size == 1 ? 1 : size == 3 ? 3 : 0;
 }
 
-extern "C" void forward_convolutional_gpu(const float *input, const float *weights, const float *packed,
-                                          const float *biases, const float *scales,
-                                          const float *rolling_mean, const float *rolling_variance,
-                                          float *output, int batch, int c, int h, int w, int n,
-                                          int groups, int size, int stride, int pad,
-                                          int batch_normalize, int activation)
+extern "C" void forward_shortcut_gpu(const float *, const float *, float *, int, int, int, int, int, int, int,
+                                     float, float, int);
+extern "C" void dn_activate_array(float *x, long n, int activation);
+
+static void conv_forward(const float *input, const float *weights, const float *packed, const float *biases,
+                         const float *scales, const float *rolling_mean, const float *rolling_variance,
+                         float *output, int batch, int c, int h, int w, int n, int groups, int size, int stride,
+                         int pad, int batch_normalize, int activation, const float *add, float *sum, float s1,
+                         float s2, int sum_act)
 {
     if (batch <= 0 || c <= 0 || h <= 0 || w <= 0 || n <= 0 || groups <= 0 || size <= 0 || stride <= 0 || pad < 0)
         dn_fatal("forward_convolutional_gpu: bad geometry");
@@ -681,10 +806,22 @@ extern "C" void forward_convolutional_gpu(const float *input, const float *weigh
         dn_fatal("forward_convolutional_gpu: tensor too large");
 
     const long K = (long)(c / groups) * size * size;
-    const int mode = conv_mode(c, groups, size, stride, pad, (long)batch * c * h * w * 4);
+    int mode = conv_mode(c, groups, size, stride, pad, (long)batch * c * h * w * 4);
+    if ((long)batch * oh * ow >= (1L << 31) - 512) mode = -1; /* the MFMA kernels index columns in 32 bits */
     if (mode < 0) {
         conv_direct_forward(input, weights, biases, scales, rolling_mean, rolling_variance, output, batch, c,
                             h, w, n, groups, size, stride, pad, batch_normalize, activation);
+        if (sum) forward_shortcut_gpu(output, add, sum, batch, ow, oh, n, ow, oh, n, s1, s2, sum_act);
+        return;
+    }
+    double slope = 1., sum_slope = 1.;
+    if (!conv_inline_activation(activation, &slope) || (sum && !conv_inline_activation(sum_act, &sum_slope))) {
+        /* an activation the epilogue does not carry: linear convolution, then the reference's own
+         * sequence of passes (activate_array, src/convolutional_layer.c:478; shortcut) */
+        conv_forward(input, weights, packed, biases, scales, rolling_mean, rolling_variance, output, batch, c, h,
+                     w, n, groups, size, stride, pad, batch_normalize, DN_LINEAR, 0, 0, 0.f, 0.f, DN_LINEAR);
+        dn_activate_array(output, (long)batch * n * oh * ow, activation);
+        if (sum) forward_shortcut_gpu(output, add, sum, batch, ow, oh, n, ow, oh, n, s1, s2, sum_act);
         return;
     }
 
@@ -721,11 +858,16 @@ extern "C" void forward_convolutional_gpu(const float *input, const float *weigh
     a.pad = pad;
     a.size = size;
     a.bn = batch_normalize ? 1 : 0;
-    a.act = activation;
+    a.slope = slope;
     a.tiles_m = a.tiles_n = a.per_xcd = 0;
     a.whole_tiles = 0;
     a.split = 1;
     a.partial = 0;
+    a.add = add;
+    a.sum = sum;
+    a.s1 = s1;
+    a.s2 = s2;
+    a.sum_slope = sum_slope;
     a.in_records = (unsigned)((long)batch * c * h * w * 4 + (long)(w + 1) * 4);
     a.wp_records = (unsigned)(conv_packed_floats(n, c, groups, size) * 4);
     if (n <= 32)
@@ -735,4 +877,33 @@ extern "C" void forward_convolutional_gpu(const float *input, const float *weigh
     else
         launch_tile<128, 128, 64, 64>(a, mode);
     dn_check_launch("forward_convolutional_gpu");
+}
+
+extern "C" void forward_convolutional_gpu(const float *input, const float *weights, const float *packed,
+                                          const float *biases, const float *scales,
+                                          const float *rolling_mean, const float *rolling_variance,
+                                          float *output, int batch, int c, int h, int w, int n,
+                                          int groups, int size, int stride, int pad,
+                                          int batch_normalize, int activation)
+{
+    conv_forward(input, weights, packed, biases, scales, rolling_mean, rolling_variance, output, batch, c, h, w,
+                 n, groups, size, stride, pad, batch_normalize, activation, 0, 0, 0.f, 0.f, DN_LINEAR);
+}
+
+extern "C" void forward_convolutional_shortcut_gpu(const float *input, const float *weights, const float *packed,
+                                                   const float *biases, const float *scales,
+                                                   const float *rolling_mean, const float *rolling_variance,
+                                                   float *output, int batch, int c, int h, int w, int n,
+                                                   int groups, int size, int stride, int pad,
+                                                   int batch_normalize, int activation, const float *add,
+                                                   float *sum_output, float alpha, float beta,
+                                                   int shortcut_activation)
+{
+    if (!add || !sum_output) dn_fatal("forward_convolutional_shortcut_gpu: null pointer");
+    if (sum_output == output) dn_fatal("forward_convolutional_shortcut_gpu: sum_output must not alias output");
+    if (shortcut_activation < 0 || shortcut_activation > DN_SELU)
+        dn_fatal("forward_convolutional_shortcut_gpu: unknown activation");
+    conv_forward(input, weights, packed, biases, scales, rolling_mean, rolling_variance, output, batch, c, h, w,
+                 n, groups, size, stride, pad, batch_normalize, activation, add, sum_output, alpha, beta,
+                 shortcut_activation);
 }

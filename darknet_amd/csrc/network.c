@@ -57,6 +57,32 @@ void set_batch_network(network *net, int b)
     for (i = 0; i < net->n; ++i) net->layers[i].batch = b;
 }
 
+static int g_fuse_shortcut = 1;
+
+/* 1 (default): a convolution followed directly by a same-geometry shortcut runs as one kernel
+ * launch sequence; 0: every layer runs on its own.  Both layers' outputs are written either way. */
+void network_set_fusion(int on) { g_fuse_shortcut = on ? 1 : 0; }
+
+/* Runs layers i and i+1 together when they are a convolution and the residual add of a
+ * darknet53 block (src/shortcut_layer.c:77-83 with equal geometries).  Returns 1 if it did. */
+static int forward_conv_shortcut_pair(network net, int i)
+{
+    layer l, s;
+    if (!g_fuse_shortcut || i + 1 >= net.n) return 0;
+    l = net.layers[i];
+    s = net.layers[i + 1];
+    if (l.type != CONVOLUTIONAL || l.xnor || s.type != SHORTCUT) return 0;
+    if (s.index < 0 || s.index >= i) return 0; /* the residual must come from an earlier layer */
+    if (s.w != s.out_w || s.h != s.out_h || s.c != s.out_c) return 0;
+    if (s.out_w != l.out_w || s.out_h != l.out_h || s.out_c != l.out_c || s.batch != l.batch) return 0;
+    forward_convolutional_shortcut_gpu(net.input_gpu, l.weights_gpu, l.weights_packed_gpu, l.biases_gpu,
+                                       l.scales_gpu, l.rolling_mean_gpu, l.rolling_variance_gpu, l.output_gpu,
+                                       l.batch, l.c, l.h, l.w, l.n, l.groups, l.size, l.stride, l.pad,
+                                       l.batch_normalize, (int)l.activation, net.layers[s.index].output_gpu,
+                                       s.output_gpu, s.alpha, s.beta, (int)s.activation);
+    return 1;
+}
+
 /* The layer loop of src/network.c:773-785 without the copies around it. */
 void forward_network_device(network *netp)
 {
@@ -67,13 +93,18 @@ void forward_network_device(network *netp)
         layer l = net.layers[i];
         net.index = i;
         if (!l.forward_gpu) dn_fatal("layer without a GPU forward");
-        l.forward_gpu(l, net);
+        if (forward_conv_shortcut_pair(net, i)) {
+            ++i;
+            l = net.layers[i];
+        } else {
+            l.forward_gpu(l, net);
+        }
         net.input_gpu = l.output_gpu;
     }
 }
 
 /* The same loop with a HIP event between consecutive layers; layer_ms[i] receives layer i's
- * time on the device.  Returns the total (first event to last) in milliseconds.  Events are
+ * time on the device (a shortcut that ran inside the convolution before it reports 0).  Returns the total (first event to last) in milliseconds.  Events are
  * created once per network size and reused. */
 float forward_network_profiled(network *netp, float *layer_ms)
 {
@@ -93,7 +124,13 @@ float forward_network_profiled(network *netp, float *layer_ms)
     for (i = 0; i < net.n; ++i) {
         layer l = net.layers[i];
         net.index = i;
-        l.forward_gpu(l, net);
+        if (forward_conv_shortcut_pair(net, i)) {
+            hip_event_record(ev[i + 1]);
+            ++i;
+            l = net.layers[i];
+        } else {
+            l.forward_gpu(l, net);
+        }
         net.input_gpu = l.output_gpu;
         hip_event_record(ev[i + 1]);
     }

@@ -103,19 +103,23 @@ __global__ void activate4_kernel(float4 *x, long n4, int a)
     }
 }
 
-extern "C" void activate_array_gpu(float *x, int n, int activation)
+/* activate_array_gpu for tensors of any length (internal: the convolution uses it for the
+ * activations its epilogue does not carry) */
+extern "C" void dn_activate_array(float *x, long n, int activation)
 {
     if (n <= 0 || activation == DN_LINEAR) return;
     if (activation < 0 || activation > DN_SELU) dn_fatal("activate_array_gpu: unknown activation");
     if (aligned16(x) && (n & 3) == 0) {
         hipLaunchKernelGGL(activate4_kernel, dim3(dn_blocks(n / 4)), dim3(DN_BLOCK), 0, dn_stream(),
-                           (float4 *)x, (long)n / 4, activation);
+                           (float4 *)x, n / 4, activation);
     } else {
-        hipLaunchKernelGGL(activate_kernel, dim3(dn_blocks(n)), dim3(DN_BLOCK), 0, dn_stream(), x,
-                           (long)n, activation);
+        hipLaunchKernelGGL(activate_kernel, dim3(dn_blocks(n)), dim3(DN_BLOCK), 0, dn_stream(), x, n,
+                           activation);
     }
     dn_check_launch("activate_array_gpu");
 }
+
+extern "C" void activate_array_gpu(float *x, int n, int activation) { dn_activate_array(x, (long)n, activation); }
 
 /* ---- batch-norm pieces as separate passes (the fused convolution does not use them; they are
  * the reference-named helpers for callers that still run the chain step by step) ----------- */

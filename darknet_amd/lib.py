@@ -45,6 +45,7 @@ SIGNATURES = {
     "binarize_gpu": (None, [V, i, V]), "binarize_weights_gpu": (None, [V, i, i, V]),
     # ---- darknet_hip.h: fused layer forwards
     "forward_convolutional_gpu": (None, [V] * 8 + [i] * 11),
+    "forward_convolutional_shortcut_gpu": (None, [V] * 8 + [i] * 11 + [V, V, f, f, i]),
     "conv_packed_floats": (z, [i, i, i, i]), "conv_pack_weights_gpu": (None, [V, V, i, i, i, i]),
     "conv_set_algo": (None, [i]),
     "xnor_weight_words": (z, [i, i, i]), "xnor_input_words": (z, [i, i, i, i]),
@@ -67,6 +68,7 @@ SIGNATURES = {
     "set_batch_network": (None, [V, i]), "network_output": (F, [V]),
     "pull_network_output": (None, [V]), "network_width": (i, [V]), "network_height": (i, [V]),
     "forward_network_device": (None, [V]), "forward_network_profiled": (f, [V, F]),
+    "network_set_fusion": (None, [i]),
     "conv_kernel_name": (C.c_char_p, [i, i, i, i]), "layer_output_host": (F, [V, i]),
     "layer_indexes_host": (I, [V, i]), "network_set_verbose": (None, [i]),
     "network_set_conv": (None, [V, i, F, F, F, F, F]),

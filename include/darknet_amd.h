@@ -210,6 +210,11 @@ void forward_network_device(network *net);
 /* forward_network_device with a HIP event after every layer: fills layer_ms[net->n] (may be
  * NULL) and returns the whole pass in milliseconds; synchronises before returning. */
 float forward_network_profiled(network *net, float *layer_ms);
+/* 1 (default): forward_network_device runs a convolution and the same-geometry shortcut right
+ * after it as one pass (forward_convolutional_shortcut_gpu); 0: layer by layer as
+ * src/network.c:773-785 does.  Every layer's output buffer is written in both modes and holds
+ * the same bits. */
+void network_set_fusion(int on);
 float *layer_output_host(network *net, int i);
 int *layer_indexes_host(network *net, int i);
 void network_set_verbose(int on);

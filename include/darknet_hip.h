@@ -117,6 +117,24 @@ void forward_convolutional_gpu(const float *input, const float *weights, const f
                                int groups, int size, int stride, int pad, int batch_normalize,
                                int activation);
 
+/* Convolution layer followed by a same-geometry shortcut layer, in one pass: `output` receives
+ * what forward_convolutional_gpu writes and `sum_output` what the shortcut layer after it would:
+ *   sum_output[i] = shortcut_activation(alpha*output[i] + beta*add[i])
+ * with add and sum_output of output's shape [batch][n][out_h][out_w].  Replaces the pair
+ * forward_convolutional_layer_gpu (src/convolutional_kernels.cu:73-135) + forward_shortcut_layer_gpu
+ * (src/shortcut_layer.c:77-83: copy_gpu, shortcut_gpu, activate_array_gpu) when the shortcut's
+ * `from` layer has the convolution's output geometry, as in every darknet53 residual block; the
+ * results equal those of the two separate calls bit for bit.  The residual is read and the sum
+ * written in the convolution's epilogue, which saves the shortcut's own pass over memory.
+ * sum_output must not alias output; add may be any other buffer. */
+void forward_convolutional_shortcut_gpu(const float *input, const float *weights, const float *packed,
+                                        const float *biases, const float *scales,
+                                        const float *rolling_mean, const float *rolling_variance,
+                                        float *output, int batch, int c, int h, int w, int n,
+                                        int groups, int size, int stride, int pad, int batch_normalize,
+                                        int activation, const float *add, float *sum_output, float alpha,
+                                        float beta, int shortcut_activation);
+
 /* Weight repack for the MFMA kernel (the natural hook is push_convolutional_layer,
  * src/convolutional_kernels.cu:286-297).  conv_packed_floats() == 0 means the layer does not
  * use a packed copy (grouped convolutions). */
@@ -128,7 +146,8 @@ void conv_pack_weights_gpu(const float *weights, float *packed, int n, int c, in
 const char *conv_kernel_name(int n, int c, int groups, int size);
 
 /* Selects the convolution kernel: 0 = automatic (default), 1 = always the plain direct
- * kernel.  The direct kernel is the in-library cross-check of the MFMA kernel. */
+ * kernel, 3 = MFMA kernel without the K-split of the last partial round of tiles.  The direct
+ * kernel is the in-library cross-check of the MFMA kernel. */
 void conv_set_algo(int algo);
 
 /* XNOR convolution (xnor=1 layers): sign(x>0) inputs, sign(w>0)*mean|w| weights, zero padding,

@@ -139,3 +139,45 @@ def test_conv_linearity_at_full_size(dn):
     y2 = run_conv(dn, x2, wt, zero, None, None, None, **kw)
     y12 = run_conv(dn, x1 + x2, wt, zero, None, None, None, **kw)
     assert norm_err(y12, y + y2) <= 1e-5
+
+
+FUSED = [  # b, c, h, w, n, size, stride, pad, groups, act, alpha, beta, shortcut act
+    (2, 64, 26, 26, 128, 3, 1, 1, 1, "leaky", 1.0, 1.0, "linear"),     # darknet53 residual block
+    (3, 128, 13, 13, 255, 1, 1, 0, 1, "linear", 0.5, -1.25, "leaky"),  # ragged M, scaled, activated
+    (1, 256, 13, 13, 512, 3, 1, 1, 1, "leaky", 1.0, 1.0, "linear"),    # batch 1: every tile K-split
+    (5, 16, 7, 9, 130, 3, 1, 1, 1, "leaky", 1.0, 2.0, "logistic"),     # tile columns cross images
+    (2, 3, 21, 23, 32, 3, 1, 1, 1, "leaky", 1.0, 1.0, "linear"),       # reference-order kernel, BM = 32
+    (2, 64, 14, 14, 64, 3, 1, 1, 32, "leaky", 1.0, 1.0, "linear"),     # grouped -> direct kernel + add
+]
+
+
+@pytest.mark.parametrize("b,c,h,w,n,size,stride,pad,groups,act,alpha,beta,sact", FUSED)
+def test_conv_shortcut_fused_equals_separate_calls(dn, b, c, h, w, n, size, stride, pad, groups, act, alpha,
+                                                    beta, sact):
+    """forward_convolutional_shortcut_gpu == forward_convolutional_gpu then forward_shortcut_gpu, bit for
+    bit, on both outputs (the shortcut itself is checked against the CPU in test_gpu_kernels)."""
+    x = synth.uniform(11, b * c * h * w).reshape(b, c, h, w)
+    wt = synth.conv_weights(12, n, c // groups, size)
+    bias, sc, mu, var = synth.bn_random(13, n)
+    oh = (h + 2 * pad - size) // stride + 1
+    ow = (w + 2 * pad - size) // stride + 1
+    total = b * n * oh * ow
+    res = synth.uniform(14, total)
+    dx, dw, db, ds, dm, dv, dres = D(x), D(wt), D(bias), D(sc), D(mu), D(var), D(res)
+    pk = None
+    pf = dn.conv_packed_floats(n, c, groups, size)
+    if pf:
+        pk = D(n=pf)
+        dn.conv_pack_weights_gpu(dw.ptr, pk.ptr, n, c, groups, size)
+    conv_args = (dx.ptr, dw.ptr, pk.ptr if pk else None, db.ptr, ds.ptr, dm.ptr, dv.ptr)
+    geom = (b, c, h, w, n, groups, size, stride, pad, 1, ACTIVATIONS.index(act))
+    out_a, sum_a = D(n=total), D(n=total)
+    dn.forward_convolutional_gpu(*conv_args, out_a.ptr, *geom)
+    dn.forward_shortcut_gpu(out_a.ptr, dres.ptr, sum_a.ptr, b, ow, oh, n, ow, oh, n, alpha, beta,
+                            ACTIVATIONS.index(sact))
+    out_b, sum_b = D(n=total), D(n=total)
+    dn.forward_convolutional_shortcut_gpu(*conv_args, out_b.ptr, *geom, dres.ptr, sum_b.ptr, alpha, beta,
+                                          ACTIVATIONS.index(sact))
+    assert np.array_equal(out_a.numpy((total,)), out_b.numpy((total,)))
+    assert np.array_equal(sum_a.numpy((total,)), sum_b.numpy((total,)))
+    assert np.abs(sum_b.numpy((total,))).max() > 0

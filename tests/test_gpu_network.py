@@ -171,3 +171,25 @@ def test_set_batch_network_shrinks(dn):
     one = net.predict(x[0])
     assert np.array_equal(one[0], full[0])
     net.free()
+
+
+def test_shortcut_fusion_changes_no_bit(dn):
+    """forward_network_device folds each residual add into the convolution before it; with the
+    fusion switched off every layer output must hold the same bits."""
+    net = api.Network(cfg_text=cfgs.yolov3(2, 160))
+    fill_params(net.set_conv, net.layers)
+    x = synth.uniform01(21, net.inputs * 2)
+    net.predict(x)
+    fused = [net.layer_output(i) for i in range(net.n)]
+    net.forward_profiled()      # the event-timed loop folds the same pairs
+    for i in range(net.n):
+        assert np.array_equal(net.layer_output(i), fused[i]), i
+    assert sum(L["type"] == "shortcut" for L in net.layers) == 23
+    net.L.network_set_fusion(0)
+    try:
+        net.predict(x)
+        for i in range(net.n):
+            assert np.array_equal(net.layer_output(i), fused[i]), i
+    finally:
+        net.L.network_set_fusion(1)
+    net.free()
