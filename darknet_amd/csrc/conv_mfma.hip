@@ -150,93 +150,82 @@ __device__ __forceinline__ dn_bn_row conv_row(const mfma_args &a, int m)
 /* Batch-norm / bias / activation and the store.  The MFMAs are issued with the pixel tile as
  * the row operand and the filter tile as the column operand, so accumulator register r of lane l
  * holds filter (l % 32) and pixel 8*(r/4) + 4*(l/32) + r%4 of its 32x32 block: a lane owns one
- * filter per 32-row block (its batch-norm constants are loaded once) and, per register quad,
- * four consecutive pixels, which go out as one 16-byte store.
- * The lane's quads sit 8 columns apart, so the (image, pixel) split of the column index is
- * computed once and then stepped: no division inside the loop. */
+ * filter per 32-row block, so its batch-norm constants are loaded once and the tail is applied
+ * in that layout.  Stored from there, every lane of a store would hit a different output row
+ * (64 separate 16-byte pieces per instruction, and the rate of such pieces, not bytes, is what
+ * the memory pipeline limits).  The finished values therefore take a turn through LDS first:
+ * each wave owns 8 KB of the (by now idle) operand buffers, holding 32 filters x 64 pixels with
+ * the 16-byte quads of a row XOR-swizzled by the row number (conflict-free both ways), and
+ * reads them back with 16 lanes per filter row: a store instruction then covers 4 rows of 256
+ * contiguous bytes, and the residual of a fused shortcut is read the same way. */
 template <int TM, int TN>
-__device__ __forceinline__ void conv_epilogue(const mfma_args &a, f32x16 (&acc)[TM][TN], int m0, long n0,
-                                              int wm0, int wn0, int li, int kh)
+__device__ __forceinline__ void conv_epilogue(const mfma_args &a, f32x16 (&acc)[TM][TN], float *E, int m0,
+                                              long n0, int wm0, int wn0, int lane)
 {
-    dn_bn_row row[TM];
-    long moff[TM];
-    bool mok[TM];
+    static_assert(TN == 2, "a wave's tile is 64 columns wide");
+    const int li = lane & 31, kh = lane >> 5;
+    const int q = lane & 15, fr = lane >> 4; /* after the turn: quad of 4 pixels, row within a group of 4 */
+    const int P = a.P;
+    const int Nt = (int)a.Ntotal;            /* Ntotal < 2^31 on this path */
+    const int n = (int)n0 + wn0 + 4 * q;
+    const int b = (int)((unsigned)n / (unsigned)P);
+    const int p = n - b * P;
+    const long off = (long)b * a.M * P + p;  /* image*M*P + pixel */
+    const bool quad_ok = p + 3 < P;          /* the quad lies in one image (then n + 3 < Ntotal too) */
+    const long wrap = (long)(a.M - 1) * P;   /* what the offset gains when the pixel index wraps */
 #pragma unroll
     for (int i = 0; i < TM; ++i) {
-        const int m = m0 + wm0 + i * 32 + li;
-        mok[i] = m < a.M;
-        const int mc = mok[i] ? m : a.M - 1;
-        row[i] = conv_row(a, mc);
-        moff[i] = (long)mc * a.P;
-    }
-    const int P = a.P;
-    int n = (int)n0 + wn0 + 4 * kh;                 /* Ntotal < 2^31 on this path */
-    const int Nt = (int)a.Ntotal;
-    int p;
-    long off;                                        /* image*M*P + pixel */
-    {
-        const int b = (int)((unsigned)n / (unsigned)P);
-        p = n - b * P;
-        off = (long)b * a.M * P + p;
-    }
-    const long wrap = (long)(a.M - 1) * P;           /* what `off` gains when the pixel index wraps */
+        const int mrow = m0 + wm0 + i * 32;
+        const dn_bn_row row = conv_row(a, mrow + li < a.M ? mrow + li : a.M - 1);
 #pragma unroll
-    for (int j = 0; j < TN; ++j) {
+        for (int j = 0; j < TN; ++j) {
 #pragma unroll
-        for (int rg = 0; rg < 4; ++rg) {
-            if (n < Nt) {
-                if (p + 3 < P) { /* the quad lies in one image (and n + 3 < Ntotal) */
-#pragma unroll
-                    for (int i = 0; i < TM; ++i) {
-                        if (!mok[i]) continue;
-                        float4u o;
-                        o.x = conv_tail_one(acc[i][j][rg * 4 + 0], row[i], a.slope);
-                        o.y = conv_tail_one(acc[i][j][rg * 4 + 1], row[i], a.slope);
-                        o.z = conv_tail_one(acc[i][j][rg * 4 + 2], row[i], a.slope);
-                        o.w = conv_tail_one(acc[i][j][rg * 4 + 3], row[i], a.slope);
-                        const long o_off = off + moff[i];
-                        *(float4u *)(a.out + o_off) = o;
-                        if (a.sum) {
-                            const float4u r = *(const float4u *)(a.add + o_off);
-                            float4u t;
-                            t.x = conv_residual_one(a, o.x, r.x);
-                            t.y = conv_residual_one(a, o.y, r.y);
-                            t.z = conv_residual_one(a, o.z, r.z);
-                            t.w = conv_residual_one(a, o.w, r.w);
-                            *(float4u *)(a.sum + o_off) = t;
-                        }
-                    }
-                } else {         /* image boundary or end of N inside the quad: element by element */
-                    int pc = p;
-                    long offc = off;
-#pragma unroll
-                    for (int c = 0; c < 4; ++c) {
-                        if (n + c < Nt) {
-                            while (pc >= P) {
-                                pc -= P;
-                                offc += wrap;
-                            }
-#pragma unroll
-                            for (int i = 0; i < TM; ++i) {
-                                if (!mok[i]) continue;
-                                const float y = conv_tail_one(acc[i][j][rg * 4 + c], row[i], a.slope);
-                                a.out[offc + moff[i]] = y;
-                                if (a.sum) a.sum[offc + moff[i]] = conv_residual_one(a, y, a.add[offc + moff[i]]);
-                            }
-                        }
-                        ++pc;
-                        ++offc;
-                    }
-                }
-            }
-            n += 8;
-            p += 8;
-            off += 8;
-            while (p >= P) {
-                p -= P;
-                off += wrap;
+            for (int rg = 0; rg < 4; ++rg) {
+                float4 o;
+                o.x = conv_tail_one(acc[i][j][rg * 4 + 0], row, a.slope);
+                o.y = conv_tail_one(acc[i][j][rg * 4 + 1], row, a.slope);
+                o.z = conv_tail_one(acc[i][j][rg * 4 + 2], row, a.slope);
+                o.w = conv_tail_one(acc[i][j][rg * 4 + 3], row, a.slope);
+                const int qq = j * 8 + 2 * rg + kh;
+                *(float4 *)&E[li * 64 + ((qq ^ (li & 15)) << 2)] = o;
             }
         }
+        __builtin_amdgcn_wave_barrier(); /* LDS operations of one wave complete in order */
+#pragma unroll
+        for (int t = 0; t < 8; ++t) {
+            const int f = fr + 4 * t;
+            const float4 o = *(const float4 *)&E[f * 64 + ((q ^ (f & 15)) << 2)];
+            const int m = mrow + f;
+            if (m >= a.M || n >= Nt) continue;
+            const long o_off = off + (long)m * P;
+            if (quad_ok) {
+                *(float4u *)(a.out + o_off) = (float4u){o.x, o.y, o.z, o.w};
+                if (a.sum) {
+                    const float4u r = *(const float4u *)(a.add + o_off);
+                    float4u s;
+                    s.x = conv_residual_one(a, o.x, r.x);
+                    s.y = conv_residual_one(a, o.y, r.y);
+                    s.z = conv_residual_one(a, o.z, r.z);
+                    s.w = conv_residual_one(a, o.w, r.w);
+                    *(float4u *)(a.sum + o_off) = s;
+                }
+            } else { /* image boundary or end of N inside the quad: element by element */
+                const float v[4] = {o.x, o.y, o.z, o.w};
+                int pc = p;
+                long offc = o_off;
+                for (int c = 0; c < 4 && n + c < Nt; ++c) {
+                    while (pc >= P) {
+                        pc -= P;
+                        offc += wrap;
+                    }
+                    a.out[offc] = v[c];
+                    if (a.sum) a.sum[offc] = conv_residual_one(a, v[c], a.add[offc]);
+                    ++pc;
+                    ++offc;
+                }
+            }
+        }
+        __builtin_amdgcn_wave_barrier();
     }
 }
 
@@ -511,7 +500,10 @@ __global__ __launch_bounds__(DN_THREADS, (BM == 128 ? 3 : 2)) void conv_mfma_ker
                 for (int r = 0; r < 16; ++r)
                     ws[((wave * TM * TN + i * TN + j) * 16 + r) * 64 + lane] = acc[i][j][r];
     } else {
-        conv_epilogue<TM, TN>(a, acc, m0, n0, wm0, wn0, li, kh);
+        __syncthreads(); /* every wave has read its last operands: the LDS buffers are free */
+        float *E = BM == 128 ? (wave == 0 ? As0 : wave == 1 ? As1 : wave == 2 ? Bs0 : Bs1)
+                             : (wave < 2 ? Bs0 : Bs1) + (wave & 1) * 2048;
+        conv_epilogue<TM, TN>(a, acc, E, m0, n0, wm0, wn0, lane);
     }
 #ifdef DN_TRACE
     if (a.trace) {
