@@ -66,7 +66,8 @@ struct mfma_args {
     long Ntotal;        /* batch * P */
     int stride, pad, size;
     int bn;
-    double slope;       /* activation as conv_inline_activation encodes it */
+    float slope_hi, slope_lo; /* activation slope (conv_inline_activation) as hi + lo floats */
+    float sum_slope_hi, sum_slope_lo;
     int tiles_m, tiles_n, per_xcd;
     unsigned in_records; /* bytes the gather may address: input + bias row */
     unsigned wp_records; /* bytes of the packed weights */
@@ -80,7 +81,6 @@ struct mfma_args {
     const float *add;
     float *sum;
     float s1, s2;
-    double sum_slope;
 #ifdef DN_TRACE
     unsigned long long *trace;
 #endif
@@ -111,7 +111,7 @@ __device__ __forceinline__ void split_k(int k, int size, int &ci, int &ky, int &
 typedef float float4u __attribute__((ext_vector_type(4), aligned(4)));
 
 /* The three activations the epilogue applies itself share one branch-free form,
- *     f(y) = y > 0 ? y : (float)(slope * (double)y),
+ *     f(y) = y > 0 ? y : (float)(slope * (double)y)      (evaluated as conv_mul_f2 below),
  * with slope .1 for leaky (src/activations.h:39), 1 for linear and 0 for relu: for relu the
  * reference's x*(x>0) (src/activations.h:35) and 0.*x agree on every input including -0, the
  * infinities and NaN.  Any other activation runs as a second pass over the output. */
@@ -124,27 +124,62 @@ __host__ __device__ inline bool conv_inline_activation(int act, double *slope)
     return true;
 }
 
-__device__ __forceinline__ float conv_slope(float y, double slope)
+/* A double constant as an unevaluated sum of two floats: x*hi + x*lo with one fused rounding,
+ * fmaf(x, hi, x*lo), reproduces (float)((double)x * c) except when the exact product lies within
+ * ~2^-48 (relative) of a float rounding boundary, at a third of the instruction cost of the
+ * convert / multiply / convert sequence in double precision. */
+struct conv_f2 {
+    float hi, lo;
+};
+
+__host__ __device__ inline conv_f2 conv_split(double c)
 {
-    return (y > 0) ? y : (float)(slope * (double)y);
+    conv_f2 r;
+    r.hi = (float)c;
+    r.lo = (float)(c - (double)r.hi);
+    return r;
 }
 
-/* batch-norm -> scale -> bias -> activation of one accumulator; without batch-norm the row holds
- * the neutral constants (mean 0, reciprocal 1, scale 1), which change no bit */
-__device__ __forceinline__ float conv_tail_one(float acc, const dn_bn_row &row, double slope)
+__device__ __forceinline__ float conv_mul_f2(float x, conv_f2 c) { return fmaf(x, c.hi, __fmul_rn(x, c.lo)); }
+
+__device__ __forceinline__ float conv_slope(float y, conv_f2 slope) { return (y > 0) ? y : conv_mul_f2(y, slope); }
+
+/* Per-filter constants of the tail: normalize (src/blas.c:154, as a multiplication by the
+ * reciprocal of the double denominator), scale, bias (src/batchnorm_layer.c:151-154), each step
+ * rounded to float as the reference's separate passes do.  Without batch-norm the constants are
+ * neutral (mean 0, reciprocal 1, scale 1) and change no bit. */
+struct conv_row_t {
+    conv_f2 inv;
+    float mean, scale, bias;
+};
+
+__device__ __forceinline__ conv_row_t conv_row(const mfma_args &a, int m)
 {
-    return conv_slope(dn_bn_apply(acc, row, 1), slope);
+    conv_row_t r;
+    r.bias = a.biases[m];
+    if (a.bn) {
+        r.inv = conv_split(1.0 / (sqrt((double)a.var[m]) + (double).000001f));
+        r.mean = a.mean[m];
+        r.scale = a.scales[m];
+    } else {
+        r.inv.hi = 1.f;
+        r.inv.lo = 0.f;
+        r.mean = 0.f;
+        r.scale = 1.f;
+    }
+    return r;
+}
+
+__device__ __forceinline__ float conv_tail_one(float acc, const conv_row_t &row, conv_f2 slope)
+{
+    float x = conv_mul_f2(__fsub_rn(acc, row.mean), row.inv);
+    x = __fadd_rn(__fmul_rn(x, row.scale), row.bias);
+    return conv_slope(x, slope);
 }
 
 __device__ __forceinline__ float conv_residual_one(const mfma_args &a, float y, float r)
 {
-    return conv_slope(__fadd_rn(__fmul_rn(a.s1, y), __fmul_rn(a.s2, r)), a.sum_slope);
-}
-
-__device__ __forceinline__ dn_bn_row conv_row(const mfma_args &a, int m)
-{
-    return dn_bn_make(a.bn, a.biases[m], a.bn ? a.scales[m] : 1.f, a.bn ? a.mean[m] : 0.f,
-                      a.bn ? a.var[m] : 1.f);
+    return conv_slope(__fadd_rn(__fmul_rn(a.s1, y), __fmul_rn(a.s2, r)), conv_f2{a.sum_slope_hi, a.sum_slope_lo});
 }
 
 /* Batch-norm / bias / activation and the store.  The MFMAs are issued with the pixel tile as
@@ -176,16 +211,16 @@ __device__ __forceinline__ void conv_epilogue(const mfma_args &a, f32x16 (&acc)[
 #pragma unroll
     for (int i = 0; i < TM; ++i) {
         const int mrow = m0 + wm0 + i * 32;
-        const dn_bn_row row = conv_row(a, mrow + li < a.M ? mrow + li : a.M - 1);
+        const conv_row_t row = conv_row(a, mrow + li < a.M ? mrow + li : a.M - 1);
 #pragma unroll
         for (int j = 0; j < TN; ++j) {
 #pragma unroll
             for (int rg = 0; rg < 4; ++rg) {
                 float4 o;
-                o.x = conv_tail_one(acc[i][j][rg * 4 + 0], row, a.slope);
-                o.y = conv_tail_one(acc[i][j][rg * 4 + 1], row, a.slope);
-                o.z = conv_tail_one(acc[i][j][rg * 4 + 2], row, a.slope);
-                o.w = conv_tail_one(acc[i][j][rg * 4 + 3], row, a.slope);
+                o.x = conv_tail_one(acc[i][j][rg * 4 + 0], row, conv_f2{a.slope_hi, a.slope_lo});
+                o.y = conv_tail_one(acc[i][j][rg * 4 + 1], row, conv_f2{a.slope_hi, a.slope_lo});
+                o.z = conv_tail_one(acc[i][j][rg * 4 + 2], row, conv_f2{a.slope_hi, a.slope_lo});
+                o.w = conv_tail_one(acc[i][j][rg * 4 + 3], row, conv_f2{a.slope_hi, a.slope_lo});
                 const int qq = j * 8 + 2 * rg + kh;
                 *(float4 *)&E[li * 64 + ((qq ^ (li & 15)) << 2)] = o;
             }
@@ -304,10 +339,10 @@ __global__ __launch_bounds__(DN_THREADS, (BM == 128 ? 3 : 2)) void conv_mfma_ker
     for (int g = 0; g < NG_PER_WAVE; ++g) {
         const long ncol = n0 + (wave * NG_PER_WAVE + g) * 16 + nl;
         const bool col_ok = ncol < a.Ntotal;
-        const long nn = col_ok ? ncol : 0;
-        const int b = (int)(nn / a.P);
-        const int p = (int)(nn - (long)b * a.P);
-        const int oy = p / a.OW;
+        const unsigned nn = col_ok ? (unsigned)ncol : 0u; /* Ntotal < 2^31 on this path */
+        const int b = (int)(nn / (unsigned)a.P);
+        const int p = (int)nn - b * a.P;
+        const int oy = (int)((unsigned)p / (unsigned)a.OW);
         const int ox = p - oy * a.OW;
         iy0[g] = col_ok ? oy * a.stride - a.pad : -0x1000000;
         ix0[g] = ox * a.stride - a.pad;
@@ -568,9 +603,9 @@ __global__ __launch_bounds__(DN_THREADS) void conv_reduce_kernel(mfma_args a)
     for (int c = 0; c < 4; ++c) {
         const int m = mbase + c;
         if (m >= a.M) break;
-        const dn_bn_row row = conv_row(a, m);
+        const conv_row_t row = conv_row(a, m);
         const long off = ((long)b * a.M + m) * a.P + p;
-        const float y = conv_tail_one(vals[c], row, a.slope);
+        const float y = conv_tail_one(vals[c], row, conv_f2{a.slope_hi, a.slope_lo});
         a.out[off] = y;
         if (a.sum) a.sum[off] = conv_residual_one(a, y, a.add[off]);
     }
@@ -850,7 +885,8 @@ static void conv_forward(const float *input, const float *weights, const float *
     a.pad = pad;
     a.size = size;
     a.bn = batch_normalize ? 1 : 0;
-    a.slope = slope;
+    a.slope_hi = conv_split(slope).hi;
+    a.slope_lo = conv_split(slope).lo;
     a.tiles_m = a.tiles_n = a.per_xcd = 0;
     a.whole_tiles = 0;
     a.split = 1;
@@ -859,7 +895,8 @@ static void conv_forward(const float *input, const float *weights, const float *
     a.sum = sum;
     a.s1 = s1;
     a.s2 = s2;
-    a.sum_slope = sum_slope;
+    a.sum_slope_hi = conv_split(sum_slope).hi;
+    a.sum_slope_lo = conv_split(sum_slope).lo;
     a.in_records = (unsigned)((long)batch * c * h * w * 4 + (long)(w + 1) * 4);
     a.wp_records = (unsigned)(conv_packed_floats(n, c, groups, size) * 4);
     if (n <= 32)
