@@ -81,9 +81,6 @@ struct mfma_args {
     const float *add;
     float *sum;
     float s1, s2;
-#ifdef DN_TRACE
-    unsigned long long *trace;
-#endif
 };
 
 /* k -> (channel, ky, kx) for a size x size kernel in the reference's im2col row order. */
@@ -282,9 +279,6 @@ __global__ __launch_bounds__(DN_THREADS, (BM == 128 ? 3 : 2)) void conv_mfma_ker
 
     /* XCD-aware tile order: workgroup id -> (xcd, slot) -> linear tile with tile_m fastest. */
     const int bid = blockIdx.x;
-#ifdef DN_TRACE
-    unsigned long long tr0 = __builtin_amdgcn_s_memrealtime(), tr1 = 0, tr2 = 0;
-#endif
     int lin, kc_begin = 0, kc_end = a.KCH, slice_id = -1;
     if (bid < 8 * a.per_xcd) {
         lin = (bid & 7) * a.per_xcd + (bid >> 3);
@@ -451,9 +445,6 @@ __global__ __launch_bounds__(DN_THREADS, (BM == 128 ? 3 : 2)) void conv_mfma_ker
     load_chunk(kc_begin, 0);
     __builtin_amdgcn_s_waitcnt(0);
     __syncthreads();
-#ifdef DN_TRACE
-    tr1 = __builtin_amdgcn_s_memrealtime();
-#endif
 
     float4 av[2][TM], bv[2][TN]; /* MFMA operands of the current chunk: [k half][32-row block] */
 
@@ -519,11 +510,6 @@ __global__ __launch_bounds__(DN_THREADS, (BM == 128 ? 3 : 2)) void conv_mfma_ker
         last(0);
     }
 
-#ifdef DN_TRACE
-    __builtin_amdgcn_sched_barrier(0);
-    tr2 = __builtin_amdgcn_s_memrealtime();
-    __builtin_amdgcn_sched_barrier(0);
-#endif
     if (slice_id >= 0) {
         /* K-slice: park the raw accumulators, lane-major so every store is a full 256-byte row */
         float *ws = a.partial + (long)slice_id * (BM * BN);
@@ -540,23 +526,6 @@ __global__ __launch_bounds__(DN_THREADS, (BM == 128 ? 3 : 2)) void conv_mfma_ker
                              : (wave < 2 ? Bs0 : Bs1) + (wave & 1) * 2048;
         conv_epilogue<TM, TN>(a, acc, E, m0, n0, wm0, wn0, lane);
     }
-#ifdef DN_TRACE
-    if (a.trace) {
-        __builtin_amdgcn_s_waitcnt(0);
-        __syncthreads();
-        if (tid == 0) {
-            const unsigned hw = __builtin_amdgcn_s_getreg(4 | (0 << 6) | (15 << 11));
-            const unsigned xcc = __builtin_amdgcn_s_getreg(20 | (0 << 6) | (3 << 11));
-            unsigned long long *t = a.trace + (long)bid * 6;
-            t[0] = ((unsigned long long)xcc << 32) | hw;
-            t[1] = tr0;
-            t[2] = tr1;
-            t[3] = tr2;
-            t[4] = __builtin_amdgcn_s_memrealtime();
-            t[5] = (unsigned long long)(kc_end - kc_begin) | ((unsigned long long)(slice_id >= 0) << 32);
-        }
-    }
-#endif
 }
 
 /* Sums the K-slices of the tail tiles in slice order (deterministic) and applies the epilogue.
@@ -748,13 +717,6 @@ static void launch_tile(const mfma_args &a0, int mode)
         a.partial = g_partial;
     }
     const dim3 grid((unsigned)(a.per_xcd * 8 + tail * split));
-#ifdef DN_TRACE
-    a.trace = 0;
-    if (getenv("DN_TRACE")) {
-        hip_check_error(hipMalloc((void **)&a.trace, (size_t)grid.x * 48));
-        hip_check_error(hipMemset(a.trace, 0, (size_t)grid.x * 48));
-    }
-#endif
     if (BM > 128 && mode != 11 && mode != 13) dn_fatal("conv dispatch: the 256-row tile is only built for the tap-blocked modes");
     switch (mode) {
     case 11: hipLaunchKernelGGL((conv_mfma_kernel<BM, BN, WM, WN, 11>), grid, dim3(DN_THREADS), 0, dn_stream(), a); break;
@@ -770,20 +732,6 @@ static void launch_tile(const mfma_args &a0, int mode)
         }
         break;
     }
-#ifdef DN_TRACE
-    if (a.trace) {
-        static int seq = 0;
-        unsigned long long *h = (unsigned long long *)malloc((size_t)grid.x * 48);
-        hip_check_error(hipDeviceSynchronize());
-        hip_check_error(hipMemcpy(h, a.trace, (size_t)grid.x * 48, hipMemcpyDeviceToHost));
-        char name[256];
-        snprintf(name, sizeof name, "%s/trace_%03d.bin", getenv("DN_TRACE"), seq++);
-        FILE *f = fopen(name, "wb");
-        if (f) { fwrite(h, 48, grid.x, f); fclose(f); }
-        free(h);
-        hip_check_error(hipFree(a.trace));
-    }
-#endif
     if (tail > 0)
         hipLaunchKernelGGL((conv_reduce_kernel<BM, BN, WM, WN>), dim3((unsigned)(tail * (BM * BN / 4 / DN_THREADS))),
                            dim3(DN_THREADS), 0, dn_stream(), a);
