@@ -243,8 +243,11 @@ def main():
             k["launches"] += 1
         # a same-geometry shortcut right after a convolution runs inside that convolution's
         # epilogue: its event interval is empty and its traffic belongs to the conv kernel
-        row["fused"] = bool(Ly["type"] == "shortcut" and i > 0 and net.layers[i - 1]["type"] == "convolutional"
-                            and ms < 0.25 * row["bytes"] / (PEAK_HBM_GBS * 1e6))
+        prev = net.layers[i - 1] if i else None
+        row["fused"] = bool(Ly["type"] == "shortcut" and prev and prev["type"] == "convolutional"
+                            and not prev["xnor"] and 0 <= Ly["index"] < i - 1
+                            and (Ly["w"], Ly["h"], Ly["c"]) == (Ly["out_w"], Ly["out_h"], Ly["out_c"])
+                            and (Ly["out_w"], Ly["out_h"], Ly["out_c"]) == (prev["out_w"], prev["out_h"], prev["out_c"]))
         row["gbs"] = row["bytes"] / ms / 1e6 if ms > 0 and not row["fused"] else 0.0
         rows.append(row)
     dom_name, dom = max(kernels.items(), key=lambda kv: kv[1]["ms"])
