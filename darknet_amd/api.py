@@ -31,6 +31,43 @@ def _fp(a):
     return a.ctypes.data_as(_F)
 
 
+class BOX(C.Structure):
+    """python/darknet.py:22-26"""
+    _fields_ = [("x", C.c_float), ("y", C.c_float), ("w", C.c_float), ("h", C.c_float)]
+
+
+class DETECTION(C.Structure):
+    """python/darknet.py:28-34"""
+    _fields_ = [("bbox", BOX), ("classes", C.c_int), ("prob", _F), ("mask", _F),
+                ("objectness", C.c_float), ("sort_class", C.c_int)]
+
+
+def _rows_of(dets, n, classes):
+    rows = np.zeros((n, 5 + classes), np.float32)
+    for i in range(n):
+        d = dets[i]
+        rows[i, :5] = (d.bbox.x, d.bbox.y, d.bbox.w, d.bbox.h, d.objectness)
+        rows[i, 5:] = np.ctypeslib.as_array(d.prob, shape=(classes,)) if classes else 0
+    return rows
+
+
+def do_nms_sort(rows: np.ndarray, classes: int, thresh: float) -> np.ndarray:
+    """do_nms_sort (python/darknet.py:98-100) on rows [n, 5 + classes] = x, y, w, h, objectness,
+    prob[classes]; returns the rows as the library leaves its detection array."""
+    L = _lib.load()
+    rows = np.ascontiguousarray(rows, np.float32)
+    n = rows.shape[0]
+    dets = (DETECTION * max(n, 1))()
+    keep = [np.ascontiguousarray(rows[i, 5:]).copy() for i in range(n)]
+    for i in range(n):
+        dets[i].bbox = BOX(*[float(v) for v in rows[i, :4]])
+        dets[i].classes = classes
+        dets[i].prob = _fp(keep[i])
+        dets[i].objectness = float(rows[i, 4])
+    L.do_nms_sort(C.cast(dets, C.c_void_p), n, classes, thresh)
+    return _rows_of(dets, n, classes)
+
+
 def set_gpu(n: int = 0):
     _lib.load().cuda_set_device(n)
 
@@ -178,6 +215,25 @@ class Network:
         L = self.layers[i]
         p = self.L.layer_indexes_host(self.net, i)
         return np.ctypeslib.as_array(p, shape=(L["batch"], L["outputs"])).copy()
+
+    def get_boxes(self, w, h, thresh, relative=1, nms=0.0, image=0):
+        """get_network_boxes (python/darknet.py:86-88) for `image` of the batch, with the
+        suppression of do_nms_sort when nms > 0 -> rows [n, 5 + classes]."""
+        num = C.c_int(0)
+        dets = self.L.get_network_boxes_image(self.net, image, w, h, thresh, relative, nms, C.byref(num))
+        classes = max([L["classes"] for L in self.layers if L["type"] == "yolo"] + [0])
+        rows = _rows_of(C.cast(dets, C.POINTER(DETECTION)), num.value, classes)
+        self.L.free_detections(dets, num.value)
+        return rows
+
+    def get_network_boxes(self, w, h, thresh, relative=1):
+        """The reference's own call (image 0, no suppression)."""
+        num = C.c_int(0)
+        dets = self.L.get_network_boxes(self.net, w, h, thresh, 0.5, None, relative, C.byref(num))
+        classes = max([L["classes"] for L in self.layers if L["type"] == "yolo"] + [0])
+        rows = _rows_of(C.cast(dets, C.POINTER(DETECTION)), num.value, classes)
+        self.L.free_detections(dets, num.value)
+        return rows
 
     def conv_flops(self):
         return float(self.L.network_conv_flops(self.net))

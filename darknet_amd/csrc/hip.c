@@ -100,6 +100,7 @@ int *hip_make_int_array(int *x, size_t n)
     hip_check_error(hipMalloc((void **)&x_gpu, size));
     if (!x_gpu) dn_fatal("hipMalloc returned a null pointer");
     if (x) hip_check_error(hipMemcpy(x_gpu, x, sizeof(int) * n, hipMemcpyHostToDevice));
+    else hip_check_error(hipMemset(x_gpu, 0, size));
     return x_gpu;
 }
 
@@ -120,6 +121,12 @@ void hip_pull_array(float *x_gpu, float *x, size_t n)
 {
     if (g_stream) hip_check_error(hipStreamSynchronize(g_stream));
     hip_check_error(hipMemcpy(x, x_gpu, sizeof(float) * n, hipMemcpyDeviceToHost));
+}
+
+void hip_push_int_array(int *x_gpu, int *x, size_t n)
+{
+    if (g_stream) hip_check_error(hipStreamSynchronize(g_stream));
+    hip_check_error(hipMemcpy(x_gpu, x, sizeof(int) * n, hipMemcpyHostToDevice));
 }
 
 void hip_pull_int_array(int *x_gpu, int *x, size_t n)

@@ -28,6 +28,8 @@ void free_network(network *net)
     free(net->input);
     free(net->seen);
     if (net->input_gpu) hip_free(net->input_gpu);
+    if (net->det_rows_gpu) hip_free(net->det_rows_gpu);
+    if (net->det_count_gpu) hip_free((float *)net->det_count_gpu);
     free(net);
 }
 

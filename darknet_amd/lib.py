@@ -25,7 +25,8 @@ SIGNATURES = {
     "hip_make_array": (V, [F, z]), "hip_make_int_array": (V, [I, z]), "hip_free": (None, [V]),
     "hip_push_array": (None, [V, F, z]), "hip_pull_array": (None, [V, F, z]),
     "hip_mag_array": (f, [V, z]), "hip_compare": (f, [V, F, z, C.c_char_p]),
-    "hip_pull_int_array": (None, [V, I, z]), "hip_synchronize": (None, []),
+    "hip_pull_int_array": (None, [V, I, z]), "hip_push_int_array": (None, [V, I, z]),
+    "hip_synchronize": (None, []),
     "hip_get_stream": (V, []), "hip_set_stream": (None, [V]), "hip_device_name": (C.c_char_p, []),
     "cuda_set_device": (None, [i]), "cuda_get_device": (i, []), "cuda_make_array": (V, [F, z]),
     "cuda_make_int_array": (V, [I, z]), "cuda_free": (None, [V]),
@@ -63,6 +64,14 @@ SIGNATURES = {
     "save_weights": (None, [V, C.c_char_p]), "save_weights_upto": (None, [V, C.c_char_p, i]),
     "get_activation": (i, [C.c_char_p]), "get_activation_string": (C.c_char_p, [i]),
     "get_layer_string": (C.c_char_p, [i]),
+    "yolo_decode_gpu": (None, [V, i, i, i, i, F, i, i, i, i, i, f, V, i, V]),
+    "nms_sort_gpu": (None, [V, i, i, f]),
+    "num_detections": (i, [V, f]), "make_network_boxes": (V, [V, f, I]),
+    "fill_network_boxes": (None, [V, i, i, f, f, I, i, V]),
+    "get_network_boxes": (V, [V, i, i, f, f, I, i, I]), "free_detections": (None, [V, i]),
+    "do_nms_sort": (None, [V, i, i, f]),
+    "get_network_boxes_image": (V, [V, i, i, i, f, i, f, I]),
+    "network_decode_image_gpu": (i, [V, i, i, i, f, i]),
     "make_network": (V, [i]), "free_network": (None, [V]), "forward_network": (None, [V]),
     "forward_network_gpu": (None, [V]), "network_predict": (F, [V, F]),
     "set_batch_network": (None, [V, i]), "network_output": (F, [V]),

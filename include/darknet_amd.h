@@ -146,7 +146,26 @@ typedef struct network {
     float *truth_gpu;
     float *delta_gpu;
     float *output_gpu;
+
+    /* additions of this library: device row buffer of the detection decode */
+    float *det_rows_gpu;
+    int *det_count_gpu;
+    int det_max_rows;
 } network;
+
+/* include/darknet.h:515-526 */
+typedef struct {
+    float x, y, w, h;
+} box;
+
+typedef struct detection {
+    box bbox;
+    int classes;
+    float *prob;
+    float *mask;
+    float objectness;
+    int sort_class;
+} detection;
 
 /* ---- cfg parsing (src/parser.c:742-889; list/option helpers src/list.c, src/option_list.c) */
 network *parse_network_cfg(char *filename);
@@ -200,6 +219,22 @@ float *network_output(network *net);                        /* src/network.c:755
 void pull_network_output(network *net);                     /* src/network.c:1123 */
 int network_width(network *net);                            /* src/network.c:674 */
 int network_height(network *net);                           /* src/network.c:675 */
+
+/* ---- detections (yolo heads only; region/detection layers are outside the path) ---------- */
+int num_detections(network *net, float thresh);                       /* src/network.c:510 */
+detection *make_network_boxes(network *net, float thresh, int *num);  /* src/network.c:526 */
+void fill_network_boxes(network *net, int w, int h, float thresh, float hier, int *map, int relative,
+                        detection *dets);                             /* src/network.c:543 */
+detection *get_network_boxes(network *net, int w, int h, float thresh, float hier, int *map,
+                             int relative, int *num);                 /* src/network.c:563 */
+void free_detections(detection *dets, int n);                         /* src/network.c:570 */
+void do_nms_sort(detection *dets, int total, int classes, float thresh); /* src/box.c:58 */
+/* additions: the same for image b of the batch (the reference reads image 0 only), with the
+ * suppression done on the device before the rows are copied back when nms > 0; and the decode
+ * alone, leaving the rows in net->det_rows_gpu and returning their number */
+detection *get_network_boxes_image(network *net, int b, int w, int h, float thresh, int relative,
+                                   float nms, int *num);
+int network_decode_image_gpu(network *net, int b, int w, int h, float thresh, int relative);
 
 /* ---- additions (no reference twin) --------------------------------------------------------
  * forward_network_device: the layer loop alone, on whatever net->input_gpu holds; no host<->

@@ -46,6 +46,7 @@ void   hip_pull_array(float *x_gpu, float *x, size_t n);/* cuda_pull_array      
 float  hip_mag_array(float *x_gpu, size_t n);           /* cuda_mag_array       src/cuda.c:167 */
 float  hip_compare(float *x_gpu, float *x, size_t n, char *s); /* cuda_compare  src/cuda.c:120 */
 void   hip_pull_int_array(int *x_gpu, int *x, size_t n);/* (maxpool indexes; no reference twin) */
+void   hip_push_int_array(int *x_gpu, int *x, size_t n);/* (counters; no reference twin)        */
 void   hip_synchronize(void);                           /* hipStreamSynchronize on the stream  */
 void  *hip_get_stream(void);                            /* hipStream_t the library launches on */
 void   hip_set_stream(void *stream);                    /* 0 selects the null stream           */
@@ -193,6 +194,31 @@ void forward_yolo_gpu(const float *input, float *output, int batch, int w, int h
 
 /* forward_avgpool_layer_gpu (src/avgpool_layer_kernels.cu:46-54). */
 void forward_avgpool_gpu(const float *input, float *output, int batch, int c, int h, int w);
+
+/* ------------------------------------------------------------------------------------------
+ * Detections: the step right after the forward pass.  A detection is a row of (5 + classes)
+ * floats in device memory: x, y, w, h, objectness, prob[classes].
+ * ---------------------------------------------------------------------------------------- */
+
+/* Thresholded decode of ONE yolo head of ONE image, appended to `rows`.  Replaces
+ * yolo_num_detections + get_yolo_detections (src/yolo_layer.c:275-343) with get_yolo_box
+ * (:83-91) and correct_yolo_boxes (:247-273): a cell/anchor whose objectness exceeds `thresh`
+ * becomes a row, prob[j] = objectness*class_j if that exceeds `thresh`, else 0; rows keep the
+ * reference's order (cells row-major, anchors inside a cell).
+ *   layer_output  device, the image's slab of the yolo layer output [n][5+classes][lh][lw]
+ *   anchors       HOST, 2*n floats: biases[2*mask[i]], biases[2*mask[i]+1]  (n <= 16)
+ *   netw,neth     network input size; w,h the original image size; relative as the reference
+ *   rows,max_rows device row buffer and its capacity in rows
+ *   count         device int: rows already present; incremented by the rows this head adds even
+ *                 past max_rows (nothing is written past it), so the caller can tell overflow */
+void yolo_decode_gpu(const float *layer_output, int lw, int lh, int n, int classes,
+                     const float *anchors, int netw, int neth, int w, int h, int relative,
+                     float thresh, float *rows, int max_rows, int *count);
+
+/* do_nms_sort (src/box.c:58-89) on device rows, in place: per class, in descending
+ * probability (ties: lower row first), a row zeroes that class's probability in every later row
+ * whose box_iou (src/box.c:152-155) with it exceeds `thresh`.  Rows keep their positions. */
+void nms_sort_gpu(float *rows, int total, int classes, float thresh);
 
 #ifdef __cplusplus
 }

@@ -176,6 +176,32 @@ class Oracle:
         self.lib.orc_yolo(_fp(x), _fp(out), b, w, h, n_anchors, classes)
         return out
 
+    def yolo_detections(self, pred, n_anchors, classes, biases, mask, netw, neth, w, h, relative, thresh):
+        """get_yolo_detections on image 0 of `pred` [n*(5+classes), lh, lw] -> rows [count, 5+classes]."""
+        pred = np.ascontiguousarray(pred, np.float32)
+        lh, lw = pred.shape[-2:]
+        rows = np.zeros((lw * lh * n_anchors, 5 + classes), np.float32)
+        bi = np.ascontiguousarray(biases, np.float32)
+        mk = np.ascontiguousarray(mask, np.int32)
+        f = self.lib.orc_yolo_detections
+        f.restype = C.c_int
+        n = f(_fp(pred), lw, lh, n_anchors, classes, _fp(bi), mk.ctypes.data_as(C.POINTER(C.c_int)),
+              netw, neth, w, h, relative, C.c_float(thresh), _fp(rows))
+        return rows[:n].copy()
+
+    def nms_sort(self, rows, classes, thresh):
+        """do_nms_sort on rows [n, 5+classes]; returns the suppressed copy (row order kept)."""
+        out = np.ascontiguousarray(rows, np.float32).copy()
+        self.lib.orc_nms_sort(_fp(out), out.shape[0], classes, C.c_float(thresh))
+        return out
+
+    def box_iou(self, a, b):
+        f = self.lib.orc_box_iou
+        f.restype = C.c_float
+        a = np.ascontiguousarray(a, np.float32)
+        b = np.ascontiguousarray(b, np.float32)
+        return float(f(_fp(a), _fp(b)))
+
     def avgpool(self, x):
         b, c, h, w = x.shape
         out = np.empty((b, c), np.float32)

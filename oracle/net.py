@@ -65,3 +65,24 @@ class OracleNet:
             outs.append(y)
             cur = y
         return outs
+
+    def get_boxes(self, outs, w, h, thresh, relative=1, nms=0.0, image=0):
+        """get_network_boxes (src/network.c:563, fill order :543-561) on layer outputs `outs`,
+        then do_nms_sort when nms > 0.  Rows [n, 5 + classes] in the reference's fill order."""
+        rows = []
+        classes = 0
+        for i, L in enumerate(self.layers):
+            if L["type"] != "yolo":
+                continue
+            classes = L["classes"]
+            anchors = L.get("anchors", [0.5] * (2 * L["total"]))
+            biases = np.full(2 * L["total"], 0.5, np.float32)
+            biases[:min(len(anchors), biases.size)] = anchors[:biases.size]
+            pred = np.asarray(outs[i], np.float32).reshape(L["batch"], L["c"], L["h"], L["w"])[image]
+            rows.append(self.orc.yolo_detections(pred, L["n"], classes, biases, L["mask"], self.net["w"],
+                                                 self.net["h"], w, h, relative, thresh))
+        rows = np.concatenate(rows) if rows else np.zeros((0, 5), np.float32)
+        if nms > 0 and len(rows):
+            rows = self.orc.nms_sort(rows, classes, nms)
+        return rows
+

@@ -13,6 +13,7 @@
 
 #include <float.h>
 #include <math.h>
+#include <stdlib.h>
 #include <string.h>
 
 /* ---- im2col: src/im2col.c:3-12 (pixel fetch with zero outside), :16-39 (unroll) -------- */
@@ -406,4 +407,129 @@ void orc_softmax(const float *input, int n, int batch, int batch_offset, int gro
         for (int g = 0; g < groups; ++g)
             softmax_one(input + b * batch_offset + g * group_offset, n, temp, stride,
                         output + b * batch_offset + g * group_offset);
+}
+
+/* ---- detections out of one yolo head: get_yolo_detections src/yolo_layer.c:316-343 for image
+ * 0 of `pred` ([anchor][entry][lh][lw]), with get_yolo_box :83-91 and correct_yolo_boxes
+ * :247-273.  Rows of (5 + classes) floats: x, y, w, h, objectness, prob[classes].  Returns the
+ * number of rows written (the caller sizes `rows` for lw*lh*n). ---------------------------- */
+int orc_yolo_detections(const float *pred, int lw, int lh, int n, int classes, const float *biases,
+                        const int *mask, int netw, int neth, int w, int h, int relative, float thresh,
+                        float *rows)
+{
+    const int cells = lw * lh;
+    const int entries = 5 + classes;
+    int count = 0;
+    for (int i = 0; i < cells; ++i) {
+        const int row = i / lw;
+        const int col = i % lw;
+        for (int a = 0; a < n; ++a) {
+            const float *p = pred + (long)a * cells * entries + i;
+            const float objectness = p[4L * cells];
+            if (objectness <= thresh) continue;
+            float *r = rows + (long)count * entries;
+            /* get_yolo_box: stride = lw*lh */
+            r[0] = (col + p[0]) / lw;
+            r[1] = (row + p[1L * cells]) / lh;
+            r[2] = exp(p[2L * cells]) * biases[2 * mask[a]] / netw;
+            r[3] = exp(p[3L * cells]) * biases[2 * mask[a] + 1] / neth;
+            r[4] = objectness;
+            for (int j = 0; j < classes; ++j) {
+                const float prob = objectness * p[(long)(5 + j) * cells];
+                r[5 + j] = (prob > thresh) ? prob : 0;
+            }
+            ++count;
+        }
+    }
+    /* correct_yolo_boxes */
+    int new_w = 0, new_h = 0;
+    if (((float)netw / w) < ((float)neth / h)) {
+        new_w = netw;
+        new_h = (h * netw) / w;
+    } else {
+        new_h = neth;
+        new_w = (w * neth) / h;
+    }
+    for (int i = 0; i < count; ++i) {
+        float *r = rows + (long)i * entries;
+        float bx = r[0], by = r[1], bw = r[2], bh = r[3];
+        bx = (bx - (netw - new_w) / 2. / netw) / ((float)new_w / netw);
+        by = (by - (neth - new_h) / 2. / neth) / ((float)new_h / neth);
+        bw *= (float)netw / new_w;
+        bh *= (float)neth / new_h;
+        if (!relative) {
+            bx *= w;
+            bw *= w;
+            by *= h;
+            bh *= h;
+        }
+        r[0] = bx;
+        r[1] = by;
+        r[2] = bw;
+        r[3] = bh;
+    }
+    return count;
+}
+
+/* box_iou: src/box.c:111-155 */
+static float orc_overlap(float x1, float w1, float x2, float w2)
+{
+    float l1 = x1 - w1 / 2;
+    float l2 = x2 - w2 / 2;
+    float left = l1 > l2 ? l1 : l2;
+    float r1 = x1 + w1 / 2;
+    float r2 = x2 + w2 / 2;
+    float right = r1 < r2 ? r1 : r2;
+    return right - left;
+}
+
+float orc_box_iou(const float *a, const float *b)
+{
+    float w = orc_overlap(a[0], a[2], b[0], b[2]);
+    float h = orc_overlap(a[1], a[3], b[1], b[3]);
+    float inter = (w < 0 || h < 0) ? 0 : w * h;
+    float uni = a[2] * a[3] + b[2] * b[3] - inter;
+    return inter / uni;
+}
+
+/* do_nms_sort: src/box.c:58-89, on rows that stay in place (the reference reorders its array;
+ * here an index permutation is sorted instead, which suppresses the same pairs).  Ties in the
+ * sort keep the lower row first. */
+struct orc_nms_key {
+    float p;
+    int i;
+};
+
+static int orc_nms_cmp(const void *pa, const void *pb)
+{
+    const struct orc_nms_key *a = (const struct orc_nms_key *)pa, *b = (const struct orc_nms_key *)pb;
+    float diff = a->p - b->p; /* nms_comparator src/box.c:5-21: descending probability */
+    if (diff < 0) return 1;
+    if (diff > 0) return -1;
+    return a->i - b->i;
+}
+
+void orc_nms_sort(float *rows, int total, int classes, float thresh)
+{
+    const int entries = 5 + classes;
+    struct orc_nms_key *keys = (struct orc_nms_key *)calloc((size_t)(total > 0 ? total : 1), sizeof *keys);
+    for (int k = 0; k < classes; ++k) {
+        int n = 0;
+        for (int i = 0; i < total; ++i) {
+            if (rows[(long)i * entries + 4] == 0) continue; /* objectness 0: dropped up front (:62-71) */
+            keys[n].p = rows[(long)i * entries + 5 + k];
+            keys[n].i = i;
+            ++n;
+        }
+        qsort(keys, (size_t)n, sizeof *keys, orc_nms_cmp);
+        for (int i = 0; i < n; ++i) {
+            float *a = rows + (long)keys[i].i * entries;
+            if (a[5 + k] == 0) continue;
+            for (int j = i + 1; j < n; ++j) {
+                float *b = rows + (long)keys[j].i * entries;
+                if (orc_box_iou(a, b) > thresh) b[5 + k] = 0;
+            }
+        }
+    }
+    free(keys);
 }

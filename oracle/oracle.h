@@ -69,6 +69,13 @@ void orc_avgpool(const float *input, float *output, int batch, int c, int h, int
 void orc_softmax(const float *input, int n, int batch, int batch_offset, int groups,
                  int group_offset, int stride, float temp, float *output);
 
+/* detections (test infrastructure like everything here): see oracle.c */
+int orc_yolo_detections(const float *pred, int lw, int lh, int n, int classes, const float *biases,
+                        const int *mask, int netw, int neth, int w, int h, int relative, float thresh,
+                        float *rows);
+float orc_box_iou(const float *a, const float *b);
+void orc_nms_sort(float *rows, int total, int classes, float thresh);
+
 #ifdef __cplusplus
 }
 #endif

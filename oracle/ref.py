@@ -68,6 +68,8 @@ class RefNet:
         H.refh_layer_indexes.restype = _I
         H.refh_layer_indexes.argtypes = [C.c_void_p, C.c_int]
         H.refh_forward_layer.argtypes = [C.c_void_p, C.c_int, _F]
+        H.refh_get_boxes.argtypes = [C.c_void_p, C.c_int, C.c_int, C.c_float, C.c_int, C.c_float, _F, C.c_int]
+        H.refh_set_output.argtypes = [C.c_void_p, C.c_int, _F]
         self.net = H.refh_load(cfg_path.encode())
         if not self.net:
             raise RuntimeError("reference failed to parse " + cfg_path)
@@ -101,6 +103,20 @@ class RefNet:
     def set_conv(self, i, weights, biases, scales=None, mean=None, var=None):
         p = lambda a: None if a is None else np.ascontiguousarray(a, np.float32).ctypes.data_as(_F)
         self.h.refh_set_conv(self.net, i, p(weights), p(biases), p(scales), p(mean), p(var))
+
+    def set_output(self, i, values):
+        """Overwrite layer i's host output (drives get_boxes with chosen yolo tensors)."""
+        v = np.ascontiguousarray(values, np.float32)
+        assert v.size == self.layers[i]["outputs"] * self.batch
+        self.h.refh_set_output(self.net, i, v.ctypes.data_as(_F))
+
+    def get_boxes(self, w, h, thresh, relative=1, nms=0.0):
+        """get_network_boxes (+ do_nms_sort when nms > 0) -> rows [n, 5 + classes]."""
+        classes = self.layers[-1]["classes"]
+        cap = sum(L["w"] * L["h"] * L["n"] for L in self.layers if L["type"] == "yolo")
+        rows = np.zeros((max(cap, 1), 5 + classes), np.float32)
+        n = self.h.refh_get_boxes(self.net, w, h, thresh, relative, nms, rows.ctypes.data_as(_F), cap)
+        return rows[:n].copy()
 
     def predict(self, x):
         x = np.ascontiguousarray(x, np.float32)

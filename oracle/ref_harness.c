@@ -130,3 +130,36 @@ void refh_forward_layer(network *net, int i, float *input)
     copy.index = i;
     l.forward(l, copy);
 }
+
+/* get_network_boxes (src/network.c:563) on the outputs of the last refh_predict, optionally
+ * followed by do_nms_sort (src/box.c:58), flattened to rows of 5 + classes floats:
+ * x, y, w, h, objectness, prob[classes].  Returns the number of detections (rows beyond `cap`
+ * are not written).  The reference leaves the array sorted by the last class after NMS; callers
+ * compare order-free. */
+int refh_get_boxes(network *net, int w, int h, float thresh, int relative, float nms, float *rows, int cap)
+{
+    int n = 0, i, j;
+    layer l = net->layers[net->n - 1];
+    detection *dets = get_network_boxes(net, w, h, thresh, .5f, 0, relative, &n);
+    if (nms > 0) do_nms_sort(dets, n, l.classes, nms);
+    for (i = 0; i < n && i < cap; ++i) {
+        float *r = rows + (size_t)i * (5 + l.classes);
+        r[0] = dets[i].bbox.x;
+        r[1] = dets[i].bbox.y;
+        r[2] = dets[i].bbox.w;
+        r[3] = dets[i].bbox.h;
+        r[4] = dets[i].objectness;
+        for (j = 0; j < l.classes; ++j) r[5 + j] = dets[i].prob[j];
+    }
+    free_detections(dets, n);
+    return n;
+}
+
+/* Overwrite a yolo layer's host output (so that decode and NMS can be driven with chosen
+ * tensors without running a network that produces them). */
+void refh_set_output(network *net, int i, const float *values)
+{
+    layer l = net->layers[i];
+    memcpy(l.output, values, sizeof(float) * (size_t)l.outputs * l.batch);
+}
+

@@ -16,6 +16,10 @@ seeded synthetic inputs; nothing from the reference's sources is stored.  Fixtur
   conv_cases.npz         single conv layers (3x3 s1/s2, 1x1, grouped, 7x7) in full
   xnor_case.npz          one xnor conv layer: input, binarised tensors, output
   maxpool_case.npz       maxpool output + indexes incl. the padded stride-1 case
+  detections_case.npz    the two yolo tensors of a yolov3-tiny forward at 96x96 and what
+                         get_network_boxes / do_nms_sort make of them (rows x,y,w,h,obj,prob[80])
+
+`python tests/golden/make_golden.py detections` rewrites only the last one.
 """
 import json
 import os
@@ -112,9 +116,38 @@ num=3
 """
 
 
+def lexsorted(rows):
+    """Rows in a canonical order (the reference leaves its array sorted by the last class after NMS)."""
+    if len(rows) == 0:
+        return rows
+    return rows[np.lexsort(rows[:, :5].T[::-1])]
+
+
+DET_CASES = {"square": (96, 96, 0.5, 1, 0.0), "wide_abs": (200, 120, 0.5, 0, 0.0), "tall_rel": (90, 160, 0.55, 1, 0.0),
+             "wide_abs_nms": (200, 120, 0.25, 0, 0.45), "square_nms": (96, 96, 0.2, 1, 0.3)}
+
+
+def detections_fixture():
+    r, _ = table(cfgs.yolov3_tiny(1, 96))
+    fill_params(r.set_conv, r.layers, seed=1200, bn="random")
+    outs = r.predict(synth.uniform01(17, r.inputs * r.batch))
+    heads = [i for i, L in enumerate(r.layers) if L["type"] == "yolo"]
+    data = {f"yolo{i}": outs[i] for i in heads}
+    for name, (w, h, thresh, relative, nms) in DET_CASES.items():
+        rows = r.get_boxes(w, h, thresh, relative, nms)
+        data[name] = rows if nms == 0 else lexsorted(rows)
+        data[name + "_spec"] = np.array([w, h, thresh, relative, nms], np.float64)
+    np.savez_compressed(os.path.join(HERE, "detections_case.npz"), **data)
+
+
 def main():
     if not ref.available():
         raise SystemExit("oracle/_ref is not built")
+    if sys.argv[1:] == ["detections"]:
+        detections_fixture()
+        print("detections_case.npz written")
+        return
+    detections_fixture()
     # ---- layer tables
     tables = {}
     for name, text in [("yolov3-tiny-416", cfgs.yolov3_tiny(1, 416)), ("yolov3-416", cfgs.yolov3(1, 416)),
