@@ -180,7 +180,7 @@ class Network:
         x = np.ascontiguousarray(x, np.float32)
         assert x.size == self.inputs * self.batch, (x.size, self.inputs, self.batch)
         out = self.L.network_predict(self.net, _fp(x))
-        last = self.layers[-1]
+        last = [L for L in self.layers if L["type"] != "cost"][-1]   # get_network_output_layer
         return np.ctypeslib.as_array(out, shape=(self.batch, last["outputs"])).copy()
 
     def push_input(self, x):

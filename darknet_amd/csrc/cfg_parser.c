@@ -36,6 +36,11 @@ static LAYER_TYPE section_type(const char *t)
     if (!strcmp(t, "[soft]") || !strcmp(t, "[softmax]")) return SOFTMAX;
     if (!strcmp(t, "[route]")) return ROUTE;
     if (!strcmp(t, "[upsample]")) return UPSAMPLE;
+    if (!strcmp(t, "[conn]") || !strcmp(t, "[connected]")) return CONNECTED;
+    if (!strcmp(t, "[dropout]")) return DROPOUT;
+    if (!strcmp(t, "[reorg]")) return REORG;
+    if (!strcmp(t, "[crop]")) return CROP;
+    if (!strcmp(t, "[cost]")) return COST;
     return BLANK;
 }
 
@@ -71,6 +76,11 @@ char *get_layer_string(LAYER_TYPE a)
     case SHORTCUT: return "shortcut";
     case UPSAMPLE: return "upsample";
     case YOLO: return "yolo";
+    case CONNECTED: return "connected";
+    case DROPOUT: return "dropout";
+    case REORG: return "reorg";
+    case CROP: return "crop";
+    case COST: return "cost";
     default: return "none";
     }
 }
@@ -211,6 +221,69 @@ static layer parse_route(cfg_section *o, size_params p, network *net)
     return r;
 }
 
+/* src/parser.c:259-268 */
+static layer parse_connected(cfg_section *o, size_params p)
+{
+    int output = cfg_find_int(o, "output", 1);
+    char *act = cfg_find_str(o, "activation", "logistic");
+    int bn = cfg_find_int_quiet(o, "batch_normalize", 0);
+    if (output < 1 || p.inputs < 1) dn_fatal("connected layer: needs inputs and output >= 1");
+    return make_connected_layer(p.batch, p.inputs, output, get_activation(act), bn, 0);
+}
+
+/* src/parser.c:513-521; the caller aliases the output to the previous layer's (:829-836) */
+static layer parse_dropout(cfg_section *o, size_params p)
+{
+    float probability = cfg_find_float(o, "probability", .5f);
+    layer l = make_dropout_layer(p.batch, p.inputs, probability);
+    l.out_w = p.w;
+    l.out_h = p.h;
+    l.out_c = p.c;
+    return l;
+}
+
+/* src/parser.c:465-481 */
+static layer parse_reorg(cfg_section *o, size_params p)
+{
+    int stride = cfg_find_int(o, "stride", 1);
+    int reverse = cfg_find_int_quiet(o, "reverse", 0);
+    int flatten = cfg_find_int_quiet(o, "flatten", 0);
+    int extra = cfg_find_int_quiet(o, "extra", 0);
+    need_image(p, "reorg");
+    return make_reorg_layer(p.batch, p.w, p.h, p.c, stride, reverse, flatten, extra);
+}
+
+/* src/parser.c:441-463 */
+static layer parse_crop(cfg_section *o, size_params p)
+{
+    int crop_height = cfg_find_int(o, "crop_height", 1);
+    int crop_width = cfg_find_int(o, "crop_width", 1);
+    int flip = cfg_find_int(o, "flip", 0);
+    float angle = cfg_find_float(o, "angle", 0);
+    float saturation = cfg_find_float(o, "saturation", 1);
+    float exposure = cfg_find_float(o, "exposure", 1);
+    int noadjust;
+    layer l;
+    need_image(p, "crop");
+    noadjust = cfg_find_int_quiet(o, "noadjust", 0);
+    l = make_crop_layer(p.batch, p.h, p.w, p.c, crop_height, crop_width, flip, angle, saturation, exposure);
+    l.shift = cfg_find_float(o, "shift", 0);
+    l.noadjust = noadjust;
+    return l;
+}
+
+/* src/parser.c:429-439 */
+static layer parse_cost(cfg_section *o, size_params p)
+{
+    float scale;
+    (void)cfg_find_str(o, "type", "sse");
+    scale = cfg_find_float_quiet(o, "scale", 1);
+    (void)cfg_find_float_quiet(o, "ratio", 0);
+    (void)cfg_find_float_quiet(o, "noobj", 1);
+    (void)cfg_find_float_quiet(o, "thresh", 0);
+    return make_cost_layer(p.batch, p.inputs, 0, scale);
+}
+
 /* src/parser.c:285-342 */
 static layer parse_yolo(cfg_section *o, size_params p)
 {
@@ -306,6 +379,16 @@ network *parse_network_cfg(char *filename)
         case UPSAMPLE: l = parse_upsample(o, p); break;
         case SHORTCUT: l = parse_shortcut(o, p, net); break;
         case YOLO: l = parse_yolo(o, p); break;
+        case CONNECTED: l = parse_connected(o, p); break;
+        case REORG: l = parse_reorg(o, p); break;
+        case CROP: l = parse_crop(o, p); break;
+        case COST: l = parse_cost(o, p); break;
+        case DROPOUT:
+            if (count == 0) dn_fatal("dropout cannot be the first layer");
+            l = parse_dropout(o, p);
+            l.output = net->layers[count - 1].output;
+            l.output_gpu = net->layers[count - 1].output_gpu;
+            break;
         default: {
             char buf[256];
             snprintf(buf, sizeof buf, "layer type %s (section %d) is outside the convolution forward path this "
@@ -329,15 +412,24 @@ network *parse_network_cfg(char *filename)
     }
     cfg_free(f);
     {
-        layer out = get_network_output_layer(net);
+        /* the output layer is the last one that is not a cost layer (src/network.c:689-697); the
+         * host sees its output after every forward (src/network.c:786) */
         layer *last = &net->layers[net->n - 1];
-        net->outputs = out.outputs;
-        net->truths = out.outputs;
+        layer *out = last;
+        for (i = net->n - 1; i >= 0; --i)
+            if (net->layers[i].type != COST) break;
+        if (i < 0) dn_fatal("network has no layers besides cost layers");
+        out = &net->layers[i];
+        net->outputs = out->outputs;
+        net->truths = out->outputs;
         if (last->truths) net->truths = last->truths;
-        /* the host sees the last layer's output after every forward (src/network.c:786) */
-        if (!last->output) last->output = (float *)dn_calloc((size_t)last->outputs * last->batch, sizeof(float));
-        net->output = last->output;
-        net->output_gpu = last->output_gpu;
+        if (!out->output) {
+            out->output = (float *)dn_calloc((size_t)out->outputs * out->batch, sizeof(float));
+            /* a dropout layer behind it shares the buffer (src/parser.c:831) */
+            if (i + 1 < net->n && net->layers[i + 1].type == DROPOUT) net->layers[i + 1].output = out->output;
+        }
+        net->output = out->output;
+        net->output_gpu = out->output_gpu;
     }
     net->input = (float *)dn_calloc((size_t)net->inputs * net->batch, sizeof(float));
     net->input_gpu = hip_make_array(net->input, (size_t)net->inputs * net->batch);

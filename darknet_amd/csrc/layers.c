@@ -369,8 +369,215 @@ void forward_softmax_layer_gpu(layer l, network net)
 }
 
 /* ---- src/layer.c:6-97 ----------------------------------------------------------------------- */
+/* ---- connected: src/connected_layer.c:14-110.  out[b][o] = sum_k in[b][k]*w[o][k] is the 1x1
+ * convolution of a 1x1 image with `inputs` channels, so the layer runs on the convolution
+ * kernel (M = outputs, K = inputs, N = batch) with the same batch-norm / bias / activation
+ * tail (forward_connected_layer :150-167: gemm, forward_batchnorm_layer or add_bias, activate). */
+layer make_connected_layer(int batch, int inputs, int outputs, ACTIVATION activation, int batch_normalize,
+                           int adam)
+{
+    layer l;
+    size_t packed;
+    int i;
+    (void)adam;
+    memset(&l, 0, sizeof l);
+    l.type = CONNECTED;
+    l.inputs = inputs;
+    l.outputs = outputs;
+    l.batch = batch;
+    l.batch_normalize = batch_normalize;
+    l.h = 1;
+    l.w = 1;
+    l.c = inputs;
+    l.out_h = 1;
+    l.out_w = 1;
+    l.out_c = outputs;
+    l.n = outputs;
+    l.size = 1;
+    l.stride = 1;
+    l.groups = 1;
+    l.activation = activation;
+    l.nweights = inputs * outputs;
+    l.nbiases = outputs;
+    if ((long)inputs * outputs >= (1L << 31)) dn_fatal("connected layer: too many weights");
+    l.weights = (float *)dn_calloc((size_t)l.nweights, sizeof(float));
+    l.biases = (float *)dn_calloc((size_t)outputs, sizeof(float));
+    l.forward_gpu = forward_connected_layer_gpu;
+    if (gpu_index < 0) dn_fatal("this library has no CPU path: gpu_index must name a device");
+    l.weights_gpu = hip_make_array(l.weights, (size_t)l.nweights);
+    l.biases_gpu = hip_make_array(l.biases, (size_t)outputs);
+    l.output_gpu = hip_make_array(0, (size_t)batch * outputs);
+    if (batch_normalize) {
+        l.scales = (float *)dn_calloc((size_t)outputs, sizeof(float));
+        for (i = 0; i < outputs; ++i) l.scales[i] = 1;
+        l.rolling_mean = (float *)dn_calloc((size_t)outputs, sizeof(float));
+        l.rolling_variance = (float *)dn_calloc((size_t)outputs, sizeof(float));
+        l.scales_gpu = hip_make_array(l.scales, (size_t)outputs);
+        l.rolling_mean_gpu = hip_make_array(l.rolling_mean, (size_t)outputs);
+        l.rolling_variance_gpu = hip_make_array(l.rolling_variance, (size_t)outputs);
+    }
+    packed = conv_packed_floats(outputs, inputs, 1, 1);
+    if (packed) {
+        l.weights_packed_gpu = hip_make_array(0, packed);
+        conv_pack_weights_gpu(l.weights_gpu, l.weights_packed_gpu, outputs, inputs, 1, 1);
+    }
+    if (dn_verbose) fprintf(stderr, "connected                            %4d  ->  %4d\n", inputs, outputs);
+    return l;
+}
+
+void forward_connected_layer_gpu(layer l, network net)
+{
+    forward_convolutional_gpu(net.input_gpu, l.weights_gpu, l.weights_packed_gpu, l.biases_gpu, l.scales_gpu,
+                              l.rolling_mean_gpu, l.rolling_variance_gpu, l.output_gpu, l.batch, l.inputs, 1, 1,
+                              l.outputs, 1, 1, 1, 0, l.batch_normalize, (int)l.activation);
+}
+
+void push_connected_layer(layer l) { push_convolutional_layer(l); }
+void pull_connected_layer(layer l) { pull_convolutional_layer(l); }
+
+/* ---- dropout: src/dropout_layer.c:7-27.  At inference the layer does nothing
+ * (forward_dropout_layer :38-41); its output IS the previous layer's output, which the cfg
+ * parser wires up as src/parser.c:829-836 does. --------------------------------------------- */
+layer make_dropout_layer(int batch, int inputs, float probability)
+{
+    layer l;
+    memset(&l, 0, sizeof l);
+    l.type = DROPOUT;
+    l.probability = probability;
+    l.inputs = inputs;
+    l.outputs = inputs;
+    l.batch = batch;
+    l.scale = (float)(1. / (1. - probability));
+    l.forward_gpu = forward_dropout_layer_gpu;
+    if (dn_verbose) fprintf(stderr, "dropout       p = %.2f               %4d  ->  %4d\n", probability, inputs, inputs);
+    return l;
+}
+
+void forward_dropout_layer_gpu(layer l, network net)
+{
+    (void)l;
+    (void)net;
+}
+
+/* ---- reorg: src/reorg_layer.c:8-58, forward :88-107 ---------------------------------------- */
+layer make_reorg_layer(int batch, int w, int h, int c, int stride, int reverse, int flatten, int extra)
+{
+    layer l;
+    memset(&l, 0, sizeof l);
+    l.type = REORG;
+    l.batch = batch;
+    l.stride = stride;
+    l.extra = extra;
+    l.h = h;
+    l.w = w;
+    l.c = c;
+    l.flatten = flatten;
+    if (stride < 1) dn_fatal("reorg layer: stride must be at least 1");
+    if (reverse) {
+        l.out_w = w * stride;
+        l.out_h = h * stride;
+        l.out_c = c / (stride * stride);
+    } else {
+        l.out_w = w / stride;
+        l.out_h = h / stride;
+        l.out_c = c * (stride * stride);
+    }
+    l.reverse = reverse;
+    l.outputs = l.out_h * l.out_w * l.out_c;
+    l.inputs = h * w * c;
+    if (l.extra) {
+        l.out_w = l.out_h = l.out_c = 0;
+        l.outputs = l.inputs + l.extra;
+    }
+    if (!extra && !flatten && l.outputs != l.inputs)
+        dn_fatal("reorg layer: stride must divide width and height (and stride*stride the channels when reversed)");
+    if (dn_verbose) {
+        if (extra) fprintf(stderr, "reorg              %4d   ->  %4d\n", l.inputs, l.outputs);
+        else fprintf(stderr, "reorg              /%2d  %4d x%4d x%4d   ->  %4d x%4d x%4d\n", stride, w, h, c, l.out_w,
+                     l.out_h, l.out_c);
+    }
+    l.forward_gpu = forward_reorg_layer_gpu;
+    l.output_gpu = hip_make_array(0, (size_t)l.outputs * batch); /* zero: the `extra` tail stays 0 */
+    return l;
+}
+
+void forward_reorg_layer_gpu(layer l, network net)
+{
+    int i;
+    if (l.flatten) {
+        flatten_gpu(net.input_gpu, l.w * l.h, l.c, l.batch, l.reverse ? 0 : 1, l.output_gpu);
+    } else if (l.extra) {
+        for (i = 0; i < l.batch; ++i)
+            copy_gpu_offset(l.inputs, net.input_gpu, i * l.inputs, 1, l.output_gpu, i * l.outputs, 1);
+    } else if (l.reverse) {
+        reorg_gpu(net.input_gpu, l.w, l.h, l.c, l.batch, l.stride, 1, l.output_gpu);
+    } else {
+        reorg_gpu(net.input_gpu, l.w, l.h, l.c, l.batch, l.stride, 0, l.output_gpu);
+    }
+}
+
+/* ---- crop: src/crop_layer.c:18-51; inference takes the centred window ---------------------- */
+layer make_crop_layer(int batch, int h, int w, int c, int crop_height, int crop_width, int flip, float angle,
+                      float saturation, float exposure)
+{
+    layer l;
+    (void)angle;
+    (void)saturation;
+    (void)exposure;
+    memset(&l, 0, sizeof l);
+    if (dn_verbose) fprintf(stderr, "Crop Layer: %d x %d -> %d x %d x %d image\n", h, w, crop_height, crop_width, c);
+    if (crop_height > h || crop_width > w || crop_height < 1 || crop_width < 1)
+        dn_fatal("crop layer: the window must fit inside the input");
+    l.type = CROP;
+    l.batch = batch;
+    l.h = h;
+    l.w = w;
+    l.c = c;
+    l.scale = (float)crop_height / h;
+    l.flip = flip;
+    l.out_w = crop_width;
+    l.out_h = crop_height;
+    l.out_c = c;
+    l.inputs = l.w * l.h * l.c;
+    l.outputs = l.out_w * l.out_h * l.out_c;
+    l.forward_gpu = forward_crop_layer_gpu;
+    l.output_gpu = hip_make_array(0, (size_t)l.outputs * batch);
+    return l;
+}
+
+void forward_crop_layer_gpu(layer l, network net)
+{
+    forward_crop_gpu(net.input_gpu, l.output_gpu, l.batch, l.c, l.h, l.w, l.out_h, l.out_w, l.noadjust);
+}
+
+/* ---- cost: src/cost_layer.c:40-63.  Without a truth the forward returns at once (:79); the
+ * layer only has to exist so that cfgs ending in [cost] parse, and is skipped when the
+ * network's output layer is looked up (src/network.c:689-697). ------------------------------- */
+layer make_cost_layer(int batch, int inputs, int cost_type, float scale)
+{
+    layer l;
+    (void)cost_type;
+    memset(&l, 0, sizeof l);
+    if (dn_verbose) fprintf(stderr, "cost                                           %4d\n", inputs);
+    l.type = COST;
+    l.scale = scale;
+    l.batch = batch;
+    l.inputs = inputs;
+    l.outputs = inputs;
+    l.forward_gpu = forward_cost_layer_gpu;
+    l.output_gpu = hip_make_array(0, (size_t)inputs * batch);
+    return l;
+}
+
+void forward_cost_layer_gpu(layer l, network net)
+{
+    (void)l;
+    (void)net;
+}
+
 void free_layer(layer l)
 {
+    if (l.type == DROPOUT) return; /* its buffers belong to the layer before it (src/layer.c:8-14) */
     free(l.mask);
     free(l.input_layers);
     free(l.input_sizes);

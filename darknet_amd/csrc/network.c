@@ -224,8 +224,8 @@ void network_set_conv(network *net, int i, const float *weights, const float *bi
                       const float *rolling_mean, const float *rolling_variance)
 {
     layer l;
-    if (i < 0 || i >= net->n || net->layers[i].type != CONVOLUTIONAL)
-        dn_fatal("network_set_conv: not a convolutional layer");
+    if (i < 0 || i >= net->n || (net->layers[i].type != CONVOLUTIONAL && net->layers[i].type != CONNECTED))
+        dn_fatal("network_set_conv: not a convolutional or connected layer");
     l = net->layers[i];
     if (weights) memcpy(l.weights, weights, sizeof(float) * (size_t)l.nweights);
     if (biases) memcpy(l.biases, biases, sizeof(float) * (size_t)l.n);
@@ -305,7 +305,7 @@ int network_route_inputs(network *net, int i, int *layers, int *sizes, int cap)
     return l.n;
 }
 
-/* numops of the reference (examples/darknet.c:81-114), convolution term only */
+/* numops of the reference (examples/darknet.c:81-114): the convolutional and connected terms */
 double network_conv_flops(network *net)
 {
     double ops = 0;
@@ -314,6 +314,8 @@ double network_conv_flops(network *net)
         layer l = net->layers[i];
         if (l.type == CONVOLUTIONAL)
             ops += 2.0 * l.n * l.size * l.size * (l.c / l.groups) * l.out_h * l.out_w;
+        else if (l.type == CONNECTED)
+            ops += 2.0 * l.inputs * l.outputs;
     }
     return ops;
 }

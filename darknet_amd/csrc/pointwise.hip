@@ -403,3 +403,86 @@ extern "C" void binarize_weights_gpu(float *weights, int n, int size, float *bin
                        (const float *)weights, n, size, binary);
     dn_check_launch("binarize_weights_gpu");
 }
+
+/* ---- reorg / flatten / crop: pure index work, bit-exact ------------------------------------ */
+/* reorg_cpu of src/blas.c:9-30 (same argument meaning as reorg_gpu, src/blas.h:73): thread i
+ * walks the (b, k, j, i) space of the c x h x w tensor x is described with; `forward` copies
+ * x[in_index] to out[out_index], otherwise out[in_index] = x[out_index]. */
+__global__ void reorg_kernel(const float *x, float *out, long n, int w, int h, int c, int stride, int forward)
+{
+    const int out_c = c / (stride * stride);
+    for (long id = blockIdx.x * (long)blockDim.x + threadIdx.x; id < n; id += (long)gridDim.x * blockDim.x) {
+        const int i = (int)(id % w);
+        long t = id / w;
+        const int j = (int)(t % h);
+        t /= h;
+        const int k = (int)(t % c);
+        const long b = t / c;
+        const int c2 = k % out_c;
+        const int offset = k / out_c;
+        const int w2 = i * stride + offset % stride;
+        const int h2 = j * stride + offset / stride;
+        const long out_index = w2 + (long)w * stride * (h2 + (long)h * stride * (c2 + (long)out_c * b));
+        if (forward) out[out_index] = x[id];
+        else out[id] = x[out_index];
+    }
+}
+
+extern "C" void reorg_gpu(float *x, int w, int h, int c, int batch, int stride, int forward, float *out)
+{
+    if (w <= 0 || h <= 0 || c <= 0 || batch <= 0 || stride <= 0) dn_fatal("reorg_gpu: bad geometry");
+    if (c % (stride * stride)) dn_fatal("reorg_gpu: stride*stride must divide the channel count");
+    const long n = (long)w * h * c * batch;
+    hipLaunchKernelGGL(reorg_kernel, dim3(dn_blocks(n)), dim3(DN_BLOCK), 0, dn_stream(), x, out, n, w, h, c, stride,
+                       forward);
+    dn_check_launch("reorg_gpu");
+}
+
+/* flatten of src/blas.c:32-49, out of place: [b][layers][spatial] <-> [b][spatial][layers] */
+__global__ void flatten_kernel(const float *x, float *out, long n, int spatial, int layers, int forward)
+{
+    for (long id = blockIdx.x * (long)blockDim.x + threadIdx.x; id < n; id += (long)gridDim.x * blockDim.x) {
+        const int i = (int)(id % spatial);
+        long t = id / spatial;
+        const int cc = (int)(t % layers);
+        const long b = t / layers;
+        const long i1 = b * layers * spatial + (long)cc * spatial + i;
+        const long i2 = b * layers * spatial + (long)i * layers + cc;
+        if (forward) out[i2] = x[i1];
+        else out[i1] = x[i2];
+    }
+}
+
+extern "C" void flatten_gpu(float *x, int spatial, int layers, int batch, int forward, float *out)
+{
+    if (spatial <= 0 || layers <= 0 || batch <= 0) dn_fatal("flatten_gpu: bad geometry");
+    const long n = (long)spatial * layers * batch;
+    hipLaunchKernelGGL(flatten_kernel, dim3(dn_blocks(n)), dim3(DN_BLOCK), 0, dn_stream(), x, out, n, spatial,
+                       layers, forward);
+    dn_check_launch("flatten_gpu");
+}
+
+/* forward_crop_layer at inference (src/crop_layer.c:67-103 with net.train == 0): the centred
+ * window, then value*scale + trans in two float roundings (scale 2, trans -1 unless noadjust) */
+__global__ void crop_kernel(const float *in, float *out, long n, int c, int h, int w, int oh, int ow, int dh,
+                            int dw, float scale, float trans)
+{
+    for (long id = blockIdx.x * (long)blockDim.x + threadIdx.x; id < n; id += (long)gridDim.x * blockDim.x) {
+        const int j = (int)(id % ow);
+        long t = id / ow;
+        const int i = (int)(t % oh);
+        const long plane = t / oh; /* b*c + k */
+        out[id] = __fadd_rn(__fmul_rn(in[(j + dw) + (long)w * ((i + dh) + (long)h * plane)], scale), trans);
+    }
+}
+
+extern "C" void forward_crop_gpu(const float *input, float *output, int batch, int c, int h, int w, int out_h,
+                                 int out_w, int noadjust)
+{
+    if (batch <= 0 || c <= 0 || h <= 0 || w <= 0 || out_h <= 0 || out_w <= 0 || out_h > h || out_w > w)
+        dn_fatal("forward_crop_gpu: bad geometry");
+    const long n = (long)batch * c * out_h * out_w;
+    hipLaunchKernelGGL(crop_kernel, dim3(dn_blocks(n)), dim3(DN_BLOCK), 0, dn_stream(), input, output, n, c, h, w,
+                       out_h, out_w, (h - out_h) / 2, (w - out_w) / 2, noadjust ? 1.f : 2.f, noadjust ? 0.f : -1.f);
+    dn_check_launch("forward_crop_gpu");
+}

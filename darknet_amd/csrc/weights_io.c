@@ -5,8 +5,9 @@
  * major, minor, revision; then `seen` as size_t when major*10+minor >= 2 (and both < 1000),
  * else as int; then, per layer in order, for a convolutional layer: biases[n]; if
  * batch_normalize (and not dontloadscales) scales[n], rolling_mean[n], rolling_variance[n];
- * weights[nweights] (src/parser.c:958-977, :1164-1215).  Other layer types on this path carry
- * no parameters.  A load ends in push_convolutional_layer, which also refreshes the packed copy
+ * weights[nweights] (src/parser.c:958-977, :1164-1215); for a connected layer: biases[outputs],
+ * weights[outputs*inputs], then the batch-norm vectors (:991-1005, :1098-1120).  Other layer
+ * types on this path carry no parameters.  A load ends in push_convolutional_layer, which also refreshes the packed copy
  * the MFMA kernel reads.
  */
 #include <stdio.h>
@@ -57,10 +58,25 @@ static void load_convolutional_weights(layer l, FILE *fp)
     push_convolutional_layer(l);
 }
 
+/* src/parser.c:1098-1120: biases, weights (transposed when the file says so), then the
+ * batch-norm vectors - note the order differs from the convolutional layer's */
+static void load_connected_weights(layer l, FILE *fp, int transpose)
+{
+    read_floats(l.biases, (size_t)l.outputs, fp, "connected biases");
+    read_floats(l.weights, (size_t)l.outputs * l.inputs, fp, "connected weights");
+    if (transpose) transpose_matrix(l.weights, l.inputs, l.outputs);
+    if (l.batch_normalize && !l.dontloadscales) {
+        read_floats(l.scales, (size_t)l.outputs, fp, "connected scales");
+        read_floats(l.rolling_mean, (size_t)l.outputs, fp, "connected rolling_mean");
+        read_floats(l.rolling_variance, (size_t)l.outputs, fp, "connected rolling_variance");
+    }
+    push_connected_layer(l);
+}
+
 void load_weights_upto(network *net, char *filename, int start, int cutoff)
 {
     FILE *fp;
-    int major, minor, revision, i;
+    int major, minor, revision, i, transpose;
     hip_set_device(net->gpu_index);
     if (dn_verbose) fprintf(stderr, "Loading weights from %s...", filename);
     fp = fopen(filename, "rb");
@@ -75,10 +91,12 @@ void load_weights_upto(network *net, char *filename, int start, int cutoff)
         if (fread(&iseen, sizeof(int), 1, fp) != 1) dn_fatal("weights file is shorter than its header");
         *net->seen = (size_t)iseen;
     }
+    transpose = (major > 1000) || (minor > 1000); /* src/parser.c:1246 */
     for (i = start; i < net->n && i < cutoff; ++i) {
         layer l = net->layers[i];
         if (l.dontload) continue;
         if (l.type == CONVOLUTIONAL) load_convolutional_weights(l, fp);
+        if (l.type == CONNECTED) load_connected_weights(l, fp, transpose);
     }
     if (dn_verbose) fprintf(stderr, "Done!\n");
     fclose(fp);
@@ -103,6 +121,17 @@ void save_weights_upto(network *net, char *filename, int cutoff)
     fwrite(net->seen, sizeof(size_t), 1, fp);
     for (i = 0; i < net->n && i < cutoff; ++i) {
         layer l = net->layers[i];
+        if (l.type == CONNECTED) { /* src/parser.c:991-1005 */
+            pull_connected_layer(l);
+            fwrite(l.biases, sizeof(float), (size_t)l.outputs, fp);
+            fwrite(l.weights, sizeof(float), (size_t)l.outputs * l.inputs, fp);
+            if (l.batch_normalize) {
+                fwrite(l.scales, sizeof(float), (size_t)l.outputs, fp);
+                fwrite(l.rolling_mean, sizeof(float), (size_t)l.outputs, fp);
+                fwrite(l.rolling_variance, sizeof(float), (size_t)l.outputs, fp);
+            }
+            continue;
+        }
         if (l.type != CONVOLUTIONAL) continue;
         pull_convolutional_layer(l);
         fwrite(l.biases, sizeof(float), (size_t)l.n, fp);

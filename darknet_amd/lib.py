@@ -64,6 +64,8 @@ SIGNATURES = {
     "save_weights": (None, [V, C.c_char_p]), "save_weights_upto": (None, [V, C.c_char_p, i]),
     "get_activation": (i, [C.c_char_p]), "get_activation_string": (C.c_char_p, [i]),
     "get_layer_string": (C.c_char_p, [i]),
+    "reorg_gpu": (None, [V, i, i, i, i, i, i, V]), "flatten_gpu": (None, [V, i, i, i, i, V]),
+    "forward_crop_gpu": (None, [V, V, i, i, i, i, i, i, i]),
     "yolo_decode_gpu": (None, [V, i, i, i, i, F, i, i, i, i, i, f, V, i, V]),
     "nms_sort_gpu": (None, [V, i, i, f]),
     "num_detections": (i, [V, f]), "make_network_boxes": (V, [V, f, I]),
@@ -94,6 +96,9 @@ STRUCT_BY_VALUE = [
     "forward_shortcut_layer_gpu", "forward_upsample_layer_gpu", "forward_yolo_layer_gpu",
     "forward_avgpool_layer_gpu", "forward_softmax_layer_gpu", "push_convolutional_layer",
     "pull_convolutional_layer", "get_network_output_layer",
+    "make_connected_layer", "make_dropout_layer", "make_reorg_layer", "make_crop_layer", "make_cost_layer",
+    "forward_connected_layer_gpu", "forward_dropout_layer_gpu", "forward_reorg_layer_gpu",
+    "forward_crop_layer_gpu", "forward_cost_layer_gpu", "push_connected_layer", "pull_connected_layer",
 ]
 
 _lib = None

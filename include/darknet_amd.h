@@ -88,6 +88,12 @@ struct layer {
     float ignore_thresh;
     float truth_thresh;
     int random;
+    int flatten;       /* reorg */
+    int extra;
+    int noadjust;      /* crop */
+    int flip;
+    float probability; /* dropout */
+    float shift;
 
     int *input_layers;
     int *input_sizes;
@@ -192,6 +198,14 @@ layer make_upsample_layer(int batch, int w, int h, int c, int stride); /* src/up
 layer make_yolo_layer(int batch, int w, int h, int n, int total, int *mask,
                       int classes);                       /* src/yolo_layer.c:13 */
 layer make_avgpool_layer(int batch, int w, int h, int c); /* src/avgpool_layer.c:5 */
+layer make_connected_layer(int batch, int inputs, int outputs, ACTIVATION activation,
+                           int batch_normalize, int adam); /* src/connected_layer.c:14 */
+layer make_dropout_layer(int batch, int inputs, float probability); /* src/dropout_layer.c:7 */
+layer make_reorg_layer(int batch, int w, int h, int c, int stride, int reverse, int flatten,
+                       int extra);                        /* src/reorg_layer.c:8 */
+layer make_crop_layer(int batch, int h, int w, int c, int crop_height, int crop_width, int flip,
+                      float angle, float saturation, float exposure); /* src/crop_layer.c:18 */
+layer make_cost_layer(int batch, int inputs, int cost_type, float scale); /* src/cost_layer.c:40 */
 layer make_softmax_layer(int batch, int inputs, int groups); /* src/softmax_layer.c:11 */
 void free_layer(layer l);                                 /* src/layer.c:6 */
 
@@ -204,6 +218,13 @@ void forward_upsample_layer_gpu(layer l, network net);      /* src/upsample_laye
 void forward_yolo_layer_gpu(layer l, network net);          /* src/yolo_layer.c:347 */
 void forward_avgpool_layer_gpu(layer l, network net);       /* src/avgpool_layer_kernels.cu:46 */
 void forward_softmax_layer_gpu(layer l, network net);       /* src/softmax_layer.c:71 */
+void forward_connected_layer_gpu(layer l, network net);     /* src/connected_layer.c:286 */
+void forward_dropout_layer_gpu(layer l, network net);       /* src/dropout_layer_kernels.cu:17 (inference: nothing) */
+void forward_reorg_layer_gpu(layer l, network net);         /* src/reorg_layer.c:149 */
+void forward_crop_layer_gpu(layer l, network net);          /* src/crop_layer_kernels.cu:183 */
+void forward_cost_layer_gpu(layer l, network net);          /* src/cost_layer.c:120 (no truth: nothing) */
+void push_connected_layer(layer l);                         /* src/connected_layer.c:268 */
+void pull_connected_layer(layer l);                         /* src/connected_layer.c:254 */
 void push_convolutional_layer(layer l);                     /* src/convolutional_kernels.cu:286 */
 void pull_convolutional_layer(layer l);                     /* src/convolutional_kernels.cu:270 */
 

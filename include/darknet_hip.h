@@ -195,6 +195,16 @@ void forward_yolo_gpu(const float *input, float *output, int batch, int w, int h
 /* forward_avgpool_layer_gpu (src/avgpool_layer_kernels.cu:46-54). */
 void forward_avgpool_gpu(const float *input, float *output, int batch, int c, int h, int w);
 
+/* reorg_gpu / flatten_gpu (src/blas.h:73-74, CPU forms src/blas.c:9-49): the index permutations
+ * of the reorg layer.  (w,h,c) describe the tensor whose flat index the loop walks; `forward`
+ * != 0 scatters x[walk] to out[permuted], 0 gathers out[walk] = x[permuted]; flatten_gpu writes
+ * to `out` instead of permuting in place.  forward_crop_gpu: forward_crop_layer at inference
+ * (src/crop_layer.c:67-103 with net.train == 0): centred window, value*2-1 unless noadjust. */
+void reorg_gpu(float *x, int w, int h, int c, int batch, int stride, int forward, float *out);
+void flatten_gpu(float *x, int spatial, int layers, int batch, int forward, float *out);
+void forward_crop_gpu(const float *input, float *output, int batch, int c, int h, int w, int out_h,
+                      int out_w, int noadjust);
+
 /* ------------------------------------------------------------------------------------------
  * Detections: the step right after the forward pass.  A detection is a row of (5 + classes)
  * floats in device memory: x, y, w, h, objectness, prob[classes].

@@ -21,6 +21,8 @@ SECTION_ALIASES = {
     "[avg]": "avgpool", "[avgpool]": "avgpool",
     "[soft]": "softmax", "[softmax]": "softmax",
     "[route]": "route", "[shortcut]": "shortcut", "[upsample]": "upsample", "[yolo]": "yolo",
+    "[conn]": "connected", "[connected]": "connected", "[dropout]": "dropout", "[reorg]": "reorg",
+    "[crop]": "crop", "[cost]": "cost",
     "[net]": "net", "[network]": "net",
 }
 
@@ -105,6 +107,36 @@ def parse(text: str) -> dict:
             L.update(groups=gi(o, "groups", 1), temperature=gf(o, "temperature", 1.0),
                      out_h=0, out_w=0, out_c=0, outputs=inputs)
             # parse_softmax sets l.w/h/c from params but leaves out_* at zero
+        elif kind == "connected":
+            # parse_connected src/parser.c:259-268, make_connected_layer src/connected_layer.c:14-33
+            outputs = gi(o, "output", 1)
+            L.update(n=outputs, size=1, stride=1, pad=0, groups=1, h=1, w=1, c=inputs,
+                     activation=o.get("activation", "logistic"),
+                     batch_normalize=gi(o, "batch_normalize", 0), binary=0, xnor=0,
+                     out_h=1, out_w=1, out_c=outputs, outputs=outputs, nweights=inputs * outputs)
+        elif kind == "dropout":
+            # parse_dropout src/parser.c:513-521: geometry passes through, output = input
+            L.update(probability=gf(o, "probability", 0.5), out_h=h, out_w=w, out_c=c, outputs=inputs,
+                     h=0, w=0, c=0)
+        elif kind == "cost":
+            L.update(out_h=0, out_w=0, out_c=0, outputs=inputs, h=0, w=0, c=0)
+        elif kind == "crop":
+            # parse_crop src/parser.c:441-463, make_crop_layer src/crop_layer.c:18-51
+            ch, cw = gi(o, "crop_height", 1), gi(o, "crop_width", 1)
+            L.update(out_h=ch, out_w=cw, out_c=c, noadjust=gi(o, "noadjust", 0), flip=gi(o, "flip", 0),
+                     inputs=h * w * c)
+        elif kind == "reorg":
+            # parse_reorg src/parser.c:465-481, make_reorg_layer src/reorg_layer.c:8-35
+            stride = gi(o, "stride", 1)
+            reverse, flat, extra = gi(o, "reverse", 0), gi(o, "flatten", 0), gi(o, "extra", 0)
+            if reverse:
+                oh, ow, oc = h * stride, w * stride, c // (stride * stride)
+            else:
+                oh, ow, oc = h // stride, w // stride, c * stride * stride
+            L.update(stride=stride, reverse=reverse, flatten=flat, extra=extra, out_h=oh, out_w=ow, out_c=oc,
+                     inputs=h * w * c, outputs=oh * ow * oc)
+            if extra:
+                L.update(out_h=0, out_w=0, out_c=0, outputs=h * w * c + extra)
         elif kind == "upsample":
             stride = gi(o, "stride", 2)
             L.update(stride=stride, scale=gf(o, "scale", 1.0),

@@ -176,6 +176,51 @@ class Oracle:
         self.lib.orc_yolo(_fp(x), _fp(out), b, w, h, n_anchors, classes)
         return out
 
+    def connected(self, x, weights, biases, scales=None, mean=None, var=None, *, outputs, batch_normalize=0,
+                  activation="logistic"):
+        x = np.ascontiguousarray(x, np.float32)
+        b, inputs = x.shape
+        out = np.empty((b, outputs), np.float32)
+        wt = np.ascontiguousarray(weights, np.float32)
+        assert wt.size == inputs * outputs
+        bi = np.ascontiguousarray(biases, np.float32)
+        bn = [None if a is None else np.ascontiguousarray(a, np.float32) for a in (scales, mean, var)]
+        self.lib.orc_connected_forward(_fp(x), _fp(wt), _fp(bi), _opt(bn[0]), _opt(bn[1]), _opt(bn[2]), _fp(out),
+                                       b, inputs, outputs, int(batch_normalize), ACTIVATIONS.index(activation))
+        return out
+
+    def reorg(self, x, w, h, c, batch, stride, forward):
+        """reorg_cpu on a flat array with the reference's own argument meaning."""
+        x = np.ascontiguousarray(x, np.float32)
+        out = np.zeros_like(x)
+        self.lib.orc_reorg(_fp(x), w, h, c, batch, stride, int(forward), _fp(out))
+        return out
+
+    def flatten(self, x, size, layers, batch, forward):
+        x = np.ascontiguousarray(x, np.float32)
+        out = np.zeros_like(x)
+        self.lib.orc_flatten(_fp(x), size, layers, batch, int(forward), _fp(out))
+        return out
+
+    def reorg_layer(self, x, stride, reverse=0, flatten=0, extra=0):
+        """forward_reorg_layer (src/reorg_layer.c:88-107) on x [b, c, h, w] -> [b, outputs]."""
+        x = np.ascontiguousarray(x, np.float32)
+        b, c, h, w = x.shape
+        if flatten:
+            return self.flatten(x, w * h, c, b, 0 if reverse else 1).reshape(b, -1)
+        if extra:
+            out = np.zeros((b, c * h * w + extra), np.float32)
+            out[:, :c * h * w] = x.reshape(b, -1)
+            return out
+        return self.reorg(x, w, h, c, b, stride, 1 if reverse else 0).reshape(b, -1)
+
+    def crop(self, x, out_h, out_w, noadjust=0):
+        x = np.ascontiguousarray(x, np.float32)
+        b, c, h, w = x.shape
+        out = np.empty((b, c, out_h, out_w), np.float32)
+        self.lib.orc_crop(_fp(x), _fp(out), b, c, h, w, out_h, out_w, int(noadjust))
+        return out
+
     def yolo_detections(self, pred, n_anchors, classes, biases, mask, netw, neth, w, h, relative, thresh):
         """get_yolo_detections on image 0 of `pred` [n*(5+classes), lh, lw] -> rows [count, 5+classes]."""
         pred = np.ascontiguousarray(pred, np.float32)

@@ -52,6 +52,19 @@ class OracleNet:
             return o.avgpool(x.reshape(b, L["c"], L["h"], L["w"]))
         if t == "softmax":
             return o.softmax(x.reshape(b, -1), L["groups"], L["temperature"])
+        if t == "connected":
+            w, bi, sc, mu, var = self.params[i]
+            return o.connected(x.reshape(b, -1), w, bi, sc, mu, var, outputs=L["outputs"],
+                               batch_normalize=L["batch_normalize"], activation=L["activation"])
+        if t == "dropout":
+            return x                                   # forward_dropout_layer returns at once when not training
+        if t == "cost":
+            return np.zeros((b, L["outputs"]), np.float32)   # no truth: the output buffer is never written
+        if t == "crop":
+            return o.crop(x.reshape(b, L["c"], L["h"], L["w"]), L["out_h"], L["out_w"], L["noadjust"])
+        if t == "reorg":
+            return o.reorg_layer(x.reshape(b, L["c"], L["h"], L["w"]), L["stride"], L["reverse"], L["flatten"],
+                                 L["extra"])
         raise NotImplementedError(t)
 
     def forward(self, x, upto=None):

@@ -533,3 +533,81 @@ void orc_nms_sort(float *rows, int total, int classes, float thresh)
     }
     free(keys);
 }
+
+/* ---- forward_connected_layer: src/connected_layer.c:150-167.  gemm(0,1,...) = gemm_nt
+ * (src/gemm.c:91-107): a register sum over k per output, added to the zero-filled output; then
+ * forward_batchnorm_layer (out_c = outputs, 1x1 spatial) or add_bias, then the activation. --- */
+void orc_connected_forward(const float *input, const float *weights, const float *biases,
+                           const float *scales, const float *rolling_mean,
+                           const float *rolling_variance, float *output, int batch, int inputs,
+                           int outputs, int batch_normalize, int activation)
+{
+    memset(output, 0, sizeof(float) * (size_t)batch * outputs);
+#pragma omp parallel for
+    for (int i = 0; i < batch; ++i)
+        for (int j = 0; j < outputs; ++j) {
+            float sum = 0;
+            for (int k = 0; k < inputs; ++k) sum += 1.f * input[(long)i * inputs + k] * weights[(long)j * inputs + k];
+            output[(long)i * outputs + j] += sum;
+        }
+    if (batch_normalize) {
+        orc_normalize(output, rolling_mean, rolling_variance, batch, outputs, 1);
+        orc_scale_bias(output, scales, batch, outputs, 1);
+        orc_add_bias(output, biases, batch, outputs, 1);
+    } else {
+        orc_add_bias(output, biases, batch, outputs, 1);
+    }
+    orc_activate_array(output, (long)outputs * batch, activation);
+}
+
+/* ---- reorg_cpu: src/blas.c:9-30 ------------------------------------------------------------ */
+void orc_reorg(const float *x, int w, int h, int c, int batch, int stride, int forward, float *out)
+{
+    const int out_c = c / (stride * stride);
+    for (int b = 0; b < batch; ++b)
+        for (int k = 0; k < c; ++k)
+            for (int j = 0; j < h; ++j)
+                for (int i = 0; i < w; ++i) {
+                    const long in_index = i + (long)w * (j + (long)h * (k + (long)c * b));
+                    const int c2 = k % out_c;
+                    const int offset = k / out_c;
+                    const int w2 = i * stride + offset % stride;
+                    const int h2 = j * stride + offset / stride;
+                    const long out_index = w2 + (long)w * stride * (h2 + (long)h * stride * (c2 + (long)out_c * b));
+                    if (forward) out[out_index] = x[in_index];
+                    else out[in_index] = x[out_index];
+                }
+}
+
+/* ---- flatten: src/blas.c:32-49 (out of place here) ----------------------------------------- */
+void orc_flatten(const float *x, int size, int layers, int batch, int forward, float *out)
+{
+    for (int b = 0; b < batch; ++b)
+        for (int c = 0; c < layers; ++c)
+            for (int i = 0; i < size; ++i) {
+                const long i1 = (long)b * layers * size + (long)c * size + i;
+                const long i2 = (long)b * layers * size + (long)i * layers + c;
+                if (forward) out[i2] = x[i1];
+                else out[i1] = x[i2];
+            }
+}
+
+/* ---- forward_crop_layer with net.train == 0: src/crop_layer.c:67-103 ----------------------- */
+void orc_crop(const float *input, float *output, int batch, int c, int h, int w, int out_h, int out_w,
+              int noadjust)
+{
+    const int dh = (h - out_h) / 2, dw = (w - out_w) / 2;
+    float scale = 2, trans = -1;
+    long count = 0;
+    if (noadjust) {
+        scale = 1;
+        trans = 0;
+    }
+    for (int b = 0; b < batch; ++b)
+        for (int k = 0; k < c; ++k)
+            for (int i = 0; i < out_h; ++i)
+                for (int j = 0; j < out_w; ++j) {
+                    const long index = (j + dw) + (long)w * ((i + dh) + (long)h * (k + (long)c * b));
+                    output[count++] = input[index] * scale + trans;
+                }
+}

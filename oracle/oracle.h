@@ -69,6 +69,15 @@ void orc_avgpool(const float *input, float *output, int batch, int c, int h, int
 void orc_softmax(const float *input, int n, int batch, int batch_offset, int groups,
                  int group_offset, int stride, float temp, float *output);
 
+void orc_connected_forward(const float *input, const float *weights, const float *biases,
+                           const float *scales, const float *rolling_mean,
+                           const float *rolling_variance, float *output, int batch, int inputs,
+                           int outputs, int batch_normalize, int activation);
+void orc_reorg(const float *x, int w, int h, int c, int batch, int stride, int forward, float *out);
+void orc_flatten(const float *x, int size, int layers, int batch, int forward, float *out);
+void orc_crop(const float *input, float *output, int batch, int c, int h, int w, int out_h, int out_w,
+              int noadjust);
+
 /* detections (test infrastructure like everything here): see oracle.c */
 int orc_yolo_detections(const float *pred, int lw, int lh, int n, int classes, const float *biases,
                         const int *mask, int netw, int neth, int w, int h, int relative, float thresh,

@@ -59,6 +59,7 @@ class RefNet:
         H.refh_route_inputs.argtypes = [C.c_void_p, C.c_int, _I, _I, C.c_int]
         H.refh_yolo_mask.argtypes = [C.c_void_p, C.c_int, _I, C.c_int, _F, C.c_int]
         H.refh_set_conv.argtypes = [C.c_void_p, C.c_int] + [_F] * 5
+        H.refh_set_connected.argtypes = [C.c_void_p, C.c_int] + [_F] * 5
         H.refh_predict.restype = _F
         H.refh_predict.argtypes = [C.c_void_p, _F]
         for f in ("refh_layer_output", "refh_layer_weights", "refh_layer_binary_weights",
@@ -102,7 +103,8 @@ class RefNet:
 
     def set_conv(self, i, weights, biases, scales=None, mean=None, var=None):
         p = lambda a: None if a is None else np.ascontiguousarray(a, np.float32).ctypes.data_as(_F)
-        self.h.refh_set_conv(self.net, i, p(weights), p(biases), p(scales), p(mean), p(var))
+        f = self.h.refh_set_connected if self.layers[i]["type"] == "connected" else self.h.refh_set_conv
+        f(self.net, i, p(weights), p(biases), p(scales), p(mean), p(var))
 
     def set_output(self, i, values):
         """Overwrite layer i's host output (drives get_boxes with chosen yolo tensors)."""

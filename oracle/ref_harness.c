@@ -107,6 +107,20 @@ void refh_set_conv(network *net, int i, const float *weights, const float *biase
     }
 }
 
+/* The same for a connected layer (its parameter vectors are sized by outputs / inputs). */
+void refh_set_connected(network *net, int i, const float *weights, const float *biases,
+                        const float *scales, const float *mean, const float *variance)
+{
+    layer l = net->layers[i];
+    if (weights) memcpy(l.weights, weights, sizeof(float) * (size_t)l.inputs * l.outputs);
+    if (biases) memcpy(l.biases, biases, sizeof(float) * (size_t)l.outputs);
+    if (l.batch_normalize) {
+        if (scales) memcpy(l.scales, scales, sizeof(float) * (size_t)l.outputs);
+        if (mean) memcpy(l.rolling_mean, mean, sizeof(float) * (size_t)l.outputs);
+        if (variance) memcpy(l.rolling_variance, variance, sizeof(float) * (size_t)l.outputs);
+    }
+}
+
 float *refh_predict(network *net, float *input)
 {
     return network_predict(net, input);

@@ -16,10 +16,12 @@ seeded synthetic inputs; nothing from the reference's sources is stored.  Fixtur
   conv_cases.npz         single conv layers (3x3 s1/s2, 1x1, grouped, 7x7) in full
   xnor_case.npz          one xnor conv layer: input, binarised tensors, output
   maxpool_case.npz       maxpool output + indexes incl. the padded stride-1 case
+  small_net2.cfg/.weights/.npz  the same for a network of crop, reorg (plain, reverse, flatten,
+                         extra), dropout, connected (with and without batch-norm), softmax, cost
   detections_case.npz    the two yolo tensors of a yolov3-tiny forward at 96x96 and what
                          get_network_boxes / do_nms_sort make of them (rows x,y,w,h,obj,prob[80])
 
-`python tests/golden/make_golden.py detections` rewrites only the last one.
+`python tests/golden/make_golden.py detections|small_net2` rewrites only that fixture.
 """
 import json
 import os
@@ -116,6 +118,85 @@ num=3
 """
 
 
+SMALL_NET2 = """[net]
+batch=2
+subdivisions=1
+width=24
+height=20
+channels=3
+
+[crop]
+crop_height=16
+crop_width=16
+flip=0
+
+[convolutional]
+batch_normalize=1
+filters=16
+size=3
+stride=1
+pad=1
+activation=leaky
+
+[reorg]
+stride=2
+
+[convolutional]
+filters=8
+size=1
+stride=1
+activation=relu
+
+[reorg]
+stride=2
+reverse=1
+
+[reorg]
+stride=1
+flatten=1
+
+[dropout]
+probability=.5
+
+[connected]
+output=40
+batch_normalize=1
+activation=leaky
+
+[dropout]
+probability=.3
+
+[connected]
+output=10
+activation=linear
+
+[reorg]
+extra=3
+stride=1
+
+[softmax]
+
+[cost]
+type=sse
+"""
+
+
+def small_net2_fixture():
+    """crop, reorg (all four modes), dropout, connected (with and without batch-norm), cost."""
+    open(os.path.join(HERE, "small_net2.cfg"), "w").write(SMALL_NET2)
+    r = ref.RefNet(os.path.join(HERE, "small_net2.cfg"))
+    fill_params(r.set_conv, r.layers, seed=640, bn="random")
+    import ctypes as C
+    lib = ref.raw()
+    lib.save_weights.argtypes = [C.c_void_p, C.c_char_p]
+    lib.save_weights(r.net, os.path.join(HERE, "small_net2.weights").encode())
+    x = synth.uniform01(13, r.inputs * r.batch)
+    outs = r.predict(x)
+    np.savez_compressed(os.path.join(HERE, "small_net2.npz"), input=x,
+                        **{f"layer{i}": o for i, o in enumerate(outs)})
+    return [{k: L[k] for k in KEYS if k in L} for L in r.layers]
+
+
 def lexsorted(rows):
     """Rows in a canonical order (the reference leaves its array sorted by the last class after NMS)."""
     if len(rows) == 0:
@@ -147,12 +228,19 @@ def main():
         detections_fixture()
         print("detections_case.npz written")
         return
+    if sys.argv[1:] == ["small_net2"]:
+        tables = json.load(open(os.path.join(HERE, "layer_tables.json")))
+        tables["small_net2"] = small_net2_fixture()
+        json.dump(tables, open(os.path.join(HERE, "layer_tables.json"), "w"), indent=0)
+        print("small_net2 fixtures written")
+        return
     detections_fixture()
     # ---- layer tables
     tables = {}
     for name, text in [("yolov3-tiny-416", cfgs.yolov3_tiny(1, 416)), ("yolov3-416", cfgs.yolov3(1, 416)),
                        ("resnext50-224", cfgs.resnext50(1, 224)), ("small_net", SMALL_NET)]:
         _, tables[name] = table(text)
+    tables["small_net2"] = small_net2_fixture()
     json.dump(tables, open(os.path.join(HERE, "layer_tables.json"), "w"), indent=0)
 
     # ---- yolov3-tiny forward checksums

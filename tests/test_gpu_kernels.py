@@ -179,3 +179,25 @@ def test_binarize_bit_exact(dn, orc):
     d_w, d_bw = D(w), D(n=w.size)
     dn.binarize_weights_gpu(d_w.ptr, 24, 288, d_bw.ptr)
     assert np.array_equal(d_bw.numpy(), orc.binarize_weights(w, 24))
+
+
+@pytest.mark.parametrize("w,h,c,b,s", [(6, 4, 8, 2, 2), (13, 13, 64, 3, 2), (5, 7, 9, 1, 3), (8, 8, 4, 2, 1)])
+def test_reorg_gpu_both_directions(dn, orc, w, h, c, b, s):
+    x = synth.uniform(4, w * h * c * b, -1, 1)
+    for forward in (1, 0):
+        out = D(n=x.size)
+        keep = D(x)
+        dn.reorg_gpu(keep.ptr, w, h, c, b, s, forward, out.ptr)
+        assert np.array_equal(out.numpy(), orc.reorg(x, w, h, c, b, s, forward))
+
+
+def test_flatten_and_crop_gpu(dn, orc):
+    x = synth.uniform(5, 3 * 10 * 6 * 7, -1, 1).reshape(3, 10, 6, 7)
+    for forward in (1, 0):
+        out, keep = D(n=x.size), D(x)
+        dn.flatten_gpu(keep.ptr, 42, 10, 3, forward, out.ptr)
+        assert np.array_equal(out.numpy(), orc.flatten(x.reshape(-1), 42, 10, 3, forward))
+    for oh, ow, noadjust in [(4, 5, 0), (6, 7, 1), (1, 1, 0), (3, 2, 1)]:
+        out, keep = D(n=3 * 10 * oh * ow), D(x)
+        dn.forward_crop_gpu(keep.ptr, out.ptr, 3, 10, 6, 7, oh, ow, noadjust)
+        assert np.array_equal(out.numpy((3, 10, oh, ow)), orc.crop(x, oh, ow, noadjust))

@@ -193,3 +193,49 @@ def test_shortcut_fusion_changes_no_bit(dn):
     finally:
         net.L.network_set_fusion(1)
     net.free()
+
+
+def test_small_net2_crop_reorg_dropout_connected_cost(dn, tmp_path):
+    """The layer types beyond the yolo family (crop, the four reorg modes, dropout, connected with
+    and without batch-norm, cost): layer table, reference-written weights file, per-layer outputs
+    (index/copy layers bit-exact, connected <= 1e-4), and the weights file round trip."""
+    text = open(os.path.join(GOLD, "small_net2.cfg")).read()
+    gold = json.load(open(os.path.join(GOLD, "layer_tables.json")))["small_net2"]
+    g = np.load(os.path.join(GOLD, "small_net2.npz"))
+    net = api.Network(cfg_text=text, weights=os.path.join(GOLD, "small_net2.weights"))
+    assert [L["type"] for L in net.layers] == [L["type"] for L in gold]
+    for i, (a, b) in enumerate(zip(net.layers, gold)):
+        for k in ("batch", "out_h", "out_w", "out_c", "inputs", "outputs"):
+            assert a[k] == b[k], (i, a["type"], k, a[k], b[k])
+    final = net.predict(g["input"])
+    exact = ("crop", "reorg", "dropout", "cost")
+    prev = g["input"].reshape(net.batch, -1)
+    for i, L in enumerate(net.layers):
+        got, want = net.layer_output(i), g[f"layer{i}"].reshape(net.batch, -1)
+        assert norm_err(got, want) <= REL_TOL or (L["type"] == "cost" and not got.any()), (i, L["type"])
+        if L["type"] in exact:
+            # bit-exact on the library's own input: re-run the CPU checker's layer on it
+            again = OracleNet(text).forward_layer(i, prev, None)
+            assert np.array_equal(got, np.ascontiguousarray(again).reshape(net.batch, -1)), (i, L["type"])
+        prev = got
+    # the network's output layer skips the trailing cost layer (src/network.c:689-697)
+    assert net.layers[-1]["type"] == "cost" and np.array_equal(final, net.layer_output(net.n - 2))
+    out = str(tmp_path / "roundtrip.weights")
+    net.save_weights(out)
+    assert open(out, "rb").read() == open(os.path.join(GOLD, "small_net2.weights"), "rb").read()
+    net.free()
+
+
+def test_connected_layers_at_classifier_sizes(dn):
+    """vgg/alexnet-like heads: K = 9216 and 4096, batch 64; K-split tails and ragged M (1000)."""
+    text = ("[net]\nbatch=64\nsubdivisions=1\nwidth=6\nheight=6\nchannels=256\n"
+            "[connected]\noutput=4096\nactivation=relu\n[dropout]\nprobability=.5\n"
+            "[connected]\noutput=1000\nbatch_normalize=1\nactivation=linear\n[softmax]\n")
+    net, orc = build_pair(text, seed=77)
+    x = synth.uniform(3, net.inputs * net.batch, -1, 1)
+    net.predict(x)
+    want = orc.forward(x)
+    for i in range(net.n):
+        assert norm_err(net.layer_output(i), want[i]) <= REL_TOL, i
+    assert abs(net.conv_flops() - 2.0 * (9216 * 4096 + 4096 * 1000)) < 1
+    net.free()

@@ -41,7 +41,8 @@ def same_table(a, b, where=""):
 @pytest.mark.parametrize("name,text", [("yolov3-tiny-416", cfgs.yolov3_tiny(1, 416)),
                                        ("yolov3-416", cfgs.yolov3(1, 416)),
                                        ("resnext50-224", cfgs.resnext50(1, 224)),
-                                       ("small_net", open(os.path.join(GOLD, "small_net.cfg")).read())])
+                                       ("small_net", open(os.path.join(GOLD, "small_net.cfg")).read()),
+                                       ("small_net2", open(os.path.join(GOLD, "small_net2.cfg")).read())])
 def test_parser_matches_golden_layer_tables(name, text):
     gold = json.load(open(os.path.join(GOLD, "layer_tables.json")))[name]
     same_table(gold, ocfg.parse(text)["layers"], name)
@@ -97,8 +98,10 @@ def test_every_in_scope_reference_cfg_parses_identically():
         kinds = set(re.findall(r"(?m)^\s*(\[[a-z]+\])", text))
         if not kinds <= set(ocfg.SECTION_ALIASES):
             continue
+        if re.search(r"(?m)^\s*(tree|map)\s*=", text):
+            continue            # needs data files relative to the reference's working directory
         mine = ocfg.parse(text)["layers"]
         theirs = ref.RefNet(path).layers
         same_table(theirs, mine, os.path.basename(path))
         done += 1
-    assert done >= 20
+    assert done >= 33

@@ -36,6 +36,18 @@ def test_small_net_matches_golden_outputs_of_every_layer():
         assert np.array_equal(o, g[f"layer{i}"]), (i, net.layers[i]["type"])
 
 
+def test_small_net2_matches_golden_outputs_of_every_layer():
+    """crop, reorg (plain / reverse / flatten / extra), dropout, connected, softmax, cost."""
+    g = np.load(os.path.join(GOLD, "small_net2.npz"))
+    net = OracleNet(open(os.path.join(GOLD, "small_net2.cfg")).read())
+    fill_params(net.set_conv, net.layers, seed=640, bn="random")
+    outs = net.forward(g["input"])
+    kinds = [L["type"] for L in net.layers]
+    assert kinds.count("reorg") == 4 and kinds.count("connected") == 2 and "crop" in kinds and "cost" in kinds
+    for i, o in enumerate(outs):
+        assert np.array_equal(o, g[f"layer{i}"]), (i, net.layers[i]["type"])
+
+
 @pytest.mark.skipif(not ref.available(), reason="oracle/_ref (compiled reference) not built")
 @pytest.mark.parametrize("name,text", [("resnext50", cfgs.resnext50(2, 64)), ("yolov3", cfgs.yolov3(1, 96)),
                                        ("tiny-xnor", cfgs.yolov3_tiny(1, 96, xnor=True))])

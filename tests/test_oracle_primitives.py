@@ -323,3 +323,71 @@ def test_binarize_semantics_and_golden(orc):
     y = y * sc.reshape(1, -1, 1) + bias.reshape(1, -1, 1)
     y = np.where(y > 0, y, 0.1 * y)
     assert norm_err(out.reshape(2, 24, -1), y) < 1e-5
+
+
+# ---- connected / reorg / flatten / crop ---------------------------------------------------------
+def test_connected_against_float64_matmul_and_closed_form(orc):
+    o = orc
+    rng = np.random.default_rng(3)
+    x = rng.uniform(-1, 1, (5, 300)).astype(np.float32)
+    w = rng.uniform(-1, 1, (70, 300)).astype(np.float32)
+    b = rng.uniform(-1, 1, 70).astype(np.float32)
+    got = o.connected(x, w, b, outputs=70, activation="linear")
+    want = x.astype(np.float64) @ w.astype(np.float64).T + b
+    assert np.abs(got - want).max() <= 1e-4 * np.abs(want).max()
+    # small integers: exact; transposing the weight matrix must change the answer (w is [outputs][inputs])
+    xi = rng.integers(-4, 5, (3, 6)).astype(np.float32)
+    wi = rng.integers(-4, 5, (4, 6)).astype(np.float32)
+    bi = rng.integers(-4, 5, 4).astype(np.float32)
+    assert np.array_equal(o.connected(xi, wi, bi, outputs=4, activation="linear"), xi @ wi.T + bi)
+    assert np.array_equal(o.connected(xi, wi, bi, outputs=4, activation="relu"), np.maximum(xi @ wi.T + bi, 0))
+    # batch-norm tail: (x - mean)/(sqrt(var)+1e-6)*scale + bias per output
+    sc, mu, var = (rng.uniform(0.5, 2, 4).astype(np.float32) for _ in range(3))
+    got = o.connected(xi, wi, bi, sc, mu, var, outputs=4, batch_normalize=1, activation="linear")
+    want = ((xi @ wi.T).astype(np.float64) - mu) / (np.sqrt(var.astype(np.float64)) + 1e-6) * sc + bi
+    assert np.abs(got - want).max() <= 1e-5
+
+
+def test_reorg_is_a_permutation_with_the_stated_index_map(orc):
+    o = orc
+    w, h, c, b, s = 6, 4, 8, 2, 2
+    x = np.arange(w * h * c * b, dtype=np.float32)
+    fwd = o.reorg(x, w, h, c, b, s, 1)
+    back = o.reorg(x, w, h, c, b, s, 0)
+    assert sorted(fwd.tolist()) == x.tolist() and sorted(back.tolist()) == x.tolist()
+    assert np.array_equal(o.reorg(fwd, w, h, c, b, s, 0), x)        # the two directions are inverses
+    # the index map, spelled independently: element (b,k,j,i) of the [c,h,w] walk pairs with
+    # (b, k % oc, j*s + (k//oc)//s, i*s + (k//oc)%s) of an [oc, h*s, w*s] tensor, oc = c/s^2
+    oc = c // (s * s)
+    big = fwd.reshape(b, oc, h * s, w * s)
+    walk = x.reshape(b, c, h, w)
+    for (bb, k, j, i) in [(0, 0, 0, 0), (1, 5, 3, 2), (0, 7, 1, 5), (1, 2, 0, 4)]:
+        assert big[bb, k % oc, j * s + (k // oc) // s, i * s + (k // oc) % s] == walk[bb, k, j, i]
+    # the layer: a 2x reorg of yolov2 turns [c, h, w] into [4c, h/2, w/2] as a pure permutation
+    img = np.arange(2 * 4 * 4 * 6, dtype=np.float32).reshape(2, 4, 4, 6)
+    out = o.reorg_layer(img, 2)
+    assert out.shape == (2, 96) and sorted(out.reshape(-1).tolist()) == img.reshape(-1).tolist()
+    # the reverse layer walks ITS input's (w,h,c) with the scatter form; it is a permutation too,
+    # but not the inverse of the forward layer (both describe the walk with their own input's
+    # geometry, src/reorg_layer.c:102-106) - pinned by the golden network, not by an identity
+    rev = o.reorg_layer(out.reshape(2, 16, 2, 3), 2, reverse=1)
+    assert sorted(rev.reshape(-1).tolist()) == img.reshape(-1).tolist()
+
+
+def test_flatten_is_a_transpose_and_extra_pads_with_zeros(orc):
+    o = orc
+    x = np.arange(2 * 5 * 12, dtype=np.float32).reshape(2, 5, 3, 4)
+    f = o.reorg_layer(x, 1, flatten=1)
+    assert np.array_equal(f.reshape(2, 12, 5), x.reshape(2, 5, 12).transpose(0, 2, 1))
+    assert np.array_equal(o.reorg_layer(f.reshape(2, 5, 3, 4), 1, reverse=1, flatten=1).reshape(x.shape), x)
+    e = o.reorg_layer(x, 1, extra=3)
+    assert e.shape == (2, 63) and np.array_equal(e[:, :60], x.reshape(2, 60)) and not e[:, 60:].any()
+
+
+def test_crop_takes_the_centred_window_and_rescales(orc):
+    o = orc
+    x = synth.uniform01(2, 2 * 3 * 9 * 12).reshape(2, 3, 9, 12)
+    got = o.crop(x, 4, 6)
+    assert np.array_equal(got, x[:, :, 2:6, 3:9] * np.float32(2) + np.float32(-1))   # (9-4)//2 = 2, (12-6)//2 = 3
+    assert np.array_equal(o.crop(x, 4, 6, noadjust=1), x[:, :, 2:6, 3:9])
+    assert np.array_equal(o.crop(x, 9, 12, noadjust=1), x)

@@ -16,17 +16,22 @@ YOLO_ABS_TOL = 1e-3
 def fill_params(setter, layers, seed=1000, bn="random"):
     """Write the same weights / BN vectors into any network object exposing set_conv()."""
     for i, L in enumerate(layers):
-        if L["type"] != "convolutional":
+        if L["type"] == "convolutional":
+            n = L["n"]
+            w = synth.conv_weights(seed + i, n, L["c"] // L["groups"], L["size"])
+        elif L["type"] == "connected":      # weights [outputs][inputs]: a 1x1 convolution of a 1x1 image
+            n = L["outputs"]
+            w = synth.conv_weights(seed + i, n, L["inputs"], 1)
+        else:
             continue
-        w = synth.conv_weights(seed + i, L["n"], L["c"] // L["groups"], L["size"])
         if L["batch_normalize"]:
             if bn == "random":
-                b, s, m, v = synth.bn_random(seed * 2 + i, L["n"])
+                b, s, m, v = synth.bn_random(seed * 2 + i, n)
             else:
-                b, s, m, v = synth.bn_identity(L["n"])
+                b, s, m, v = synth.bn_identity(n)
             setter(i, w, b, s, m, v)
         else:
-            b = synth.uniform(seed * 3 + i, L["n"], -0.5, 0.5) if bn == "random" else np.zeros(L["n"], np.float32)
+            b = synth.uniform(seed * 3 + i, n, -0.5, 0.5) if bn == "random" else np.zeros(n, np.float32)
             setter(i, w, b, None, None, None)
 
 
