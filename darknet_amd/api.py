@@ -42,6 +42,52 @@ class DETECTION(C.Structure):
                 ("objectness", C.c_float), ("sort_class", C.c_int)]
 
 
+class IMAGE(C.Structure):
+    """python/darknet.py:36-40; data is [c][h][w] float32"""
+    _fields_ = [("w", C.c_int), ("h", C.c_int), ("c", C.c_int), ("data", _F)]
+
+
+def _image_of(arr):
+    arr = np.ascontiguousarray(arr, np.float32)
+    c, h, w = arr.shape
+    return IMAGE(w, h, c, _fp(arr)), arr
+
+
+def _bind_image_calls(L):
+    if getattr(L, "_image_calls_bound", False):
+        return
+    for name in ("letterbox_image", "resize_image"):
+        f = getattr(L, name)
+        f.argtypes = [IMAGE, C.c_int, C.c_int]
+        f.restype = IMAGE
+    L.free_image.argtypes = [IMAGE]
+    L.free_image.restype = None
+    L.network_predict_image.argtypes = [C.c_void_p, IMAGE]
+    L.network_predict_image.restype = _F
+    L.network_letterbox_input.argtypes = [C.c_void_p, C.c_int, IMAGE]
+    L.network_letterbox_input.restype = None
+    L._image_calls_bound = True
+
+
+def _image_call(name, arr, w, h):
+    L = _lib.load()
+    _bind_image_calls(L)
+    im, keep = _image_of(arr)
+    out = getattr(L, name)(im, w, h)
+    res = np.ctypeslib.as_array(out.data, shape=(out.c, out.h, out.w)).copy()
+    L.free_image(out)
+    return res
+
+
+def letterbox_image(arr, w, h):
+    """letterbox_image (python/darknet.py:102-104) on an array [c, h, w]."""
+    return _image_call("letterbox_image", arr, w, h)
+
+
+def resize_image(arr, w, h):
+    return _image_call("resize_image", arr, w, h)
+
+
 def _rows_of(dets, n, classes):
     rows = np.zeros((n, 5 + classes), np.float32)
     for i in range(n):
@@ -215,6 +261,22 @@ class Network:
         L = self.layers[i]
         p = self.L.layer_indexes_host(self.net, i)
         return np.ctypeslib.as_array(p, shape=(L["batch"], L["outputs"])).copy()
+
+    def predict_image(self, arr):
+        """network_predict_image (python/darknet.py:106-108): letterbox on the device, batch 1."""
+        _bind_image_calls(self.L)
+        im, keep = _image_of(arr)
+        out = self.L.network_predict_image(self.net, im)
+        self.batch = 1
+        last = [L for L in self.layers if L["type"] != "cost"][-1]
+        return np.ctypeslib.as_array(out, shape=(1, last["outputs"])).copy()
+
+    def letterbox_input(self, b, arr):
+        """Letterbox an image [c, h, w] into slot b of the device input (no forward)."""
+        _bind_image_calls(self.L)
+        im, keep = _image_of(arr)
+        self.L.network_letterbox_input(self.net, b, im)
+        self.L.hip_synchronize()      # `keep` may be released once the frame has left the host
 
     def get_boxes(self, w, h, thresh, relative=1, nms=0.0, image=0):
         """get_network_boxes (python/darknet.py:86-88) for `image` of the batch, with the

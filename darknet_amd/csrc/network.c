@@ -149,6 +149,19 @@ void pull_network_output(network *net)
     hip_pull_array(l.output_gpu, l.output, (size_t)l.outputs * l.batch);
 }
 
+/* What the host reads after a forward: the yolo heads (the reference pulls them inside
+ * forward_yolo_layer_gpu, src/yolo_layer.c:359-361) and the output layer (src/network.c:786). */
+void network_pull_outputs(network *netp)
+{
+    network net = *netp;
+    int i;
+    for (i = 0; i < net.n - 1; ++i) {
+        layer l = net.layers[i];
+        if (l.type == YOLO) hip_pull_array(l.output_gpu, l.output, (size_t)l.batch * l.outputs);
+    }
+    pull_network_output(netp);
+}
+
 /* src/network.c:762-788 */
 void forward_network_gpu(network *netp)
 {
@@ -157,11 +170,8 @@ void forward_network_gpu(network *netp)
     hip_set_device(net.gpu_index);
     hip_push_array(net.input_gpu, net.input, (size_t)net.inputs * net.batch);
     forward_network_device(netp);
-    for (i = 0; i < net.n - 1; ++i) {
-        layer l = net.layers[i];
-        if (l.type == YOLO) hip_pull_array(l.output_gpu, l.output, (size_t)l.batch * l.outputs);
-    }
-    pull_network_output(netp);
+    (void)i;
+    network_pull_outputs(netp);
 }
 
 /* src/network.c:188-211 */

@@ -66,6 +66,8 @@ SIGNATURES = {
     "get_layer_string": (C.c_char_p, [i]),
     "reorg_gpu": (None, [V, i, i, i, i, i, i, V]), "flatten_gpu": (None, [V, i, i, i, i, V]),
     "forward_crop_gpu": (None, [V, V, i, i, i, i, i, i, i]),
+    "resize_image_gpu": (None, [V, i, i, i, V, i, i]), "letterbox_image_gpu": (None, [V, i, i, i, V, i, i]),
+    "network_pull_outputs": (None, [V]),
     "yolo_decode_gpu": (None, [V, i, i, i, i, F, i, i, i, i, i, f, V, i, V]),
     "nms_sort_gpu": (None, [V, i, i, f]),
     "num_detections": (i, [V, f]), "make_network_boxes": (V, [V, f, I]),
@@ -99,6 +101,8 @@ STRUCT_BY_VALUE = [
     "make_connected_layer", "make_dropout_layer", "make_reorg_layer", "make_crop_layer", "make_cost_layer",
     "forward_connected_layer_gpu", "forward_dropout_layer_gpu", "forward_reorg_layer_gpu",
     "forward_crop_layer_gpu", "forward_cost_layer_gpu", "push_connected_layer", "pull_connected_layer",
+    "make_image", "make_empty_image", "free_image", "resize_image", "letterbox_image", "network_predict_image",
+    "network_letterbox_input",
 ]
 
 _lib = None

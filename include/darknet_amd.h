@@ -241,6 +241,25 @@ void pull_network_output(network *net);                     /* src/network.c:112
 int network_width(network *net);                            /* src/network.c:674 */
 int network_height(network *net);                           /* src/network.c:675 */
 
+/* ---- input side: include/darknet.h:508-513 and src/image.c / src/network.c:579 ------------- */
+typedef struct {
+    int w;
+    int h;
+    int c;
+    float *data;
+} image;
+image make_image(int w, int h, int c);                     /* src/image.c:743 */
+image make_empty_image(int w, int h, int c);               /* src/image.c:734 */
+void free_image(image m);                                  /* src/image.c:1368 */
+image resize_image(image im, int w, int h);                /* src/image.c:1199 */
+image letterbox_image(image im, int w, int h);             /* src/image.c:812 */
+float *network_predict_image(network *net, image im);      /* src/network.c:579 */
+/* additions: letterbox `im` straight into image slot b of the device input (one upload of the
+ * frame at its own size through a pinned staging buffer, no host-side resize); and the host
+ * pulls network_predict ends with (yolo heads + output layer) on their own */
+void network_letterbox_input(network *net, int b, image im);
+void network_pull_outputs(network *net);
+
 /* ---- detections (yolo heads only; region/detection layers are outside the path) ---------- */
 int num_detections(network *net, float thresh);                       /* src/network.c:510 */
 detection *make_network_boxes(network *net, float thresh, int *num);  /* src/network.c:526 */

@@ -206,6 +206,17 @@ void forward_crop_gpu(const float *input, float *output, int batch, int c, int h
                       int out_w, int noadjust);
 
 /* ------------------------------------------------------------------------------------------
+ * Input side.  Images are [c][h][w] floats as the reference's `image` (include/darknet.h:508).
+ * ---------------------------------------------------------------------------------------- */
+
+/* resize_image (src/image.c:1199-1241): the reference's two-pass bilinear filter, bit for bit
+ * (the horizontal pass's float intermediate is recomputed, not stored).  letterbox_image
+ * (src/image.c:812-831): the image resized to fit box_w x box_h with its aspect kept, centred
+ * on a .5 background (fill_image, embed_image :428-439).  All pointers are device pointers. */
+void resize_image_gpu(const float *im, int w, int h, int c, float *out, int out_w, int out_h);
+void letterbox_image_gpu(const float *im, int w, int h, int c, float *boxed, int box_w, int box_h);
+
+/* ------------------------------------------------------------------------------------------
  * Detections: the step right after the forward pass.  A detection is a row of (5 + classes)
  * floats in device memory: x, y, w, h, objectness, prob[classes].
  * ---------------------------------------------------------------------------------------- */

@@ -221,6 +221,20 @@ class Oracle:
         self.lib.orc_crop(_fp(x), _fp(out), b, c, h, w, out_h, out_w, int(noadjust))
         return out
 
+    def resize_image(self, im, ow, oh):
+        im = np.ascontiguousarray(im, np.float32)
+        c, h, w = im.shape
+        out = np.empty((c, oh, ow), np.float32)
+        self.lib.orc_resize_image(_fp(im), w, h, c, _fp(out), ow, oh)
+        return out
+
+    def letterbox_image(self, im, bw, bh):
+        im = np.ascontiguousarray(im, np.float32)
+        c, h, w = im.shape
+        out = np.empty((c, bh, bw), np.float32)
+        self.lib.orc_letterbox_image(_fp(im), w, h, c, _fp(out), bw, bh)
+        return out
+
     def yolo_detections(self, pred, n_anchors, classes, biases, mask, netw, neth, w, h, relative, thresh):
         """get_yolo_detections on image 0 of `pred` [n*(5+classes), lh, lw] -> rows [count, 5+classes]."""
         pred = np.ascontiguousarray(pred, np.float32)

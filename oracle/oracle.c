@@ -611,3 +611,64 @@ void orc_crop(const float *input, float *output, int batch, int c, int h, int w,
                     output[count++] = input[index] * scale + trans;
                 }
 }
+
+/* ---- resize_image: src/image.c:1199-1241.  Horizontal pass into `part`, vertical pass from it;
+ * images are [c][h][w]. ---------------------------------------------------------------------- */
+void orc_resize_image(const float *im, int imw, int imh, int imc, float *resized, int w, int h)
+{
+    float *part = (float *)calloc((size_t)w * imh * imc, sizeof(float));
+    const float w_scale = (float)(imw - 1) / (w - 1);
+    const float h_scale = (float)(imh - 1) / (h - 1);
+    for (int k = 0; k < imc; ++k)
+        for (int r = 0; r < imh; ++r)
+            for (int c = 0; c < w; ++c) {
+                float val = 0;
+                if (c == w - 1 || imw == 1) {
+                    val = im[(long)k * imh * imw + (long)r * imw + imw - 1];
+                } else {
+                    float sx = c * w_scale;
+                    int ix = (int)sx;
+                    float dx = sx - ix;
+                    val = (1 - dx) * im[(long)k * imh * imw + (long)r * imw + ix] +
+                          dx * im[(long)k * imh * imw + (long)r * imw + ix + 1];
+                }
+                part[(long)k * imh * w + (long)r * w + c] = val;
+            }
+    for (int k = 0; k < imc; ++k)
+        for (int r = 0; r < h; ++r) {
+            float sy = r * h_scale;
+            int iy = (int)sy;
+            float dy = sy - iy;
+            for (int c = 0; c < w; ++c)
+                resized[(long)k * h * w + (long)r * w + c] = (1 - dy) * part[(long)k * imh * w + (long)iy * w + c];
+            if (r == h - 1 || imh == 1) continue;
+            for (int c = 0; c < w; ++c)
+                resized[(long)k * h * w + (long)r * w + c] += dy * part[(long)k * imh * w + (long)(iy + 1) * w + c];
+        }
+    free(part);
+}
+
+/* ---- letterbox_image: src/image.c:812-831 with fill_image(.5) and embed_image :428-439 ----- */
+void orc_letterbox_image(const float *im, int imw, int imh, int imc, float *boxed, int w, int h)
+{
+    int new_w = imw, new_h = imh;
+    if (((float)w / imw) < ((float)h / imh)) {
+        new_w = w;
+        new_h = (imh * w) / imw;
+    } else {
+        new_h = h;
+        new_w = (imw * h) / imh;
+    }
+    float *resized = (float *)calloc((size_t)new_w * new_h * imc, sizeof(float));
+    orc_resize_image(im, imw, imh, imc, resized, new_w, new_h);
+    for (long i = 0; i < (long)w * h * imc; ++i) boxed[i] = .5;
+    const int dx = (w - new_w) / 2, dy = (h - new_h) / 2;
+    for (int k = 0; k < imc; ++k)
+        for (int y = 0; y < new_h; ++y)
+            for (int x = 0; x < new_w; ++x) {
+                const int X = dx + x, Y = dy + y;
+                if (X < 0 || Y < 0 || X >= w || Y >= h) continue;
+                boxed[(long)k * h * w + (long)Y * w + X] = resized[(long)k * new_h * new_w + (long)y * new_w + x];
+            }
+    free(resized);
+}

@@ -78,6 +78,9 @@ void orc_flatten(const float *x, int size, int layers, int batch, int forward, f
 void orc_crop(const float *input, float *output, int batch, int c, int h, int w, int out_h, int out_w,
               int noadjust);
 
+void orc_resize_image(const float *im, int imw, int imh, int imc, float *resized, int w, int h);
+void orc_letterbox_image(const float *im, int imw, int imh, int imc, float *boxed, int w, int h);
+
 /* detections (test infrastructure like everything here): see oracle.c */
 int orc_yolo_detections(const float *pred, int lw, int lh, int n, int classes, const float *biases,
                         const int *mask, int netw, int neth, int w, int h, int relative, float thresh,

@@ -43,6 +43,28 @@ def raw(variant: str = "o2"):
     return C.CDLL(os.path.join(_HERE, "_ref", name))
 
 
+def _harness(variant="o2"):
+    raw(variant)
+    return C.CDLL(_path(variant))
+
+
+def resize_image(im, ow, oh, variant="o2"):
+    """resize_image of the compiled reference on an array [c, h, w]."""
+    im = np.ascontiguousarray(im, np.float32)
+    c, h, w = im.shape
+    out = np.empty((c, oh, ow), np.float32)
+    _harness(variant).refh_resize_image(im.ctypes.data_as(_F), w, h, c, ow, oh, out.ctypes.data_as(_F))
+    return out
+
+
+def letterbox_image(im, bw, bh, variant="o2"):
+    im = np.ascontiguousarray(im, np.float32)
+    c, h, w = im.shape
+    out = np.empty((c, bh, bw), np.float32)
+    _harness(variant).refh_letterbox_image(im.ctypes.data_as(_F), w, h, c, bw, bh, out.ctypes.data_as(_F))
+    return out
+
+
 class RefNet:
     """A network parsed and run by the compiled reference (CPU build)."""
 

@@ -177,3 +177,20 @@ void refh_set_output(network *net, int i, const float *values)
     memcpy(l.output, values, sizeof(float) * (size_t)l.outputs * l.batch);
 }
 
+/* resize_image / letterbox_image (src/image.c:1199, :812) on a caller's [c][h][w] array */
+void refh_resize_image(float *data, int w, int h, int c, int ow, int oh, float *out)
+{
+    image im = {w, h, c, data};
+    image r = resize_image(im, ow, oh);
+    memcpy(out, r.data, sizeof(float) * (size_t)ow * oh * c);
+    free_image(r);
+}
+
+void refh_letterbox_image(float *data, int w, int h, int c, int bw, int bh, float *out)
+{
+    image im = {w, h, c, data};
+    image r = letterbox_image(im, bw, bh);
+    memcpy(out, r.data, sizeof(float) * (size_t)bw * bh * c);
+    free_image(r);
+}
+

@@ -18,10 +18,11 @@ seeded synthetic inputs; nothing from the reference's sources is stored.  Fixtur
   maxpool_case.npz       maxpool output + indexes incl. the padded stride-1 case
   small_net2.cfg/.weights/.npz  the same for a network of crop, reorg (plain, reverse, flatten,
                          extra), dropout, connected (with and without batch-norm), softmax, cost
+  image_cases.npz        letterbox_image / resize_image of small images (down, up, both aspects)
   detections_case.npz    the two yolo tensors of a yolov3-tiny forward at 96x96 and what
                          get_network_boxes / do_nms_sort make of them (rows x,y,w,h,obj,prob[80])
 
-`python tests/golden/make_golden.py detections|small_net2` rewrites only that fixture.
+`python tests/golden/make_golden.py detections|small_net2|images` rewrites only that fixture.
 """
 import json
 import os
@@ -197,6 +198,21 @@ def small_net2_fixture():
     return [{k: L[k] for k in KEYS if k in L} for L in r.layers]
 
 
+IMAGE_CASES = {"wide": (3, 37, 53, 32, 32), "tall": (3, 41, 19, 24, 40), "up": (1, 9, 12, 30, 26),
+               "same": (2, 16, 16, 16, 16)}
+
+
+def images_fixture():
+    """letterbox_image and resize_image of the reference on small seeded images [c, h, w]."""
+    data = {}
+    for name, (c, h, w, bw, bh) in IMAGE_CASES.items():
+        im = synth.uniform01(31, c * h * w).reshape(c, h, w)
+        data[name + "_in"] = im
+        data[name + "_box"] = ref.letterbox_image(im, bw, bh)
+        data[name + "_resized"] = ref.resize_image(im, bw, bh)
+    np.savez_compressed(os.path.join(HERE, "image_cases.npz"), **data)
+
+
 def lexsorted(rows):
     """Rows in a canonical order (the reference leaves its array sorted by the last class after NMS)."""
     if len(rows) == 0:
@@ -228,6 +244,10 @@ def main():
         detections_fixture()
         print("detections_case.npz written")
         return
+    if sys.argv[1:] == ["images"]:
+        images_fixture()
+        print("image_cases.npz written")
+        return
     if sys.argv[1:] == ["small_net2"]:
         tables = json.load(open(os.path.join(HERE, "layer_tables.json")))
         tables["small_net2"] = small_net2_fixture()
@@ -235,6 +255,7 @@ def main():
         print("small_net2 fixtures written")
         return
     detections_fixture()
+    images_fixture()
     # ---- layer tables
     tables = {}
     for name, text in [("yolov3-tiny-416", cfgs.yolov3_tiny(1, 416)), ("yolov3-416", cfgs.yolov3(1, 416)),
