@@ -17,9 +17,9 @@ static int network_max_detections(network *net, int *classes)
     int i, s = 0, cl = -1;
     for (i = 0; i < net->n; ++i) {
         layer l = net->layers[i];
-        if (l.type != YOLO) continue;
+        if (l.type != YOLO && l.type != REGION) continue;
         s += l.w * l.h * l.n;
-        if (cl >= 0 && cl != l.classes) dn_fatal("detections: yolo heads disagree on the number of classes");
+        if (cl >= 0 && cl != l.classes) dn_fatal("detections: heads disagree on the number of classes");
         cl = l.classes;
     }
     if (classes) *classes = cl < 0 ? 0 : cl;
@@ -48,9 +48,15 @@ int network_decode_image_gpu(network *net, int b, int w, int h, float thresh, in
     for (i = 0; i < net->n; ++i) {
         layer l = net->layers[i];
         float anchors[32];
-        if (l.type == REGION || l.type == DETECTION) dn_fatal("detections: only yolo heads are decoded");
-        if (l.type != YOLO) continue;
+        if (l.type == DETECTION) dn_fatal("detections: the yolov1 detection layer is not decoded");
+        if (l.type != YOLO && l.type != REGION) continue;
         if (l.n > 16) dn_fatal("detections: more than 16 anchors per head");
+        if (l.type == REGION) { /* src/network.c:553-556 */
+            region_decode_gpu(l.output_gpu + (size_t)b * l.outputs, l.w, l.h, l.n, l.classes, l.coords,
+                              l.background, l.biases, net->w, net->h, w, h, relative, thresh, net->det_rows_gpu,
+                              net->det_max_rows, net->det_count_gpu);
+            continue;
+        }
         for (j = 0; j < l.n; ++j) {
             anchors[2 * j] = l.biases[2 * l.mask[j]];
             anchors[2 * j + 1] = l.biases[2 * l.mask[j] + 1];

@@ -41,6 +41,7 @@ static LAYER_TYPE section_type(const char *t)
     if (!strcmp(t, "[reorg]")) return REORG;
     if (!strcmp(t, "[crop]")) return CROP;
     if (!strcmp(t, "[cost]")) return COST;
+    if (!strcmp(t, "[region]")) return REGION;
     return BLANK;
 }
 
@@ -81,6 +82,7 @@ char *get_layer_string(LAYER_TYPE a)
     case REORG: return "reorg";
     case CROP: return "crop";
     case COST: return "cost";
+    case REGION: return "region";
     default: return "none";
     }
 }
@@ -284,6 +286,36 @@ static layer parse_cost(cfg_section *o, size_params p)
     return make_cost_layer(p.batch, p.inputs, 0, scale);
 }
 
+/* src/parser.c:353-403 */
+static layer parse_region(cfg_section *o, size_params p)
+{
+    static const char *training_keys[] = {"log", "sqrt", "max", "jitter", "rescore", "thresh", "classfix",
+                                          "absolute", "random", "coord_scale", "object_scale", "noobject_scale",
+                                          "mask_scale", "class_scale", "bias_match", 0};
+    int coords = cfg_find_int(o, "coords", 4);
+    int classes = cfg_find_int(o, "classes", 20);
+    int num = cfg_find_int(o, "num", 1);
+    char *a;
+    int i;
+    layer l = make_region_layer(p.batch, p.w, p.h, num, classes, coords);
+    if (l.outputs != p.inputs) dn_fatal("region layer: the layer before it must output num*(classes+coords+1) channels");
+    l.softmax = cfg_find_int(o, "softmax", 0);
+    l.background = cfg_find_int_quiet(o, "background", 0);
+    for (i = 0; training_keys[i]; ++i) (void)cfg_find(o, training_keys[i]);
+    if (cfg_find_str(o, "tree", 0)) dn_fatal("region layer: tree= (hierarchical softmax) is not supported");
+    if (cfg_find_str(o, "map", 0)) dn_fatal("region layer: map= is not supported");
+    a = cfg_find_str(o, "anchors", 0);
+    if (a) {
+        int n = count_commas(a);
+        for (i = 0; i < n && i < 2 * num; ++i) {
+            char *next = strchr(a, ',');
+            l.biases[i] = (float)atof(a);
+            a = next ? next + 1 : a + strlen(a);
+        }
+    }
+    return l;
+}
+
 /* src/parser.c:285-342 */
 static layer parse_yolo(cfg_section *o, size_params p)
 {
@@ -383,6 +415,7 @@ network *parse_network_cfg(char *filename)
         case REORG: l = parse_reorg(o, p); break;
         case CROP: l = parse_crop(o, p); break;
         case COST: l = parse_cost(o, p); break;
+        case REGION: l = parse_region(o, p); break;
         case DROPOUT:
             if (count == 0) dn_fatal("dropout cannot be the first layer");
             l = parse_dropout(o, p);

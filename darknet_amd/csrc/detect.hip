@@ -145,6 +145,112 @@ extern "C" void yolo_decode_gpu(const float *layer_output, int lw, int lh, int n
     dn_check_launch("yolo_decode_gpu");
 }
 
+/* ---- region head (yolov2): get_region_detections src/region_layer.c:364-437 ----------------
+ * Every anchor of every cell becomes a row, at index anchor*cells + cell (no compaction: the
+ * reference returns w*h*n detections); objectness below the threshold is stored as 0 and leaves
+ * the class probabilities at 0.  Boxes: get_region_box :76-84 (anchors in cell units, divided
+ * by the layer size) and correct_region_boxes :336-362. */
+struct region_decode_args {
+    const float *pred; /* one image's region output: [n][coords + 1 + classes][lh][lw] */
+    float *rows;
+    int *count;
+    int max_rows;
+    int lw, lh, n, classes, coords, background;
+    int netw, neth, w, h, new_w, new_h, relative;
+    float thresh;
+    float anchors[2 * DN_MAX_ANCHORS];
+};
+
+__global__ void region_decode_kernel(region_decode_args a)
+{
+    const int cells = a.lw * a.lh;
+    const int total = cells * a.n;
+    const int entries = a.coords + a.classes + 1;
+    const int base = *a.count;
+    for (int idx = blockIdx.x * blockDim.x + threadIdx.x; idx < total; idx += gridDim.x * blockDim.x) {
+        if (base + idx >= a.max_rows) continue;
+        const int n = idx / cells, cell = idx - n * cells;
+        const int col = cell % a.lw, row = cell / a.lw;
+        const float *p = a.pred + (long)n * entries * cells + cell;
+        const float scale = a.background ? 1.f : p[(long)a.coords * cells];
+        float bx = __fdiv_rn(__fadd_rn((float)col, p[0]), (float)a.lw);
+        float by = __fdiv_rn(__fadd_rn((float)row, p[(long)cells]), (float)a.lh);
+        float bw = (float)(exp((double)p[2L * cells]) * (double)a.anchors[2 * n] / (double)a.lw);
+        float bh = (float)(exp((double)p[3L * cells]) * (double)a.anchors[2 * n + 1] / (double)a.lh);
+        bx = (float)(((double)bx - (double)(a.netw - a.new_w) / 2. / (double)a.netw) /
+                     (double)__fdiv_rn((float)a.new_w, (float)a.netw));
+        by = (float)(((double)by - (double)(a.neth - a.new_h) / 2. / (double)a.neth) /
+                     (double)__fdiv_rn((float)a.new_h, (float)a.neth));
+        bw = __fmul_rn(bw, __fdiv_rn((float)a.netw, (float)a.new_w));
+        bh = __fmul_rn(bh, __fdiv_rn((float)a.neth, (float)a.new_h));
+        if (!a.relative) {
+            bx = __fmul_rn(bx, (float)a.w);
+            bw = __fmul_rn(bw, (float)a.w);
+            by = __fmul_rn(by, (float)a.h);
+            bh = __fmul_rn(bh, (float)a.h);
+        }
+        float *r = a.rows + (long)(base + idx) * (5 + a.classes);
+        const float obj = scale > a.thresh ? scale : 0.f;
+        r[0] = bx;
+        r[1] = by;
+        r[2] = bw;
+        r[3] = bh;
+        r[4] = obj;
+        const float *cls = p + (long)(a.coords + 1) * cells;
+        for (int j = 0; j < a.classes; ++j) {
+            float v = 0.f;
+            if (obj != 0.f) {
+                const float prob = __fmul_rn(scale, cls[(long)j * cells]);
+                v = (prob > a.thresh) ? prob : 0.f;
+            }
+            r[5 + j] = v;
+        }
+    }
+}
+
+__global__ void add_count_kernel(int *count, int n) { *count += n; }
+
+extern "C" void region_decode_gpu(const float *layer_output, int lw, int lh, int n, int classes, int coords,
+                                  int background, const float *anchors, int netw, int neth, int w, int h,
+                                  int relative, float thresh, float *rows, int max_rows, int *count)
+{
+    if (!layer_output || !anchors || !rows || !count) dn_fatal("region_decode_gpu: null pointer");
+    if (lw <= 0 || lh <= 0 || n <= 0 || classes < 0 || netw <= 0 || neth <= 0 || w <= 0 || h <= 0 || max_rows < 0)
+        dn_fatal("region_decode_gpu: bad geometry");
+    if (coords != 4) dn_fatal("region_decode_gpu: only coords=4 (no masks) is decoded");
+    if (n > DN_MAX_ANCHORS) dn_fatal("region_decode_gpu: more than 16 anchors");
+    region_decode_args a;
+    a.pred = layer_output;
+    a.rows = rows;
+    a.count = count;
+    a.max_rows = max_rows;
+    a.lw = lw;
+    a.lh = lh;
+    a.n = n;
+    a.classes = classes;
+    a.coords = coords;
+    a.background = background;
+    a.netw = netw;
+    a.neth = neth;
+    a.w = w;
+    a.h = h;
+    a.relative = relative;
+    a.thresh = thresh;
+    if (((float)netw / w) < ((float)neth / h)) {
+        a.new_w = netw;
+        a.new_h = (h * netw) / w;
+    } else {
+        a.new_h = neth;
+        a.new_w = (w * neth) / h;
+    }
+    if (a.new_w <= 0 || a.new_h <= 0) dn_fatal("region_decode_gpu: image too thin for the network input");
+    for (int i = 0; i < 2 * DN_MAX_ANCHORS; ++i) a.anchors[i] = i < 2 * n ? anchors[i] : 0.f;
+    const int total = lw * lh * n;
+    hipLaunchKernelGGL(region_decode_kernel, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, dn_stream(), a);
+    hipLaunchKernelGGL(add_count_kernel, dim3(1), dim3(1), 0, dn_stream(), count, total);
+    dn_check_launch("region_decode_gpu");
+}
+
 /* ---- non-maximum suppression ------------------------------------------------------------- */
 /* box_iou of src/box.c:111-155 in the reference's float arithmetic */
 __device__ __forceinline__ float dn_overlap(float x1, float w1, float x2, float w2)

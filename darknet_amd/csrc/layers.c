@@ -575,6 +575,42 @@ void forward_cost_layer_gpu(layer l, network net)
     (void)net;
 }
 
+/* ---- region (yolov2 head): src/region_layer.c:13-56.  biases hold the n anchors in cell
+ * units (default .5). --------------------------------------------------------------------------- */
+layer make_region_layer(int batch, int w, int h, int n, int classes, int coords)
+{
+    layer l;
+    int i;
+    memset(&l, 0, sizeof l);
+    l.type = REGION;
+    l.n = n;
+    l.batch = batch;
+    l.h = h;
+    l.w = w;
+    l.c = n * (classes + coords + 1);
+    l.out_w = l.w;
+    l.out_h = l.h;
+    l.out_c = l.c;
+    l.classes = classes;
+    l.coords = coords;
+    l.biases = (float *)dn_calloc((size_t)n * 2, sizeof(float));
+    l.outputs = h * w * n * (classes + coords + 1);
+    l.inputs = l.outputs;
+    l.truths = 30 * (l.coords + 1);
+    l.output = (float *)dn_calloc((size_t)batch * l.outputs, sizeof(float));
+    for (i = 0; i < n * 2; ++i) l.biases[i] = .5f;
+    l.forward_gpu = forward_region_layer_gpu;
+    l.output_gpu = hip_make_array(0, (size_t)batch * l.outputs);
+    if (dn_verbose) fprintf(stderr, "detection\n");
+    return l;
+}
+
+void forward_region_layer_gpu(layer l, network net)
+{
+    forward_region_gpu(net.input_gpu, l.output_gpu, l.batch, l.w, l.h, l.n, l.classes, l.coords, l.background,
+                       l.softmax);
+}
+
 void free_layer(layer l)
 {
     if (l.type == DROPOUT) return; /* its buffers belong to the layer before it (src/layer.c:8-14) */

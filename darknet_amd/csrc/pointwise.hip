@@ -6,6 +6,7 @@
  * 256 CUs several times.
  */
 #include <hip/hip_runtime.h>
+#include <float.h>
 #include <stdint.h>
 
 #include "device_math.h"
@@ -485,4 +486,63 @@ extern "C" void forward_crop_gpu(const float *input, float *output, int batch, i
     hipLaunchKernelGGL(crop_kernel, dim3(dn_blocks(n)), dim3(DN_BLOCK), 0, dn_stream(), input, output, n, c, h, w,
                        out_h, out_w, (h - out_h) / 2, (w - out_w) / 2, noadjust ? 1.f : 2.f, noadjust ? 0.f : -1.f);
     dn_check_launch("forward_crop_gpu");
+}
+
+/* ---- region head (yolov2): src/region_layer.c:158-184, the inference part of the CPU build -- */
+/* copy + logistic on x, y, on objectness unless `background`, on the classes unless a softmax
+ * follows; layout [b][anchor][coords + 1 + classes][h][w] */
+__global__ void region_kernel(const float *in, float *out, long n, int plane, int entries, int coords,
+                              int background, int softmax)
+{
+    for (long i = blockIdx.x * (long)blockDim.x + threadIdx.x; i < n; i += (long)gridDim.x * blockDim.x) {
+        const int e = (int)((i / plane) % entries);
+        const float v = in[i];
+        const bool act = e < 2 || (e == coords && !background) || (e > coords && !softmax);
+        out[i] = act ? dn_activate(v, DN_LOGISTIC) : v;
+    }
+}
+
+/* softmax over the classes of one (image, anchor, cell): softmax_cpu with stride = plane
+ * (src/blas.c:305-332), one thread per cell so that neighbouring threads read neighbouring
+ * addresses and the float sum runs in the reference's order */
+__global__ void region_softmax_kernel(const float *in, float *out, long rows, int plane, int entries, int first,
+                                      int n)
+{
+    for (long r = blockIdx.x * (long)blockDim.x + threadIdx.x; r < rows; r += (long)gridDim.x * blockDim.x) {
+        const long group = r / plane;
+        const int cell = (int)(r - group * plane);
+        const float *x = in + (group * entries + first) * plane + cell;
+        float *y = out + (group * entries + first) * plane + cell;
+        float largest = -FLT_MAX;
+        for (int i = 0; i < n; ++i) {
+            const float v = x[(long)i * plane];
+            if (v > largest) largest = v;
+        }
+        float sum = 0;
+        for (int i = 0; i < n; ++i) {
+            const float e = (float)exp((double)__fsub_rn(x[(long)i * plane], largest)); /* temp == 1 */
+            sum = __fadd_rn(sum, e);
+            y[(long)i * plane] = e;
+        }
+        for (int i = 0; i < n; ++i) y[(long)i * plane] = __fdiv_rn(y[(long)i * plane], sum);
+    }
+}
+
+extern "C" void forward_region_gpu(const float *input, float *output, int batch, int w, int h, int n_anchors,
+                                   int classes, int coords, int background, int softmax)
+{
+    if (batch <= 0 || w <= 0 || h <= 0 || n_anchors <= 0 || classes < 0 || coords < 4)
+        dn_fatal("forward_region_gpu: bad geometry");
+    if (input == output) dn_fatal("forward_region_gpu: in-place operation is not supported");
+    const int entries = coords + classes + 1;
+    const int plane = w * h;
+    const long n = (long)batch * n_anchors * entries * plane;
+    hipLaunchKernelGGL(region_kernel, dim3(dn_blocks(n)), dim3(DN_BLOCK), 0, dn_stream(), input, output, n, plane,
+                       entries, coords, background, softmax);
+    if (softmax && classes + background > 0) {
+        const long rows = (long)batch * n_anchors * plane;
+        hipLaunchKernelGGL(region_softmax_kernel, dim3(dn_blocks(rows)), dim3(DN_BLOCK), 0, dn_stream(), input,
+                           output, rows, plane, entries, coords + !background, classes + background);
+    }
+    dn_check_launch("forward_region_gpu");
 }

@@ -70,6 +70,8 @@ SIGNATURES = {
     "network_pull_outputs": (None, [V]),
     "yolo_decode_gpu": (None, [V, i, i, i, i, F, i, i, i, i, i, f, V, i, V]),
     "nms_sort_gpu": (None, [V, i, i, f]),
+    "region_decode_gpu": (None, [V, i, i, i, i, i, i, F, i, i, i, i, i, f, V, i, V]),
+    "forward_region_gpu": (None, [V, V, i, i, i, i, i, i, i, i]),
     "num_detections": (i, [V, f]), "make_network_boxes": (V, [V, f, I]),
     "fill_network_boxes": (None, [V, i, i, f, f, I, i, V]),
     "get_network_boxes": (V, [V, i, i, f, f, I, i, I]), "free_detections": (None, [V, i]),
@@ -101,6 +103,7 @@ STRUCT_BY_VALUE = [
     "make_connected_layer", "make_dropout_layer", "make_reorg_layer", "make_crop_layer", "make_cost_layer",
     "forward_connected_layer_gpu", "forward_dropout_layer_gpu", "forward_reorg_layer_gpu",
     "forward_crop_layer_gpu", "forward_cost_layer_gpu", "push_connected_layer", "pull_connected_layer",
+    "make_region_layer", "forward_region_layer_gpu",
     "make_image", "make_empty_image", "free_image", "resize_image", "letterbox_image", "network_predict_image",
     "network_letterbox_input",
 ]

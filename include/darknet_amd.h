@@ -88,6 +88,9 @@ struct layer {
     float ignore_thresh;
     float truth_thresh;
     int random;
+    int coords;        /* region */
+    int background;
+    int softmax;
     int flatten;       /* reorg */
     int extra;
     int noadjust;      /* crop */
@@ -206,6 +209,7 @@ layer make_reorg_layer(int batch, int w, int h, int c, int stride, int reverse, 
 layer make_crop_layer(int batch, int h, int w, int c, int crop_height, int crop_width, int flip,
                       float angle, float saturation, float exposure); /* src/crop_layer.c:18 */
 layer make_cost_layer(int batch, int inputs, int cost_type, float scale); /* src/cost_layer.c:40 */
+layer make_region_layer(int batch, int w, int h, int n, int classes, int coords); /* src/region_layer.c:13 */
 layer make_softmax_layer(int batch, int inputs, int groups); /* src/softmax_layer.c:11 */
 void free_layer(layer l);                                 /* src/layer.c:6 */
 
@@ -223,6 +227,7 @@ void forward_dropout_layer_gpu(layer l, network net);       /* src/dropout_layer
 void forward_reorg_layer_gpu(layer l, network net);         /* src/reorg_layer.c:149 */
 void forward_crop_layer_gpu(layer l, network net);          /* src/crop_layer_kernels.cu:183 */
 void forward_cost_layer_gpu(layer l, network net);          /* src/cost_layer.c:120 (no truth: nothing) */
+void forward_region_layer_gpu(layer l, network net);        /* src/region_layer.c:439 */
 void push_connected_layer(layer l);                         /* src/connected_layer.c:268 */
 void pull_connected_layer(layer l);                         /* src/connected_layer.c:254 */
 void push_convolutional_layer(layer l);                     /* src/convolutional_kernels.cu:286 */
@@ -260,7 +265,7 @@ float *network_predict_image(network *net, image im);      /* src/network.c:579 
 void network_letterbox_input(network *net, int b, image im);
 void network_pull_outputs(network *net);
 
-/* ---- detections (yolo heads only; region/detection layers are outside the path) ---------- */
+/* ---- detections (yolo and region heads; the yolov1 detection layer is outside the path) ---- */
 int num_detections(network *net, float thresh);                       /* src/network.c:510 */
 detection *make_network_boxes(network *net, float thresh, int *num);  /* src/network.c:526 */
 void fill_network_boxes(network *net, int w, int h, float thresh, float hier, int *map, int relative,

@@ -192,6 +192,13 @@ void forward_shortcut_gpu(const float *in, const float *add, float *out, int bat
 void forward_yolo_gpu(const float *input, float *output, int batch, int w, int h, int n_anchors,
                       int classes);
 
+/* forward_region_layer_gpu, inference part (src/region_layer.c:439-485 on the GPU; the CPU form
+ * :158-184 defines the result): copy, logistic on x, y, on objectness unless `background`, and
+ * on the classes unless `softmax`, in which case softmax_cpu runs over the classes (+background)
+ * of every (image, anchor, cell) with stride w*h.  Layout [b][anchor][coords+1+classes][h][w]. */
+void forward_region_gpu(const float *input, float *output, int batch, int w, int h, int n_anchors,
+                        int classes, int coords, int background, int softmax);
+
 /* forward_avgpool_layer_gpu (src/avgpool_layer_kernels.cu:46-54). */
 void forward_avgpool_gpu(const float *input, float *output, int batch, int c, int h, int w);
 
@@ -235,6 +242,15 @@ void letterbox_image_gpu(const float *im, int w, int h, int c, float *boxed, int
 void yolo_decode_gpu(const float *layer_output, int lw, int lh, int n, int classes,
                      const float *anchors, int netw, int neth, int w, int h, int relative,
                      float thresh, float *rows, int max_rows, int *count);
+
+/* The same for ONE region head (yolov2), get_region_detections src/region_layer.c:364-437 with
+ * get_region_box :76-84 and correct_region_boxes :336-362: all lw*lh*n rows are written, row
+ * anchor*lw*lh + cell after the `*count` rows already there (the reference returns every anchor
+ * of every cell; objectness at or below `thresh` is stored as 0 and leaves the probabilities
+ * 0); anchors: HOST, the layer's 2*n biases, in cell units.  coords must be 4. */
+void region_decode_gpu(const float *layer_output, int lw, int lh, int n, int classes, int coords,
+                       int background, const float *anchors, int netw, int neth, int w, int h,
+                       int relative, float thresh, float *rows, int max_rows, int *count);
 
 /* do_nms_sort (src/box.c:58-89) on device rows, in place: per class, in descending
  * probability (ties: lower row first), a row zeroes that class's probability in every later row

@@ -22,7 +22,7 @@ SECTION_ALIASES = {
     "[soft]": "softmax", "[softmax]": "softmax",
     "[route]": "route", "[shortcut]": "shortcut", "[upsample]": "upsample", "[yolo]": "yolo",
     "[conn]": "connected", "[connected]": "connected", "[dropout]": "dropout", "[reorg]": "reorg",
-    "[crop]": "crop", "[cost]": "cost",
+    "[crop]": "crop", "[cost]": "cost", "[region]": "region",
     "[net]": "net", "[network]": "net",
 }
 
@@ -137,6 +137,22 @@ def parse(text: str) -> dict:
                      inputs=h * w * c, outputs=oh * ow * oc)
             if extra:
                 L.update(out_h=0, out_w=0, out_c=0, outputs=h * w * c + extra)
+        elif kind == "region":
+            # parse_region src/parser.c:353-403, make_region_layer src/region_layer.c:13-56
+            if "tree" in o or "map" in o:
+                raise NotImplementedError("region layer with tree/map")
+            coords, classes, num = gi(o, "coords", 4), gi(o, "classes", 20), gi(o, "num", 1)
+            anchors = [0.5] * (2 * num)
+            if "anchors" in o:
+                for i, t in enumerate(o["anchors"].split(",")):
+                    if i < 2 * num:
+                        anchors[i] = _atof(t)
+            L.update(n=num, classes=classes, coords=coords, softmax=gi(o, "softmax", 0),
+                     background=gi(o, "background", 0), anchors=anchors,
+                     c=num * (classes + coords + 1), out_h=h, out_w=w, out_c=num * (classes + coords + 1))
+            L["outputs"] = h * w * L["out_c"]
+            if L["outputs"] != inputs:
+                raise ValueError("region layer: outputs != inputs")
         elif kind == "upsample":
             stride = gi(o, "stride", 2)
             L.update(stride=stride, scale=gf(o, "scale", 1.0),

@@ -235,6 +235,25 @@ class Oracle:
         self.lib.orc_letterbox_image(_fp(im), w, h, c, _fp(out), bw, bh)
         return out
 
+    def region(self, x, n_anchors, classes, coords=4, background=0, softmax=1):
+        x = np.ascontiguousarray(x, np.float32)
+        b, c, h, w = x.shape
+        assert c == n_anchors * (coords + classes + 1)
+        out = np.empty_like(x)
+        self.lib.orc_region(_fp(x), _fp(out), b, w, h, n_anchors, classes, coords, background, softmax)
+        return out
+
+    def region_detections(self, pred, n_anchors, classes, coords, background, biases, netw, neth, w, h, relative,
+                          thresh):
+        """get_region_detections on image 0 of `pred` -> all lw*lh*n rows [*, 5 + classes]."""
+        pred = np.ascontiguousarray(pred, np.float32)
+        lh, lw = pred.shape[-2:]
+        rows = np.zeros((lw * lh * n_anchors, 5 + classes), np.float32)
+        bi = np.ascontiguousarray(biases, np.float32)
+        self.lib.orc_region_detections(_fp(pred), lw, lh, n_anchors, classes, coords, background, _fp(bi), netw,
+                                       neth, w, h, relative, C.c_float(thresh), _fp(rows))
+        return rows
+
     def yolo_detections(self, pred, n_anchors, classes, biases, mask, netw, neth, w, h, relative, thresh):
         """get_yolo_detections on image 0 of `pred` [n*(5+classes), lh, lw] -> rows [count, 5+classes]."""
         pred = np.ascontiguousarray(pred, np.float32)

@@ -52,6 +52,9 @@ class OracleNet:
             return o.avgpool(x.reshape(b, L["c"], L["h"], L["w"]))
         if t == "softmax":
             return o.softmax(x.reshape(b, -1), L["groups"], L["temperature"])
+        if t == "region":
+            return o.region(x.reshape(b, L["c"], L["h"], L["w"]), L["n"], L["classes"], L["coords"],
+                            L["background"], L["softmax"])
         if t == "connected":
             w, bi, sc, mu, var = self.params[i]
             return o.connected(x.reshape(b, -1), w, bi, sc, mu, var, outputs=L["outputs"],
@@ -85,6 +88,13 @@ class OracleNet:
         rows = []
         classes = 0
         for i, L in enumerate(self.layers):
+            if L["type"] == "region":
+                classes = L["classes"]
+                pred = np.asarray(outs[i], np.float32).reshape(L["batch"], L["c"], L["h"], L["w"])[image]
+                rows.append(self.orc.region_detections(pred, L["n"], classes, L["coords"], L["background"],
+                                                       L["anchors"], self.net["w"], self.net["h"], w, h, relative,
+                                                       thresh))
+                continue
             if L["type"] != "yolo":
                 continue
             classes = L["classes"]

@@ -672,3 +672,101 @@ void orc_letterbox_image(const float *im, int imw, int imh, int imc, float *boxe
             }
     free(resized);
 }
+
+/* ---- forward_region_layer, inference part of the CPU build: src/region_layer.c:158-184 with
+ * entry_index :150-155 and softmax_cpu / softmax src/blas.c:305-332 (temp 1, stride w*h). ----- */
+void orc_region(const float *input, float *output, int batch, int w, int h, int n_anchors, int classes,
+                int coords, int background, int softmax)
+{
+    const long plane = (long)w * h;
+    const long entries = coords + classes + 1;
+    const long outputs = plane * entries * n_anchors;
+    memcpy(output, input, sizeof(float) * (size_t)(outputs * batch));
+    for (int b = 0; b < batch; ++b)
+        for (int n = 0; n < n_anchors; ++n) {
+            float *base = output + b * outputs + n * plane * entries;
+            orc_activate_array(base, 2 * plane, 0);
+            if (!background) orc_activate_array(base + coords * plane, plane, 0);
+            if (!softmax) orc_activate_array(base + (coords + 1) * plane, classes * plane, 0);
+        }
+    if (softmax) {
+        const long first = (coords + !background) * plane;
+        const int cnt = classes + background;
+        for (long g = 0; g < (long)batch * n_anchors; ++g)
+            for (long cell = 0; cell < plane; ++cell) {
+                const float *x = input + g * (outputs / n_anchors) + first + cell;
+                float *y = output + g * (outputs / n_anchors) + first + cell;
+                float sum = 0;
+                float largest = -FLT_MAX;
+                for (int i = 0; i < cnt; ++i)
+                    if (x[i * plane] > largest) largest = x[i * plane];
+                for (int i = 0; i < cnt; ++i) {
+                    float e = exp(x[i * plane] / 1.f - largest / 1.f);
+                    sum += e;
+                    y[i * plane] = e;
+                }
+                for (int i = 0; i < cnt; ++i) y[i * plane] /= sum;
+            }
+    }
+}
+
+/* ---- get_region_detections: src/region_layer.c:364-437 (no tree, no map, coords 4) for image 0
+ * of `pred`; writes all lw*lh*n rows, row anchor*lw*lh + cell. -------------------------------- */
+int orc_region_detections(const float *pred, int lw, int lh, int n, int classes, int coords, int background,
+                          const float *biases, int netw, int neth, int w, int h, int relative, float thresh,
+                          float *rows)
+{
+    const int cells = lw * lh;
+    const int entries = coords + classes + 1;
+    const int out_entries = 5 + classes;
+    for (int i = 0; i < cells; ++i) {
+        const int row = i / lw;
+        const int col = i % lw;
+        for (int a = 0; a < n; ++a) {
+            const int index = a * cells + i;
+            float *r = rows + (long)index * out_entries;
+            const float *p = pred + (long)a * cells * entries + i;
+            for (int j = 0; j < classes; ++j) r[5 + j] = 0;
+            const float scale = background ? 1 : p[(long)coords * cells];
+            r[0] = (col + p[0]) / lw;
+            r[1] = (row + p[1L * cells]) / lh;
+            r[2] = exp(p[2L * cells]) * biases[2 * a] / lw;
+            r[3] = exp(p[3L * cells]) * biases[2 * a + 1] / lh;
+            r[4] = scale > thresh ? scale : 0;
+            if (r[4]) {
+                for (int j = 0; j < classes; ++j) {
+                    const float prob = scale * p[(long)(coords + 1 + j) * cells];
+                    r[5 + j] = (prob > thresh) ? prob : 0;
+                }
+            }
+        }
+    }
+    /* correct_region_boxes :336-362 */
+    int new_w = 0, new_h = 0;
+    if (((float)netw / w) < ((float)neth / h)) {
+        new_w = netw;
+        new_h = (h * netw) / w;
+    } else {
+        new_h = neth;
+        new_w = (w * neth) / h;
+    }
+    for (int i = 0; i < cells * n; ++i) {
+        float *r = rows + (long)i * out_entries;
+        float bx = r[0], by = r[1], bw = r[2], bh = r[3];
+        bx = (bx - (netw - new_w) / 2. / netw) / ((float)new_w / netw);
+        by = (by - (neth - new_h) / 2. / neth) / ((float)new_h / neth);
+        bw *= (float)netw / new_w;
+        bh *= (float)neth / new_h;
+        if (!relative) {
+            bx *= w;
+            bw *= w;
+            by *= h;
+            bh *= h;
+        }
+        r[0] = bx;
+        r[1] = by;
+        r[2] = bw;
+        r[3] = bh;
+    }
+    return cells * n;
+}

@@ -81,6 +81,12 @@ void orc_crop(const float *input, float *output, int batch, int c, int h, int w,
 void orc_resize_image(const float *im, int imw, int imh, int imc, float *resized, int w, int h);
 void orc_letterbox_image(const float *im, int imw, int imh, int imc, float *boxed, int w, int h);
 
+void orc_region(const float *input, float *output, int batch, int w, int h, int n_anchors, int classes,
+                int coords, int background, int softmax);
+int orc_region_detections(const float *pred, int lw, int lh, int n, int classes, int coords, int background,
+                          const float *biases, int netw, int neth, int w, int h, int relative, float thresh,
+                          float *rows);
+
 /* detections (test infrastructure like everything here): see oracle.c */
 int orc_yolo_detections(const float *pred, int lw, int lh, int n, int classes, const float *biases,
                         const int *mask, int netw, int neth, int w, int h, int relative, float thresh,

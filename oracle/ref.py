@@ -137,7 +137,7 @@ class RefNet:
     def get_boxes(self, w, h, thresh, relative=1, nms=0.0):
         """get_network_boxes (+ do_nms_sort when nms > 0) -> rows [n, 5 + classes]."""
         classes = self.layers[-1]["classes"]
-        cap = sum(L["w"] * L["h"] * L["n"] for L in self.layers if L["type"] == "yolo")
+        cap = sum(L["w"] * L["h"] * L["n"] for L in self.layers if L["type"] in ("yolo", "region"))
         rows = np.zeros((max(cap, 1), 5 + classes), np.float32)
         n = self.h.refh_get_boxes(self.net, w, h, thresh, relative, nms, rows.ctypes.data_as(_F), cap)
         return rows[:n].copy()

@@ -19,10 +19,11 @@ seeded synthetic inputs; nothing from the reference's sources is stored.  Fixtur
   small_net2.cfg/.weights/.npz  the same for a network of crop, reorg (plain, reverse, flatten,
                          extra), dropout, connected (with and without batch-norm), softmax, cost
   image_cases.npz        letterbox_image / resize_image of small images (down, up, both aspects)
+  region_case.npz        a yolov2-style region head (region_net.cfg): layer input/output, boxes, NMS
   detections_case.npz    the two yolo tensors of a yolov3-tiny forward at 96x96 and what
                          get_network_boxes / do_nms_sort make of them (rows x,y,w,h,obj,prob[80])
 
-`python tests/golden/make_golden.py detections|small_net2|images` rewrites only that fixture.
+`python tests/golden/make_golden.py detections|small_net2|images|region` rewrites only that fixture.
 """
 import json
 import os
@@ -213,6 +214,25 @@ def images_fixture():
     np.savez_compressed(os.path.join(HERE, "image_cases.npz"), **data)
 
 
+REGION_CASES = {"square": (64, 96, 0.3, 1, 0.0), "wide_abs": (200, 100, 0.25, 0, 0.0),
+                "wide_abs_nms": (200, 100, 0.2, 0, 0.4)}
+
+
+def region_fixture():
+    """A yolov2-style head (region_net.cfg, written by hand next to this script): the region layer's
+    input and output, and what get_network_boxes / do_nms_sort make of it (NMS rows: objectness > 0,
+    canonical order)."""
+    r = ref.RefNet(os.path.join(HERE, "region_net.cfg"))
+    fill_params(r.set_conv, r.layers, seed=40, bn="random")
+    outs = r.predict(synth.uniform01(3, r.inputs * r.batch))
+    data = {"region_in": outs[-2], "region_out": outs[-1]}
+    for name, (w, h, thresh, relative, nms) in REGION_CASES.items():
+        rows = r.get_boxes(w, h, thresh, relative, nms)
+        data[name] = rows if nms == 0 else lexsorted(rows[rows[:, 4] > 0])
+        data[name + "_spec"] = np.array([w, h, thresh, relative, nms], np.float64)
+    np.savez_compressed(os.path.join(HERE, "region_case.npz"), **data)
+
+
 def lexsorted(rows):
     """Rows in a canonical order (the reference leaves its array sorted by the last class after NMS)."""
     if len(rows) == 0:
@@ -244,6 +264,10 @@ def main():
         detections_fixture()
         print("detections_case.npz written")
         return
+    if sys.argv[1:] == ["region"]:
+        region_fixture()
+        print("region_case.npz written")
+        return
     if sys.argv[1:] == ["images"]:
         images_fixture()
         print("image_cases.npz written")
@@ -256,6 +280,7 @@ def main():
         return
     detections_fixture()
     images_fixture()
+    region_fixture()
     # ---- layer tables
     tables = {}
     for name, text in [("yolov3-tiny-416", cfgs.yolov3_tiny(1, 416)), ("yolov3-416", cfgs.yolov3(1, 416)),

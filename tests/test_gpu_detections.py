@@ -14,7 +14,7 @@ from darknet_amd import api, cfgs, synth
 from oracle.cpu import Oracle
 from oracle.net import OracleNet
 
-from util import fill_params
+from util import REL_TOL, fill_params, norm_err
 
 pytestmark = pytest.mark.gpu
 GOLD = os.path.join(os.path.dirname(__file__), "golden")
@@ -115,4 +115,59 @@ def test_network_boxes_against_checker_on_the_librarys_own_outputs(dn):
     # an impossible threshold: no detections, valid empty result
     assert net.get_boxes(160, 160, 2.0).shape == (0, 85)
     assert net.L.num_detections(net.net, 2.0) == 0
+    net.free()
+
+
+# ---- region head (yolov2) ----------------------------------------------------------------------
+def test_region_forward_and_decode_on_the_reference_golden_tensors(dn):
+    g = np.load(os.path.join(GOLD, "region_case.npz"))
+    text = open(os.path.join(GOLD, "region_net.cfg")).read()
+    onet = OracleNet(text)
+    L = onet.layers[-1]
+    x = D(g["region_in"])
+    y = D(n=g["region_in"].size)
+    dn.forward_region_gpu(x.ptr, y.ptr, 1, L["w"], L["h"], L["n"], L["classes"], L["coords"], L["background"],
+                          L["softmax"])
+    got = y.numpy(g["region_out"].shape)
+    assert np.abs(got - g["region_out"]).max() <= 1e-6          # logistic / exp: device libm vs glibc
+    assert np.array_equal(got.reshape(6, 9, -1)[:, 2:4], g["region_in"].reshape(6, 9, -1)[:, 2:4])
+    # decode the REFERENCE's region output, so that every threshold decision is on identical inputs
+    pred = D(g["region_out"])
+    an = np.array(L["anchors"], np.float32)
+    cap = L["w"] * L["h"] * L["n"]
+    for name in [k[:-5] for k in g.files if k.endswith("_spec")]:
+        w, h, thresh, relative, nms = g[name + "_spec"]
+        rows = D(n=cap * 9)
+        cnt = dn.hip_make_int_array(None, 1)
+        dn.region_decode_gpu(pred.ptr, L["w"], L["h"], L["n"], L["classes"], 4, 0, an.ctypes.data_as(api._F), 64, 96,
+                             int(w), int(h), int(relative), float(thresh), rows.ptr, cap, cnt)
+        assert device_count(dn, cnt) == cap
+        if nms > 0:
+            dn.nms_sort_gpu(rows.ptr, cap, L["classes"], float(nms))
+        r = rows.numpy((cap, 9))
+        if nms > 0:
+            r = r[r[:, 4] > 0]
+            r = r[np.lexsort(r[:, :5].T[::-1])]
+            assert np.array_equal(r[:, 4], g[name][:, 4])
+        check_rows(r, g[name])
+        dn.hip_free(cnt)
+
+
+def test_region_network_boxes_against_checker(dn):
+    text = open(os.path.join(GOLD, "region_net.cfg")).read().replace("batch=1", "batch=3")
+    net = api.Network(cfg_text=text)
+    onet = OracleNet(text)
+    fill_params(net.set_conv, net.layers, seed=40, bn="random")
+    fill_params(onet.set_conv, onet.layers, seed=40, bn="random")
+    x = synth.uniform01(3, net.inputs * 3)
+    net.predict(x)
+    want = onet.forward(x)
+    for i in range(net.n):
+        assert norm_err(net.layer_output(i), want[i]) <= REL_TOL, i
+    outs = [None] * (net.n - 1) + [net.layer_output(net.n - 1)]
+    check_rows(net.get_network_boxes(200, 100, 0.25, relative=0), onet.get_boxes(outs, 200, 100, 0.25, 0, 0.0))
+    for image in (1, 2):
+        got = net.get_boxes(200, 100, 0.2, 0, 0.4, image)
+        check_rows(got, onet.get_boxes(outs, 200, 100, 0.2, 0, 0.4, image))
+        assert (got[:, 5:] > 0).sum() > 100
     net.free()

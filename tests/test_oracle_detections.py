@@ -150,3 +150,77 @@ def test_nms_matches_brute_force_on_grid_boxes():
         want[live] = brute_force_nms(rows[live], classes, thresh)
         assert np.array_equal(got, want)
         assert (got[:, 5:] != rows[:, 5:]).sum() > (100 if thresh < 0.3 else 5)
+
+
+# ---- region head (yolov2) ----------------------------------------------------------------------
+REGION_CFG = open(os.path.join(GOLD, "region_net.cfg")).read()
+
+
+def test_region_forward_and_boxes_match_golden():
+    g = np.load(os.path.join(GOLD, "region_case.npz"))
+    net = OracleNet(REGION_CFG)
+    L = net.layers[-1]
+    assert L["type"] == "region" and L["softmax"] == 1 and L["n"] == 6
+    out = net.forward_layer(net.net["n"] - 1, g["region_in"], None)
+    assert np.array_equal(np.ascontiguousarray(out).reshape(1, -1), g["region_out"])
+    outs = [None] * (net.net["n"] - 1) + [g["region_out"]]
+    for name in [k[:-5] for k in g.files if k.endswith("_spec")]:
+        w, h, thresh, relative, nms = g[name + "_spec"]
+        rows = net.get_boxes(outs, int(w), int(h), float(thresh), int(relative), float(nms))
+        if nms > 0:
+            rows = lexsorted(rows[rows[:, 4] > 0])
+        assert np.array_equal(rows, g[name]), name
+    assert (g["wide_abs_nms"][:, 5:] > 0).sum() > 300
+
+
+@pytest.mark.skipif(not ref.available(), reason="oracle/_ref (compiled reference) not built")
+def test_region_matches_compiled_reference():
+    p = write_cfg(REGION_CFG.replace("softmax=1", "softmax=0").replace("height=96", "height=64"))
+    r = ref.RefNet(p)
+    text = open(p).read()
+    os.unlink(p)
+    o = OracleNet(text)
+    fill_params(r.set_conv, o.layers, seed=77)
+    fill_params(o.set_conv, o.layers, seed=77)
+    x = synth.uniform01(8, r.inputs)
+    ro, oo = r.predict(x), o.forward(x)
+    assert np.array_equal(ro[-1].reshape(-1), oo[-1].reshape(-1))          # logistic class scores
+    assert np.array_equal(r.get_boxes(100, 80, 0.3, 1, 0.0), o.get_boxes(ro, 100, 80, 0.3, 1, 0.0))
+
+
+def test_region_forward_properties():
+    o = Oracle()
+    n, classes = 3, 5
+    x = synth.uniform(2, 2 * n * (5 + classes) * 4 * 6, -3, 3).reshape(2, n * (5 + classes), 4, 6)
+    y = o.region(x, n, classes, softmax=1).reshape(2, n, 5 + classes, 4, 6)
+    xv = x.reshape(2, n, 5 + classes, 4, 6).astype(np.float64)
+    assert np.allclose(y[:, :, 5:].sum(axis=2), 1.0, atol=1e-6)                      # softmax over classes
+    e = np.exp(xv[:, :, 5:] - xv[:, :, 5:].max(axis=2, keepdims=True))
+    assert np.abs(y[:, :, 5:] - e / e.sum(axis=2, keepdims=True)).max() <= 1e-6
+    assert np.abs(y[:, :, [0, 1, 4]] - 1 / (1 + np.exp(-xv[:, :, [0, 1, 4]]))).max() <= 1e-6
+    assert np.array_equal(y[:, :, 2:4], x.reshape(2, n, 5 + classes, 4, 6)[:, :, 2:4])   # w, h stay raw
+    # without softmax the classes get the logistic; with background the objectness stays raw
+    y2 = o.region(x, n, classes, softmax=0).reshape(2, n, 5 + classes, 4, 6)
+    assert np.abs(y2[:, :, 5:] - 1 / (1 + np.exp(-xv[:, :, 5:]))).max() <= 1e-6
+    y3 = o.region(x, n, classes, background=1, softmax=1).reshape(2, n, 5 + classes, 4, 6)
+    assert np.allclose(y3[:, :, 4:].sum(axis=2), 1.0, atol=1e-6)                     # softmax spans objectness too
+
+
+def test_region_decode_closed_form():
+    """Anchors are in cell units and divided by the LAYER size (yolo: pixels / network size)."""
+    o = Oracle()
+    lw, lh, n, classes = 4, 3, 2, 3
+    pred = np.zeros((n * (5 + classes), lh, lw), np.float32)
+    a, row, col = 1, 2, 3
+    base = a * (5 + classes)
+    pred[base + 0:base + 5, row, col] = [0.25, 0.75, np.log(2.0), 0.0, 0.75]
+    pred[base + 5:base + 8, row, col] = [0.5, 1.0, 0.125]
+    rows = o.region_detections(pred, n, classes, 4, 0, [1, 2, 1.5, 0.75], 128, 96, 256, 192, 1, 0.3)
+    assert rows.shape == (lw * lh * n, 8)
+    r = rows[a * lw * lh + row * lw + col]                      # anchor-major row index
+    assert (r[0], r[1]) == (np.float32(3.25) / 4, np.float32(2.75) / 3)
+    assert abs(r[2] - 2.0 * 1.5 / 4) < 1e-7 and r[3] == np.float32(0.75 / 3)
+    assert r[4] == 0.75 and list(r[5:]) == [0.375, 0.75, 0.0]
+    others = np.delete(rows, a * lw * lh + row * lw + col, axis=0)
+    assert not others[:, 4:].any()                              # objectness 0 <= thresh: stored as 0, no classes
+    assert np.all(others[:, 2] > 0)                             # but every cell still has its box
