@@ -104,4 +104,4 @@ def test_every_in_scope_reference_cfg_parses_identically():
         theirs = ref.RefNet(path).layers
         same_table(theirs, mine, os.path.basename(path))
         done += 1
-    assert done >= 33
+    assert done >= 37
