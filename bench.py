@@ -7,8 +7,8 @@ forward_network_gpu, src/network.c:773-785, without the host<->device copies aro
 Default workload: yolov3 at 416x416, batch 64, fp32 - the configuration the headline metric is
 quoted on.  Prints ONE JSON line on stdout; progress goes to stderr.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload yolov3-416|yolov3-tiny-416|
-                    resnext50-224|yolov3-608] [--batch B] [--per-layer FILE] [--no-cpu]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload yolov3-416|yolov3-608|yolov3-tiny-416|
+                    yolov3-tiny-xnor-416|resnext50-224] [--batch B] [--per-layer FILE] [--no-cpu]
 
 The line carries, besides the driver's fields:
   roofline      the dominant kernel's algorithmic FLOP/s against the fp32 MFMA peak, from HIP
@@ -39,7 +39,15 @@ WORKLOADS = {
     "yolov3-608": ("yolov3", 608),
     "yolov3-tiny-416": ("yolov3_tiny", 416),
     "resnext50-224": ("resnext50", 224),
+    "yolov3-tiny-xnor-416": ("yolov3_tiny_xnor", 416),
 }
+
+
+def cfg_generator(cfg_name):
+    from darknet_amd import cfgs
+    if cfg_name == "yolov3_tiny_xnor":       # binary=1 xnor=1 on every conv but the first and the last
+        return lambda batch, size: cfgs.yolov3_tiny(batch, size, xnor=True)
+    return getattr(cfgs, cfg_name)
 
 
 def log(*a):
@@ -96,7 +104,7 @@ def cpu_baseline(kind_pref, cfg_name, size, budget_s=20.0):
     from darknet_amd import cfgs, synth
     from oracle import ref
     threads = int(os.environ.get("OMP_NUM_THREADS", os.cpu_count() or 1))
-    gen = getattr(cfgs, cfg_name)
+    gen = cfg_generator(cfg_name)
     if kind_pref == "reference" and ref.available("fast"):
         kind = "reference"
 
@@ -168,7 +176,7 @@ def main():
     from darknet_amd import api, cfgs, synth
 
     cfg_name, size = WORKLOADS[args.workload]
-    text = getattr(cfgs, cfg_name)(args.batch, size)
+    text = cfg_generator(cfg_name)(args.batch, size)
     api.set_gpu(0)
     L = api._lib.load()
     dev = L.hip_device_name().decode()

@@ -76,6 +76,9 @@ struct mfma_args {
      * whole_tiles + j / split and leaves raw accumulators in `partial` for the reduce kernel */
     int whole_tiles, split;
     float *partial;
+    /* grouped layers (see conv_grouped_tile): every 32-filter tile reads its own 32 input
+     * channels and its own block of packed weights; 0 for ordinary layers */
+    int grouped;
     /* fused residual add (null = none): sum[i] = act2(s1*out[i] + s2*add[i]) over the same
      * geometry as out, the arithmetic of src/blas.c:36 followed by src/shortcut_layer.c:64 */
     const float *add;
@@ -359,7 +362,7 @@ __global__ __launch_bounds__(DN_THREADS, (BM == 128 ? 3 : 2)) void conv_mfma_ker
         }
     }
     /* tap-blocked loop state of the chunk being fetched (wave-uniform) */
-    int ld_cb = kc_begin / TAPS, ld_tap = kc_begin - (kc_begin / TAPS) * TAPS;
+    int ld_cb = kc_begin / TAPS + (a.grouped ? tile_m * 2 : 0), ld_tap = kc_begin - (kc_begin / TAPS) * TAPS;
 
     typedef __attribute__((address_space(3))) void *lds_ptr;
 
@@ -380,7 +383,9 @@ __global__ __launch_bounds__(DN_THREADS, (BM == 128 ? 3 : 2)) void conv_mfma_ker
                     /* BM == 32: one wave-load covers two slots of 32 rows each */
                     const int q2 = wl * 2 + (lane >> 5);
                     const unsigned voff = (unsigned)((((long)q2 * a.Mpad) + (lane & 31)) * 16);
-                    const unsigned soff = (unsigned)(((long)kc * 4 * a.Mpad + m0) * 16);
+                    /* grouped: Mpad == 32 and the tile's chunks follow each other */
+                    const unsigned soff = a.grouped ? (unsigned)(((long)(tile_m * a.KCH + kc) * 4 * 32) * 16)
+                                                    : (unsigned)(((long)kc * 4 * a.Mpad + m0) * 16);
                     __builtin_amdgcn_raw_ptr_buffer_load_lds(w_rsrc, (lds_ptr)&(buf ? As1 : As0)[(wl * 2 * BM) * 4], 16, voff,
                                                              soff, 0, 0);
                 }
@@ -603,6 +608,44 @@ __global__ void pack_weights_kernel(const float *w, float *packed, int M, int K,
     }
 }
 
+/* Grouped layers whose groups have as many filters as channels, at most 32 of each (ResNeXt's
+ * 32-group 3x3: 4, 8, 16 or 32 per group): filters [32t, 32t+32) then read exactly input
+ * channels [32t, 32t+32), so tile t is a dense 32 x (32*taps) GEMM over those channels with
+ * block-diagonal weights (zeros between groups).  The zeros cost 32/cg times the layer's nominal
+ * FLOPs on the matrix cores, which is still 10-50x less time than a per-group direct loop, and
+ * nothing at all at 32 channels per group.  Returns taps (9 or 1), 0 if the layer does not fit. */
+static inline int conv_grouped_tile(int n, int c, int groups, int size)
+{
+    if (groups <= 1 || n % groups || c % groups) return 0;
+    const int cg = c / groups, fg = n / groups;
+    if (cg != fg || cg > 32 || (32 % cg) != 0 || (n % 32) != 0) return 0;
+    if (size == 3) return 9;
+    if (size == 1) return 1;
+    return 0;
+}
+
+/* packed[((tile*KCH + chunk)*4 + slot)*32 + r][j]: filter 32*tile + r, tap-blocked k inside the
+ * tile's 32 channels; weights are [n][cg][size*size] */
+__global__ void pack_grouped_kernel(const float *w, float *packed, int cg, int taps, long total)
+{
+    const int kch = 2 * taps;
+    for (long i = blockIdx.x * (long)blockDim.x + threadIdx.x; i < total; i += (long)gridDim.x * blockDim.x) {
+        const int j = (int)(i & 3);
+        long t = i >> 2;
+        const int r = (int)(t & 31);
+        t >>= 5;
+        const int q = (int)(t & 3);
+        t >>= 2;
+        const int kc = (int)(t % kch);
+        const int tile = (int)(t / kch);
+        const int cb = kc / taps, tap = kc - cb * taps;
+        const int ch = cb * DN_BK + q * 4 + j;  /* channel inside the tile, 0..31 */
+        const int f = tile * 32 + r;             /* filter */
+        const bool same_group = (r / cg) == (ch / cg);
+        packed[i] = same_group ? w[((long)f * cg + (ch % cg)) * taps + tap] : 0.f;
+    }
+}
+
 /* K order of a layer, from the layer geometry alone so that packing and forward agree. */
 static inline int tap_blocked_taps(int c, int groups, int size)
 {
@@ -614,6 +657,8 @@ static inline int tap_blocked_taps(int c, int groups, int size)
 
 extern "C" size_t conv_packed_floats(int n, int c, int groups, int size)
 {
+    const int gt = conv_grouped_tile(n, c, groups, size);
+    if (gt) return (size_t)(n / 32) * (size_t)(2 * gt) * DN_BK * 32;
     if (groups != 1) return 0;
     const long K = (long)c * size * size;
     const long kch = (K + DN_BK - 1) / DN_BK;
@@ -625,6 +670,15 @@ extern "C" void conv_pack_weights_gpu(const float *weights, float *packed, int n
 {
     const size_t total = conv_packed_floats(n, c, groups, size);
     if (!total) return;
+    const int gt = conv_grouped_tile(n, c, groups, size);
+    if (gt) {
+        long gb = (long)((total + 255) / 256);
+        if (gb > 8192) gb = 8192;
+        hipLaunchKernelGGL(pack_grouped_kernel, dim3((int)gb), dim3(256), 0, dn_stream(), weights, packed,
+                           c / groups, gt, (long)total);
+        dn_check_launch("conv_pack_weights_gpu");
+        return;
+    }
     const int K = c * size * size;
     const int mpad = (n + DN_MPAD - 1) / DN_MPAD * DN_MPAD;
     long blocks = (long)((total + 255) / 256);
@@ -644,6 +698,10 @@ extern "C" const char *conv_kernel_name(int n, int c, int groups, int size)
 {
     static char name[96];
     const int mode = conv_mode(c, groups, size, 1, size / 2, 0);
+    if (conv_grouped_tile(n, c, groups, size) && g_algo != 1) {
+        snprintf(name, sizeof name, "conv_mfma_kernel<32,256,32,64,%d>", size == 3 ? 13 : 11);
+        return name;
+    }
     if (mode < 0) return "conv_direct_kernel";
     if (n <= 32)
         snprintf(name, sizeof name, "conv_mfma_kernel<32,256,32,64,%d>", mode);
@@ -782,6 +840,10 @@ static void conv_forward(const float *input, const float *weights, const float *
 
     const long K = (long)(c / groups) * size * size;
     int mode = conv_mode(c, groups, size, stride, pad, (long)batch * c * h * w * 4);
+    /* grouped layers that fit the 32-filter block-diagonal scheme run on the tap-blocked kernel */
+    const int gtaps = (g_algo != 1 && (long)batch * c * h * w * 4 + (1L << 20) < (1L << 32) &&
+                       !(size == 3 && pad != 1)) ? conv_grouped_tile(n, c, groups, size) : 0;
+    if (gtaps) mode = 10 + size;
     if ((long)batch * oh * ow >= (1L << 31) - 512) mode = -1; /* the MFMA kernels index columns in 32 bits */
     if (mode < 0) {
         conv_direct_forward(input, weights, biases, scales, rolling_mean, rolling_variance, output, batch, c,
@@ -826,6 +888,13 @@ static void conv_forward(const float *input, const float *weights, const float *
     a.K = (int)K;
     a.KCH = (int)((K + DN_BK - 1) / DN_BK);
     a.Mpad = (n + DN_MPAD - 1) / DN_MPAD * DN_MPAD;
+    a.grouped = 0;
+    if (gtaps && mode >= 10) { /* per 32-filter tile: 32 channels x taps */
+        a.grouped = 1;
+        a.K = 32 * gtaps;
+        a.KCH = 2 * gtaps;
+        a.Mpad = 32;
+    }
     a.P = oh * ow;
     a.OW = ow;
     a.Ntotal = (long)batch * a.P;
@@ -847,7 +916,7 @@ static void conv_forward(const float *input, const float *weights, const float *
     a.sum_slope_lo = conv_split(sum_slope).lo;
     a.in_records = (unsigned)((long)batch * c * h * w * 4 + (long)(w + 1) * 4);
     a.wp_records = (unsigned)(conv_packed_floats(n, c, groups, size) * 4);
-    if (n <= 32)
+    if (n <= 32 || a.grouped)
         launch_tile<32, 256, 32, 64>(a, mode);
     else if (n <= 64)
         launch_tile<64, 256, 64, 64>(a, mode);

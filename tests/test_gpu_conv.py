@@ -54,6 +54,12 @@ SHAPES = [  # b, c, h, w, n, size, stride, pad, groups, act
     (2, 128, 14, 14, 128, 3, 1, 1, 32, "leaky"),    # resnext grouped 3x3, 4 channels per group
     (2, 256, 14, 14, 256, 3, 2, 1, 32, "leaky"),    # grouped, stride 2
     (1, 16, 1, 1, 16, 3, 1, 1, 1, "leaky"),         # 1x1 image
+    (2, 512, 7, 7, 512, 3, 1, 1, 32, "leaky"),      # grouped, 16 per group (block-diagonal MFMA tiles)
+    (1, 1024, 9, 7, 1024, 3, 2, 1, 32, "leaky"),    # grouped, 32 per group: one group per tile, stride 2
+    (3, 64, 10, 10, 64, 1, 1, 0, 16, "linear"),     # grouped 1x1, 4 per group
+    (2, 64, 12, 12, 64, 3, 1, 1, 64, "relu"),       # depthwise: 1 per group
+    (2, 48, 9, 9, 96, 3, 1, 1, 3, "leaky"),         # 16 channels -> 32 filters per group: direct kernel
+    (2, 96, 9, 9, 96, 3, 1, 1, 2, "leaky"),         # 48 per group: direct kernel
 ]
 
 
