@@ -78,6 +78,7 @@ layer make_convolutional_layer(int batch, int h, int w, int c, int n, int groups
         l.xnor_wbits_gpu = (unsigned *)hip_make_int_array(0, xnor_weight_words(n, c, size));
         l.xnor_xbits_gpu = (unsigned *)hip_make_int_array(0, xnor_input_words(batch, c, h, w));
         l.xnor_wmean_gpu = hip_make_array(0, (size_t)n);
+        xnor_pack_weights_gpu(l.weights_gpu, l.xnor_wbits_gpu, l.xnor_wmean_gpu, n, c, size);
     } else {
         packed = conv_packed_floats(n, c, groups, size);
         if (packed) {
@@ -98,10 +99,11 @@ layer make_convolutional_layer(int batch, int h, int w, int c, int n, int groups
 void forward_convolutional_layer_gpu(layer l, network net)
 {
     if (l.xnor) {
-        forward_convolutional_xnor_gpu(net.input_gpu, l.weights_gpu, l.xnor_wbits_gpu, l.xnor_wmean_gpu,
-                                       l.xnor_xbits_gpu, l.biases_gpu, l.scales_gpu, l.rolling_mean_gpu,
-                                       l.rolling_variance_gpu, l.output_gpu, l.batch, l.c, l.h, l.w, l.n,
-                                       l.size, l.stride, l.pad, l.batch_normalize, (int)l.activation);
+        /* sign bits and mean|w| were written when the weights last changed (push_convolutional_layer) */
+        forward_convolutional_xnor_packed_gpu(net.input_gpu, l.xnor_wbits_gpu, l.xnor_wmean_gpu,
+                                              l.xnor_xbits_gpu, l.biases_gpu, l.scales_gpu, l.rolling_mean_gpu,
+                                              l.rolling_variance_gpu, l.output_gpu, l.batch, l.c, l.h, l.w, l.n,
+                                              l.size, l.stride, l.pad, l.batch_normalize, (int)l.activation);
         return;
     }
     forward_convolutional_gpu(net.input_gpu, l.weights_gpu, l.weights_packed_gpu, l.biases_gpu, l.scales_gpu,
@@ -124,6 +126,7 @@ void push_convolutional_layer(layer l)
     }
     if (l.weights_packed_gpu)
         conv_pack_weights_gpu(l.weights_gpu, l.weights_packed_gpu, l.n, l.c, l.groups, l.size);
+    if (l.xnor_wbits_gpu) xnor_pack_weights_gpu(l.weights_gpu, l.xnor_wbits_gpu, l.xnor_wmean_gpu, l.n, l.c, l.size);
 }
 
 void pull_convolutional_layer(layer l)

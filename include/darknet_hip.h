@@ -156,7 +156,8 @@ void conv_set_algo(int algo);
  * tail.  Replaces the xnor branch of forward_convolutional_layer_gpu
  * (src/convolutional_kernels.cu:77-87) with the CPU semantics of
  * src/convolutional_layer.c:28-49,451-456.
- *   wbits  : scratch, xnor_weight_words(n,c,size) uint32;  wmean: scratch, n floats
+ *   wbits  : scratch, xnor_weight_words(n,c,size) uint32 ([tap][slice][n padded to 16] sign bits, then the
+ *            per-(filter, tap) popcounts);  wmean: scratch, n floats
  *   xbits  : scratch, xnor_input_words(batch,c,h,w) uint32 */
 size_t xnor_weight_words(int n, int c, int size);
 size_t xnor_input_words(int batch, int c, int h, int w);
@@ -168,6 +169,14 @@ void forward_convolutional_xnor_gpu(const float *input, const float *weights, un
                                     const float *rolling_variance, float *output, int batch,
                                     int c, int h, int w, int n, int size, int stride, int pad,
                                     int batch_normalize, int activation);
+/* The same with wbits / wmean already written by xnor_pack_weights_gpu for the current weights
+ * (binarize_weights depends on the weights alone, so a caller that knows when they change - the
+ * natural hook is push_convolutional_layer - packs once instead of on every forward). */
+void forward_convolutional_xnor_packed_gpu(const float *input, const unsigned *wbits, const float *wmean,
+                                           unsigned *xbits, const float *biases, const float *scales,
+                                           const float *rolling_mean, const float *rolling_variance,
+                                           float *output, int batch, int c, int h, int w, int n, int size,
+                                           int stride, int pad, int batch_normalize, int activation);
 
 /* forward_maxpool_layer_gpu (src/maxpool_layer_kernels.cu:87-99), CPU semantics of
  * src/maxpool_layer.c:79-114: window origin (-pad)/2, outside = -FLT_MAX, first maximum wins.

@@ -57,7 +57,12 @@ def test_xnor_pack_bits_and_layer_output(dn, orc, b, c, h, w, n, size, stride):
     want_x = pack_bits((bi.reshape(b, c, h * w) > 0).transpose(0, 2, 1), c)          # [b][hw][cw]
     assert np.array_equal(xbits.reshape(b, -1, h * w).transpose(0, 2, 1), want_x)
     want_w = pack_bits((bw.reshape(n, c, size * size) > 0).transpose(0, 2, 1), c)     # [n][tap][cw]
-    assert np.array_equal(wbits.reshape(n, size * size, -1), want_w)
+    # device layout: [tap][slice][n padded to 16], then the per-(filter, tap) popcounts
+    cw, npad, ss = (c + 31) // 32, (n + 15) // 16 * 16, size * size
+    dev_w = wbits[:ss * cw * npad].reshape(ss, cw, npad)
+    assert np.array_equal(dev_w[:, :, :n].transpose(2, 0, 1), want_w) and not dev_w[:, :, n:].any()
+    pops = np.array([[sum(bin(int(v)).count("1") for v in want_w[f, t]) for t in range(ss)] for f in range(n)])
+    assert np.array_equal(wbits[ss * cw * npad:].view(np.int32).reshape(n, ss), pops)
     assert np.array_equal(wmean, np.abs(bw.reshape(n, -1))[:, 0])                     # mean|w| per filter
     assert norm_err(got, want) <= REL_TOL
 
