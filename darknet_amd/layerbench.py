@@ -19,14 +19,20 @@ from . import lib as _lib
 PEAK = 157.3
 
 
-def time_layer(batch, c, h, w, n, size, stride, pad=None, groups=1, bn=1, act=7, iters=20, warmup=3):
+def time_layer(batch, c, h, w, n, size, stride, pad=None, groups=1, bn=1, act=7, iters=20, warmup=3,
+               data="random"):
     L = _lib.load()
     if pad is None:
         pad = size // 2
     oh = (h + 2 * pad - size) // stride + 1
     ow = (w + 2 * pad - size) // stride + 1
-    x = api.DeviceArray(synth.uniform(1, batch * c * h * w))
-    wt = api.DeviceArray(synth.conv_weights(2, n, c // groups, size))
+    xh = synth.uniform(1, batch * c * h * w)
+    wh = synth.conv_weights(2, n, c // groups, size)
+    if data == "zeros":          # same instruction stream, no operand bits toggling: shows what the
+        xh[:] = 0                # part's clock management costs on real data
+        wh[:] = 0
+    x = api.DeviceArray(xh)
+    wt = api.DeviceArray(wh)
     b, s, m, v = [api.DeviceArray(a) for a in synth.bn_random(3, n)]
     out = api.DeviceArray(n=batch * n * oh * ow)
     pf = L.conv_packed_floats(n, c, groups, size)
@@ -67,6 +73,7 @@ def main():
     ap.add_argument("--iters", type=int, default=20)
     ap.add_argument("--sweep", action="store_true")
     ap.add_argument("--algo", type=int, default=0)
+    ap.add_argument("--data", default="random", choices=["random", "zeros"])
     a = ap.parse_args()
     api.set_gpu(0)
     _lib.load().conv_set_algo(a.algo)
@@ -78,7 +85,8 @@ def main():
                 print(json.dumps(r), flush=True)
     else:
         print(json.dumps(time_layer(a.batch, a.c, a.hw, a.hw, a.n, a.size, a.stride,
-                                    pad=a.size // 2 if a.size > 1 else 0, groups=a.groups, iters=a.iters)),
+                                    pad=a.size // 2 if a.size > 1 else 0, groups=a.groups, iters=a.iters,
+                                    data=a.data)),
               flush=True)
 
 
