@@ -76,7 +76,7 @@ def layer_bytes(L):
         wbytes = 4 * L["nweights"] + (16 * L["n"] if L["batch_normalize"] else 4 * L["n"])
         return 4 * b * (L["inputs"] + L["outputs"]) + wbytes
     if t == "maxpool":
-        return 4 * b * (L["inputs"] + 2 * L["outputs"])  # output + indexes
+        return 4 * b * (L["inputs"] + L["outputs"])  # inference leaves the argmax indexes out
     if t == "shortcut":
         add = min(L["c"], L["out_c"]) * min(L["h"], L["out_h"]) * min(L["w"], L["out_w"])
         return 4 * b * (2 * L["outputs"] + add)

@@ -169,10 +169,10 @@ layer make_maxpool_layer(int batch, int h, int w, int c, int size, int stride, i
 
 void forward_maxpool_layer_gpu(layer l, network net)
 {
-    /* indexes feed only the backward pass; inference writes them when asked to train-compatible
-     * behaviour is wanted (net.train) or a caller reads them through layer_indexes_host. */
-    forward_maxpool_gpu(net.input_gpu, l.output_gpu, l.indexes_gpu, l.batch, l.c, l.h, l.w, l.size, l.stride,
-                        l.pad);
+    /* the argmax indexes feed only the backward pass: inference leaves them out (a quarter of the
+     * layer's write traffic); layer_indexes_host() computes them on demand */
+    forward_maxpool_gpu(net.input_gpu, l.output_gpu, net.train ? l.indexes_gpu : 0, l.batch, l.c, l.h, l.w, l.size,
+                        l.stride, l.pad);
 }
 
 /* ---- route: src/route_layer.c:7-38 --------------------------------------------------------- */

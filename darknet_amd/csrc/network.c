@@ -224,8 +224,12 @@ int *layer_indexes_host(network *net, int i)
     layer *l;
     if (i < 0 || i >= net->n) dn_fatal("layer_indexes_host: layer index out of range");
     l = &net->layers[i];
-    if (!l->indexes_gpu) dn_fatal("layer_indexes_host: layer has no indexes");
+    if (l->type != MAXPOOL || !l->indexes_gpu) dn_fatal("layer_indexes_host: layer has no indexes");
     if (!l->indexes) l->indexes = (int *)dn_calloc((size_t)l->outputs * l->batch, sizeof(int));
+    /* the forward pass leaves the argmax out (only the backward pass reads it): compute it now from
+     * the layer's input, which is still resident (nothing is recycled between layers) */
+    forward_maxpool_gpu(i ? net->layers[i - 1].output_gpu : net->input_gpu, l->output_gpu, l->indexes_gpu,
+                        l->batch, l->c, l->h, l->w, l->size, l->stride, l->pad);
     hip_pull_int_array(l->indexes_gpu, l->indexes, (size_t)l->outputs * l->batch);
     return l->indexes;
 }
