@@ -168,8 +168,8 @@ def main():
     ap.add_argument("--cpu-kind", default="reference", choices=["reference", "port"])
     args = ap.parse_args()
     if args.gpus != 1:
-        log("bench.py: this build runs on one GPU only (the forward path has no exchange step; "
-            "see DESIGN.md for how it shards by batch). Use --gpus 1.")
+        log("bench.py: this build runs on one GPU only (the forward path has no exchange step: it shards "
+            "by batch, every GPU running the same forward on its share of the images). Use --gpus 1.")
         sys.exit(2)
 
     import numpy as np

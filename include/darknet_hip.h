@@ -96,7 +96,7 @@ void binarize_weights_gpu(float *weights, int n, int size, float *binary); /* co
 /* ------------------------------------------------------------------------------------------
  * Fused layer forwards.  Each replaces the body of the reference's forward_*_layer_gpu for
  * the inference case (net.train == 0); a darknet tree calls them from those functions with the
- * fields of `layer` / `network` spelled out (INTEGRATION.md shows the adapters).
+ * fields of `layer` / `network` spelled out.
  * ---------------------------------------------------------------------------------------- */
 
 /* Convolution + batch-norm/bias + activation in one pass.
