@@ -25,7 +25,7 @@ C_SOURCES = ["hip.c", "cfg_reader.c", "cfg_parser.c", "layers.c", "network.c", "
 HIP_FLAGS = ["--offload-arch=gfx950", "-O3", "-fPIC", "-ffp-contract=off", "-Wno-comment",
              "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
              "-I" + CSRC, "-I" + INCLUDE]
-C_FLAGS = ["-O2", "-fPIC", "-Wall", "-Wno-comment", "-D__HIP_PLATFORM_AMD__=1",
+C_FLAGS = ["-O2", "-fPIC", "-fopenmp", "-Wall", "-Wno-comment", "-D__HIP_PLATFORM_AMD__=1",
            "-I" + CSRC, "-I" + INCLUDE, "-I" + os.path.join(ROCM, "include")]
 
 
@@ -56,7 +56,7 @@ def build(verbose: bool = False, jobs: int = 6) -> str:
             if verbose and out.strip():
                 print(out)
     out = _run([hipcc, "--offload-arch=gfx950", "-shared", "-fPIC", "-Wl,-Bsymbolic", "-o", LIB] + objs +
-               ["-L" + os.path.join(ROCM, "lib"), "-lamdhip64", "-lm"])
+               ["-L" + os.path.join(ROCM, "lib"), "-lamdhip64", "-lm", "-lgomp"])
     if verbose and out.strip():
         print(out)
     return LIB
