@@ -201,3 +201,23 @@ def test_flatten_and_crop_gpu(dn, orc):
         out, keep = D(n=3 * 10 * oh * ow), D(x)
         dn.forward_crop_gpu(keep.ptr, out.ptr, 3, 10, 6, 7, oh, ow, noadjust)
         assert np.array_equal(out.numpy((3, 10, oh, ow)), orc.crop(x, oh, ow, noadjust))
+
+
+@pytest.mark.parametrize("n", [(4 << 20) // 4 - 1, (4 << 20) // 4, (16 << 20) // 4 + 123, (48 << 20) // 4 + 5,
+                               (16 << 20) // 4 * 2])
+def test_large_copies_round_trip_through_the_staging_buffers(dn, n):
+    """Copies of 4 MB and more are cut into 16 MB chunks that alternate between two pinned buffers;
+    sizes sit on and around the chunk and threshold boundaries."""
+    x = synth.uniform(n % 97, n, -1, 1)
+    d = D(x)                       # hip_make_array: plain copy
+    back = np.empty_like(x)
+    dn.hip_pull_array(d.ptr, api._fp(back), n)
+    assert np.array_equal(back, x)
+    y = synth.uniform(7, n, -1, 1)
+    dn.hip_push_array(d.ptr, api._fp(y), n)
+    dn.hip_pull_array(d.ptr, api._fp(back), n)
+    assert np.array_equal(back, y)
+    # a kernel queued before the pull must be seen by it
+    dn.fill_gpu(1000, 3.5, d.ptr, 1)
+    dn.hip_pull_array(d.ptr, api._fp(back), n)
+    assert np.all(back[:1000] == 3.5) and np.array_equal(back[1000:], y[1000:])
