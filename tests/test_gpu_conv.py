@@ -113,6 +113,25 @@ def test_mfma_kernel_agrees_with_direct_kernel_and_unpacked_call(dn):
     assert norm_err(fast, direct) <= 2e-6
 
 
+def test_grouped_mfma_tiles_agree_with_direct_kernel_and_unpacked_call(dn):
+    """Block-diagonal 32-filter tiles (8 channels per group here) against the per-group direct loop."""
+    b, c, h, w, n, groups = 3, 128, 15, 17, 128, 16
+    x = synth.uniform(4, b * c * h * w).reshape(b, c, h, w)
+    wt = synth.conv_weights(5, n, c // groups, 3)
+    bias, sc, mu, var = synth.bn_random(6, n)
+    kw = dict(n=n, size=3, stride=2, pad=1, groups=groups, bn=1, act="leaky")
+    assert dn.conv_kernel_name(n, c, groups, 3).decode() == "conv_mfma_kernel<32,256,32,64,13>"
+    fast = run_conv(dn, x, wt, bias, sc, mu, var, **kw)
+    assert np.array_equal(fast, run_conv(dn, x, wt, bias, sc, mu, var, packed=False, **kw))
+    dn.conv_set_algo(1)
+    try:
+        assert dn.conv_kernel_name(n, c, groups, 3).decode() == "conv_direct_kernel"
+        direct = run_conv(dn, x, wt, bias, sc, mu, var, **kw)
+    finally:
+        dn.conv_set_algo(0)
+    assert norm_err(fast, direct) <= 2e-6
+
+
 def test_conv_golden_vectors(dn):
     g = np.load(os.path.join(GOLD, "conv_cases.npz"))
     for name in sorted(k[:-5] for k in g.files if k.endswith("_spec")):
