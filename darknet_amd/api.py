@@ -249,6 +249,13 @@ class Network:
         total = self.L.forward_network_profiled(self.net, buf)
         return float(total), [float(v) for v in buf]
 
+    def forward_profiled_kernels(self):
+        """forward_profiled plus each convolution's main-kernel duration alone (ms, -1 = none)."""
+        buf = (C.c_float * self.n)()
+        kbuf = (C.c_float * self.n)()
+        total = self.L.forward_network_profiled_kernels(self.net, buf, kbuf)
+        return float(total), [float(v) for v in buf], [float(v) for v in kbuf]
+
     def synchronize(self):
         self.L.hip_synchronize()
 

@@ -37,6 +37,7 @@
  * XCD (ids are dealt round-robin over the 8 XCDs, each with its own L2).
  */
 #include <hip/hip_runtime.h>
+#include <hip/hip_ext.h>
 #include <stdint.h>
 #include <stdio.h>
 #include <stdlib.h>
@@ -689,6 +690,17 @@ extern "C" void conv_pack_weights_gpu(const float *weights, float *packed, int n
 }
 
 /* ---- dispatch ---------------------------------------------------------------------------- */
+/* One-shot kernel timing: the next MFMA convolution launches its main kernel with these two
+ * events attached to the dispatch itself (start and end of the kernel as the GPU stamps them,
+ * no extra packets on the stream), then forgets them. */
+static hipEvent_t g_prof_start = 0, g_prof_stop = 0;
+extern "C" void conv_profile_next(void *start_event, void *stop_event)
+{
+    g_prof_start = (hipEvent_t)start_event;
+    g_prof_stop = (hipEvent_t)stop_event;
+}
+extern "C" int conv_profile_pending(void) { return g_prof_start != 0; }
+
 static int g_algo = 0;
 extern "C" void conv_set_algo(int algo) { g_algo = algo; }
 
@@ -746,6 +758,15 @@ static long plan_split(long tiles, int kch, int cus, int *split)
     return *split > 1 ? whole : tiles;
 }
 
+#define DN_LAUNCH(K)                                                                                        \
+    do {                                                                                                    \
+        if (g_prof_start)                                                                                   \
+            hipExtLaunchKernelGGL(K, grid, dim3(DN_THREADS), 0, dn_stream(), g_prof_start, g_prof_stop, 0, a); \
+        else                                                                                                \
+            hipLaunchKernelGGL(K, grid, dim3(DN_THREADS), 0, dn_stream(), a);                              \
+        g_prof_start = g_prof_stop = 0;                                                                     \
+    } while (0)
+
 template <int BM, int BN, int WM, int WN>
 static void launch_tile(const mfma_args &a0, int mode)
 {
@@ -777,16 +798,16 @@ static void launch_tile(const mfma_args &a0, int mode)
     const dim3 grid((unsigned)(a.per_xcd * 8 + tail * split));
     if (BM > 128 && mode != 11 && mode != 13) dn_fatal("conv dispatch: the 256-row tile is only built for the tap-blocked modes");
     switch (mode) {
-    case 11: hipLaunchKernelGGL((conv_mfma_kernel<BM, BN, WM, WN, 11>), grid, dim3(DN_THREADS), 0, dn_stream(), a); break;
-    case 13: hipLaunchKernelGGL((conv_mfma_kernel<BM, BN, WM, WN, 13>), grid, dim3(DN_THREADS), 0, dn_stream(), a); break;
+    case 11: DN_LAUNCH((conv_mfma_kernel<BM, BN, WM, WN, 11>)); break;
+    case 13: DN_LAUNCH((conv_mfma_kernel<BM, BN, WM, WN, 13>)); break;
     default:
         if constexpr (BM <= 128) {
             if (mode == 1)
-                hipLaunchKernelGGL((conv_mfma_kernel<BM, BN, WM, WN, 1>), grid, dim3(DN_THREADS), 0, dn_stream(), a);
+                DN_LAUNCH((conv_mfma_kernel<BM, BN, WM, WN, 1>));
             else if (mode == 3)
-                hipLaunchKernelGGL((conv_mfma_kernel<BM, BN, WM, WN, 3>), grid, dim3(DN_THREADS), 0, dn_stream(), a);
+                DN_LAUNCH((conv_mfma_kernel<BM, BN, WM, WN, 3>));
             else
-                hipLaunchKernelGGL((conv_mfma_kernel<BM, BN, WM, WN, 0>), grid, dim3(DN_THREADS), 0, dn_stream(), a);
+                DN_LAUNCH((conv_mfma_kernel<BM, BN, WM, WN, 0>));
         }
         break;
     }

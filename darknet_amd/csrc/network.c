@@ -106,32 +106,54 @@ void forward_network_device(network *netp)
 }
 
 /* The same loop with a HIP event between consecutive layers; layer_ms[i] receives layer i's
- * time on the device (a shortcut that ran inside the convolution before it reports 0).  Returns the total (first event to last) in milliseconds.  Events are
- * created once per network size and reused. */
-float forward_network_profiled(network *netp, float *layer_ms)
+ * time on the device (a shortcut that ran inside the convolution before it reports 0), and, when
+ * kernel_ms is not NULL, kernel_ms[i] the duration of a convolution's main kernel alone as stamped
+ * on its dispatch (-1 for layers without one).  Returns the total (first event to last) in
+ * milliseconds.  Events are created once per network size and reused. */
+float forward_network_profiled_kernels(network *netp, float *layer_ms, float *kernel_ms)
 {
-    static void **ev = 0;
+    static void **ev = 0, **ks = 0, **ke = 0;
     static int nev = 0;
     network net = *netp;
     int i;
     float total;
     if (nev < net.n + 1) {
         ev = (void **)realloc(ev, sizeof(void *) * (size_t)(net.n + 1));
-        if (!ev) dn_fatal("Malloc error");
-        for (i = nev; i < net.n + 1; ++i) ev[i] = hip_event_create();
+        ks = (void **)realloc(ks, sizeof(void *) * (size_t)(net.n + 1));
+        ke = (void **)realloc(ke, sizeof(void *) * (size_t)(net.n + 1));
+        if (!ev || !ks || !ke) dn_fatal("Malloc error");
+        for (i = nev; i < net.n + 1; ++i) {
+            ev[i] = hip_event_create();
+            ks[i] = hip_event_create();
+            ke[i] = hip_event_create();
+        }
         nev = net.n + 1;
     }
     net.train = 0;
     hip_event_record(ev[0]);
     for (i = 0; i < net.n; ++i) {
         layer l = net.layers[i];
+        const int first = i;
+        int timed = 0;
         net.index = i;
+        if (kernel_ms && (l.type == CONVOLUTIONAL || l.type == CONNECTED) && !l.xnor) {
+            conv_profile_next(ks[i], ke[i]);
+            timed = 1;
+        }
         if (forward_conv_shortcut_pair(net, i)) {
             hip_event_record(ev[i + 1]);
             ++i;
+            if (kernel_ms) kernel_ms[i] = -1.f;
             l = net.layers[i];
         } else {
             l.forward_gpu(l, net);
+        }
+        if (kernel_ms) {
+            if (timed && conv_profile_pending()) { /* another kernel served the layer */
+                conv_profile_next(0, 0);
+                timed = 0;
+            }
+            kernel_ms[first] = timed ? 0.f : -1.f; /* 0 = to be read after the pass */
         }
         net.input_gpu = l.output_gpu;
         hip_event_record(ev[i + 1]);
@@ -139,7 +161,15 @@ float forward_network_profiled(network *netp, float *layer_ms)
     total = hip_event_elapsed_ms(ev[0], ev[net.n]);
     if (layer_ms)
         for (i = 0; i < net.n; ++i) layer_ms[i] = hip_event_elapsed_ms(ev[i], ev[i + 1]);
+    if (kernel_ms)
+        for (i = 0; i < net.n; ++i)
+            if (kernel_ms[i] == 0.f) kernel_ms[i] = hip_event_elapsed_ms(ks[i], ke[i]);
     return total;
+}
+
+float forward_network_profiled(network *netp, float *layer_ms)
+{
+    return forward_network_profiled_kernels(netp, layer_ms, 0);
 }
 
 /* src/network.c:1123-1127 */

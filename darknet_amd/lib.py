@@ -85,6 +85,8 @@ SIGNATURES = {
     "pull_network_output": (None, [V]), "network_width": (i, [V]), "network_height": (i, [V]),
     "forward_network_device": (None, [V]), "forward_network_profiled": (f, [V, F]),
     "network_set_fusion": (None, [i]),
+    "forward_network_profiled_kernels": (f, [V, F, F]),
+    "conv_profile_next": (None, [V, V]), "conv_profile_pending": (i, []),
     "conv_kernel_name": (C.c_char_p, [i, i, i, i]), "layer_output_host": (F, [V, i]),
     "layer_indexes_host": (I, [V, i]), "network_set_verbose": (None, [i]),
     "network_set_conv": (None, [V, i, F, F, F, F, F]),

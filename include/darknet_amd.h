@@ -290,6 +290,9 @@ void forward_network_device(network *net);
 /* forward_network_device with a HIP event after every layer: fills layer_ms[net->n] (may be
  * NULL) and returns the whole pass in milliseconds; synchronises before returning. */
 float forward_network_profiled(network *net, float *layer_ms);
+/* the same, plus kernel_ms[net->n]: the duration of each convolutional / connected layer's main
+ * kernel alone, from events attached to its dispatch (-1 where there is none) */
+float forward_network_profiled_kernels(network *net, float *layer_ms, float *kernel_ms);
 /* 1 (default): forward_network_device runs a convolution and the same-geometry shortcut right
  * after it as one pass (forward_convolutional_shortcut_gpu); 0: layer by layer as
  * src/network.c:773-785 does.  Every layer's output buffer is written in both modes and holds

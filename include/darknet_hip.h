@@ -146,6 +146,14 @@ void conv_pack_weights_gpu(const float *weights, float *packed, int n, int c, in
  * profiler trace (e.g. "conv_mfma_kernel<128,128,64,64,3>"); for reports only. */
 const char *conv_kernel_name(int n, int c, int groups, int size);
 
+/* Kernel timing for reports: the next forward_convolutional[_shortcut]_gpu call that runs on the
+ * MFMA kernel attaches these two events (hip_event_create) to its main kernel's dispatch, so
+ * hip_event_elapsed_ms(start, stop) is the kernel's own duration as a profiler reports it (the
+ * K-split reduce pass and launch gaps excluded).  conv_profile_pending() != 0 afterwards means the
+ * call took another kernel and the events were not recorded. */
+void conv_profile_next(void *start_event, void *stop_event);
+int conv_profile_pending(void);
+
 /* Selects the convolution kernel: 0 = automatic (default), 1 = always the plain direct
  * kernel, 3 = MFMA kernel without the K-split of the last partial round of tiles.  The direct
  * kernel is the in-library cross-check of the MFMA kernel. */

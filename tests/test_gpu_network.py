@@ -195,6 +195,28 @@ def test_shortcut_fusion_changes_no_bit(dn):
     net.free()
 
 
+def test_kernel_stamped_timing(dn):
+    """forward_network_profiled_kernels: every MFMA convolution's main kernel carries its own
+    start/stop events; the stamped duration is positive, no longer than the interval between the
+    events around its layer (plus timer slack), other layers report -1, and no output bit changes."""
+    net = api.Network(cfg_text=cfgs.yolov3(2, 160))
+    fill_params(net.set_conv, net.layers)
+    x = synth.uniform01(22, net.inputs * 2)
+    net.predict(x)
+    want = [net.layer_output(i) for i in range(net.n)]
+    for _ in range(2):
+        total, layer_ms, kernel_ms = net.forward_profiled_kernels()
+    assert dn.conv_profile_pending() == 0
+    for i, L in enumerate(net.layers):
+        assert np.array_equal(net.layer_output(i), want[i]), i
+        if L["type"] == "convolutional":
+            assert 0 < kernel_ms[i] <= layer_ms[i] + 0.05, (i, kernel_ms[i], layer_ms[i])
+        else:
+            assert kernel_ms[i] == -1.0, (i, L["type"], kernel_ms[i])
+    assert sum(k for k in kernel_ms if k > 0) < total
+    net.free()
+
+
 def test_small_net2_crop_reorg_dropout_connected_cost(dn, tmp_path):
     """The layer types beyond the yolo family (crop, the four reorg modes, dropout, connected with
     and without batch-norm, cost): layer table, reference-written weights file, per-layer outputs
