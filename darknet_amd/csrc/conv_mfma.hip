@@ -46,6 +46,8 @@
 #include "hip.h"
 
 typedef float f32x16 __attribute__((ext_vector_type(16)));
+typedef float f32x8 __attribute__((ext_vector_type(8)));
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 
 #define DN_BK 16
 #define DN_MPAD 128
@@ -265,7 +267,7 @@ __device__ __forceinline__ void conv_epilogue(const mfma_args &a, f32x16 (&acc)[
     }
 }
 
-template <int BM, int BN, int WM, int WN, int MODE>
+template <int BM, int BN, int WM, int WN, int MODE, bool BF16 = false>
 __global__ __launch_bounds__(DN_THREADS, (BM == 128 ? 3 : 2)) void conv_mfma_kernel(mfma_args a)
 {
     constexpr int TM = WM / 32, TN = WN / 32;
@@ -481,6 +483,37 @@ __global__ __launch_bounds__(DN_THREADS, (BM == 128 ? 3 : 2)) void conv_mfma_ker
         }
     };
 
+    /* Reduced-precision variant: the same fp32 tiles in LDS, each lane's eight k values of a row
+     * (two slots) rounded to bf16 (round to nearest even) on the way into one
+     * v_mfma_f32_32x32x16_bf16, which contracts all 16 k of the chunk at once; products and
+     * sums stay fp32, so does everything after the accumulators.  Which k sits in which lane half
+     * and position does not matter as long as A and B agree, and they share the slot layout. */
+    auto mfma_chunk = [&]() {
+        if constexpr (BF16) {
+            bf16x8 a8[TM], b8[TN];
+#pragma unroll
+            for (int i = 0; i < TM; ++i) {
+                const f32x8 f = {av[0][i].x, av[0][i].y, av[0][i].z, av[0][i].w,
+                                 av[1][i].x, av[1][i].y, av[1][i].z, av[1][i].w};
+                a8[i] = __builtin_convertvector(f, bf16x8);
+            }
+#pragma unroll
+            for (int j = 0; j < TN; ++j) {
+                const f32x8 f = {bv[0][j].x, bv[0][j].y, bv[0][j].z, bv[0][j].w,
+                                 bv[1][j].x, bv[1][j].y, bv[1][j].z, bv[1][j].w};
+                b8[j] = __builtin_convertvector(f, bf16x8);
+            }
+#pragma unroll
+            for (int i = 0; i < TM; ++i)
+#pragma unroll
+                for (int j = 0; j < TN; ++j)
+                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(b8[j], a8[i], acc[i][j], 0, 0, 0);
+        } else {
+            mfma_half(0);
+            mfma_half(1);
+        }
+    };
+
     /* One pipeline step, in program order (pinned by scheduling barriers):
      *   1. direct-to-LDS loads of chunk kc+1 into the other buffer (nobody reads it: every wave
      *      passed the previous barrier only after its MFMAs had consumed that buffer)
@@ -491,16 +524,14 @@ __global__ __launch_bounds__(DN_THREADS, (BM == 128 ? 3 : 2)) void conv_mfma_ker
         __builtin_amdgcn_sched_barrier(0);
         read_operands(buf);
         __builtin_amdgcn_sched_barrier(0);
-        mfma_half(0);
-        mfma_half(1);
+        mfma_chunk();
         __builtin_amdgcn_sched_barrier(0);
         __builtin_amdgcn_s_waitcnt(0);
         __syncthreads();
     };
     auto last = [&](int buf) {
         read_operands(buf);
-        mfma_half(0);
-        mfma_half(1);
+        mfma_chunk();
     };
 
     int kc = kc_begin;
@@ -704,23 +735,30 @@ extern "C" int conv_profile_pending(void) { return g_prof_start != 0; }
 static int g_algo = 0;
 extern "C" void conv_set_algo(int algo) { g_algo = algo; }
 
+/* 0 = fp32 operands (default, the reference's arithmetic); 1 = the tap-blocked MFMA kernels round
+ * both operands to bf16 and accumulate in fp32 (layers on other kernels stay fp32). */
+static int g_precision = 0;
+extern "C" void conv_set_precision(int precision)
+{
+    if (precision != 0 && precision != 1) dn_fatal("conv_set_precision: 0 (fp32) or 1 (bf16 operands)");
+    g_precision = precision;
+}
+extern "C" int conv_get_precision(void) { return g_precision; }
+
 static int conv_mode(int c, int groups, int size, int stride, int pad, long in_bytes);
 
 extern "C" const char *conv_kernel_name(int n, int c, int groups, int size)
 {
     static char name[96];
-    const int mode = conv_mode(c, groups, size, 1, size / 2, 0);
+    int mode = conv_mode(c, groups, size, 1, size / 2, 0);
+    int bm = n <= 32 ? 32 : n <= 64 ? 64 : 128;
     if (conv_grouped_tile(n, c, groups, size) && g_algo != 1) {
-        snprintf(name, sizeof name, "conv_mfma_kernel<32,256,32,64,%d>", size == 3 ? 13 : 11);
-        return name;
+        mode = size == 3 ? 13 : 11;
+        bm = 32;
     }
     if (mode < 0) return "conv_direct_kernel";
-    if (n <= 32)
-        snprintf(name, sizeof name, "conv_mfma_kernel<32,256,32,64,%d>", mode);
-    else if (n <= 64)
-        snprintf(name, sizeof name, "conv_mfma_kernel<64,256,64,64,%d>", mode);
-    else
-        snprintf(name, sizeof name, "conv_mfma_kernel<128,128,64,64,%d>", mode);
+    snprintf(name, sizeof name, "conv_mfma_kernel<%d,%d,%d,64,%d%s>", bm, bm == 128 ? 128 : 256, bm == 32 ? 32 : 64,
+             mode, (g_precision == 1 && mode >= 10) ? ",true" : "");
     return name;
 }
 
@@ -798,8 +836,18 @@ static void launch_tile(const mfma_args &a0, int mode)
     const dim3 grid((unsigned)(a.per_xcd * 8 + tail * split));
     if (BM > 128 && mode != 11 && mode != 13) dn_fatal("conv dispatch: the 256-row tile is only built for the tap-blocked modes");
     switch (mode) {
-    case 11: DN_LAUNCH((conv_mfma_kernel<BM, BN, WM, WN, 11>)); break;
-    case 13: DN_LAUNCH((conv_mfma_kernel<BM, BN, WM, WN, 13>)); break;
+    case 11:
+        if (g_precision == 1)
+            DN_LAUNCH((conv_mfma_kernel<BM, BN, WM, WN, 11, true>));
+        else
+            DN_LAUNCH((conv_mfma_kernel<BM, BN, WM, WN, 11>));
+        break;
+    case 13:
+        if (g_precision == 1)
+            DN_LAUNCH((conv_mfma_kernel<BM, BN, WM, WN, 13, true>));
+        else
+            DN_LAUNCH((conv_mfma_kernel<BM, BN, WM, WN, 13>));
+        break;
     default:
         if constexpr (BM <= 128) {
             if (mode == 1)

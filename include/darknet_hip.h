@@ -159,6 +159,14 @@ int conv_profile_pending(void);
  * kernel is the in-library cross-check of the MFMA kernel. */
 void conv_set_algo(int algo);
 
+/* Operand precision of the tap-blocked MFMA convolution kernels (channels a multiple of 16, 1x1 or
+ * 3x3 pad 1; grouped 32-filter tiles): 0 = fp32 (default; the reference's arithmetic, the parity
+ * bar applies), 1 = both operands rounded to bf16 (nearest even) inside the kernel, products and
+ * sums in fp32, epilogue unchanged.  Layers served by other kernels (first layer, direct, xnor)
+ * stay fp32.  An opt-in speed/precision trade with no counterpart in the reference. */
+void conv_set_precision(int precision);
+int conv_get_precision(void);
+
 /* XNOR convolution (xnor=1 layers): sign(x>0) inputs, sign(w>0)*mean|w| weights, zero padding,
  * computed as XOR + popcount on bit-packed operands, then the same batch-norm/bias/activation
  * tail.  Replaces the xnor branch of forward_convolutional_layer_gpu

@@ -1,0 +1,123 @@
+"""The opt-in bf16-operand mode of the tap-blocked MFMA convolution kernels.
+
+What the mode computes is pinned exactly: the CPU checker run on operands rounded to bf16 (round
+to nearest even, done here in integer arithmetic) must agree with the kernel to the fp32 bar
+(<= 1e-4 max-normalised; the products of two bf16 numbers are exact in fp32, so only the
+summation order differs).  Against the unrounded fp32 checker the mode's error is measured and
+bounded loosely (it is a precision trade, not a parity claim), and the default fp32 mode must be
+untouched by a round trip through the switch."""
+import numpy as np
+import pytest
+
+from darknet_amd import api, cfgs, synth
+from oracle.net import OracleNet
+
+from test_gpu_conv import run_conv
+from util import REL_TOL, fill_params, norm_err
+
+pytestmark = pytest.mark.gpu
+
+
+def round_bf16(x):
+    """fp32 -> nearest bf16 (ties to even) -> fp32, on the bit patterns."""
+    u = np.ascontiguousarray(x, dtype=np.float32).view(np.uint32).astype(np.uint64)
+    u = (u + 0x7FFF + ((u >> 16) & 1)) & 0xFFFF0000
+    return u.astype(np.uint32).view(np.float32).reshape(np.shape(x))
+
+
+def test_round_bf16_helper():
+    x = np.array([1.0, 1.0 + 2.0 ** -8, 1.0 + 3 * 2.0 ** -8, 1.0 + 2.0 ** -8 + 2.0 ** -20, -0.1, 0.0], np.float32)
+    r = round_bf16(x)
+    # ties go to the even mantissa: 1+2^-8 -> 1, 1+3*2^-8 -> 1+2^-6; above a tie rounds up
+    assert r[0] == 1.0 and r[1] == 1.0 and r[2] == np.float32(1.0 + 2.0 ** -6) and r[3] == np.float32(1 + 2.0 ** -7)
+    assert abs(r[4] + 0.1) < 0.1 * 2.0 ** -8 and r[5] == 0.0
+    assert np.all((r.view(np.uint32) & 0xFFFF) == 0)
+
+
+@pytest.fixture
+def bf16(dn):
+    dn.conv_set_precision(1)
+    yield dn
+    dn.conv_set_precision(0)
+
+
+BF16_SHAPES = [  # b, c, h, w, n, size, stride, pad, groups, act
+    (2, 256, 26, 26, 512, 3, 1, 1, 1, "leaky"),
+    (2, 512, 52, 52, 256, 1, 1, 0, 1, "leaky"),
+    (2, 128, 104, 104, 256, 3, 2, 1, 1, "leaky"),
+    (2, 32, 30, 30, 64, 3, 2, 1, 1, "leaky"),       # 64-row tile
+    (1, 64, 19, 19, 32, 1, 1, 0, 1, "linear"),      # 32-row tile
+    (2, 1024, 13, 13, 255, 1, 1, 0, 1, "linear"),   # ragged M, K-split at this size
+    (2, 128, 14, 14, 128, 3, 1, 1, 32, "leaky"),    # grouped 32-filter tiles
+]
+
+
+@pytest.mark.parametrize("b,c,h,w,n,size,stride,pad,groups,act", BF16_SHAPES)
+def test_bf16_mode_is_fp32_conv_of_rounded_operands(bf16, orc, b, c, h, w, n, size, stride, pad, groups, act):
+    x = synth.uniform(11, b * c * h * w).reshape(b, c, h, w)
+    wt = synth.conv_weights(12, n, c // groups, size)
+    bias, sc, mu, var = synth.bn_random(13, n)
+    kw = dict(n=n, size=size, stride=stride, pad=pad, groups=groups)
+    assert ",true>" in bf16.conv_kernel_name(n, c, groups, size).decode()
+    got = run_conv(bf16, x, wt, bias, sc, mu, var, bn=1, act=act, **kw)
+    want = orc.conv(round_bf16(x), round_bf16(wt), bias, sc, mu, var, batch_normalize=1, activation=act, **kw)
+    assert norm_err(got, want) <= REL_TOL
+    full = orc.conv(x, wt, bias, sc, mu, var, batch_normalize=1, activation=act, **kw)
+    err = norm_err(got, full)
+    print(f"bf16-operand error vs fp32, {size}x{size}/{stride} {c}->{n} g{groups}: {err:.2e}")
+    assert 1e-5 < err < 2e-2          # really reduced precision, and no worse than bf16 rounding explains
+
+
+def test_layers_on_other_kernels_stay_fp32(bf16, orc):
+    """3 input channels -> reference-order kernel: the switch must not touch it."""
+    b, c, h, w, n = 2, 3, 33, 35, 32
+    x = synth.uniform(14, b * c * h * w).reshape(b, c, h, w)
+    wt = synth.conv_weights(15, n, c, 3)
+    bias, sc, mu, var = synth.bn_random(16, n)
+    assert ",true>" not in bf16.conv_kernel_name(n, c, 1, 3).decode()
+    got1 = run_conv(bf16, x, wt, bias, sc, mu, var, n=n, size=3, stride=1, pad=1, groups=1, bn=1, act="leaky")
+    bf16.conv_set_precision(0)
+    got0 = run_conv(bf16, x, wt, bias, sc, mu, var, n=n, size=3, stride=1, pad=1, groups=1, bn=1, act="leaky")
+    assert np.array_equal(got0, got1)
+
+
+def test_switch_round_trip_restores_fp32_bits(dn):
+    b, c, h, w, n = 2, 64, 20, 20, 128
+    x = synth.uniform(17, b * c * h * w).reshape(b, c, h, w)
+    wt = synth.conv_weights(18, n, c, 3)
+    bias, sc, mu, var = synth.bn_random(19, n)
+    kw = dict(n=n, size=3, stride=1, pad=1, groups=1, bn=1, act="leaky")
+    before = run_conv(dn, x, wt, bias, sc, mu, var, **kw)
+    dn.conv_set_precision(1)
+    try:
+        mid = run_conv(dn, x, wt, bias, sc, mu, var, **kw)
+    finally:
+        dn.conv_set_precision(0)
+    after = run_conv(dn, x, wt, bias, sc, mu, var, **kw)
+    assert dn.conv_get_precision() == 0
+    assert np.array_equal(before, after) and not np.array_equal(before, mid)
+
+
+def test_yolov3_bf16_measured_error(bf16):
+    """Whole network, bf16 operands in 74 of 75 convolutions: the error against the fp32 checker is
+    measured per layer and at the yolo heads; the bounds are loose sanity limits, not parity."""
+    text = cfgs.yolov3(1, 160)
+    net = api.Network(cfg_text=text)
+    ref = OracleNet(text)
+    fill_params(net.set_conv, net.layers, bn="random")
+    fill_params(ref.set_conv, ref.layers, bn="random")
+    x = synth.uniform01(23, net.inputs)
+    net.predict(x)
+    outs = ref.forward(x)
+    worst_conv = 0.0
+    yolo_abs = 0.0
+    for i, L in enumerate(net.layers):
+        got, want = net.layer_output(i), outs[i]
+        if L["type"] == "convolutional":
+            worst_conv = max(worst_conv, norm_err(got, want))
+        elif L["type"] == "yolo":
+            yolo_abs = max(yolo_abs, float(np.max(np.abs(got - want))))
+    print(f"yolov3-160 bf16 operands: worst conv layer {worst_conv:.2e} max-normalised, yolo heads {yolo_abs:.2e} abs")
+    assert 1e-4 < worst_conv < 5e-2
+    assert yolo_abs < 0.5
+    net.free()
