@@ -62,6 +62,9 @@ extern "C" void conv_direct_forward(const float *, const float *, const float *,
 struct mfma_args {
     const float *in;
     const float *wp; /* packed weights */
+    const void *wp16; /* the bf16 copy of the packed weights (bf16-operand mode) */
+    unsigned wp16_records;
+    int Mpad16;
     const float *biases, *scales, *mean, *var;
     float *out;
     int C, H, W, M, K, KCH, Mpad;
@@ -280,8 +283,14 @@ __global__ __launch_bounds__(DN_THREADS, (BM == 128 ? 3 : 2)) void conv_mfma_ker
     /* Four separate LDS objects rather than two [2][...] arrays: the compiler makes every LDS read
      * wait (vmcnt) for direct-to-LDS loads it cannot prove disjoint from it, and it can only
      * prove that for distinct objects. */
-    __shared__ __attribute__((aligned(16))) float As0[BM * DN_BK], As1[BM * DN_BK];
+    constexpr int A_FLOATS = BF16 ? BM * DN_BK / 2 : BM * DN_BK; /* bf16 rows are 32 bytes */
+    __shared__ __attribute__((aligned(16))) float As0[A_FLOATS], As1[A_FLOATS];
     __shared__ __attribute__((aligned(16))) float Bs0[BN * DN_BK], Bs1[BN * DN_BK];
+    /* the bf16 variant keeps three chunks in flight: four stages */
+    __shared__ __attribute__((aligned(16))) float As2[BF16 ? A_FLOATS : 4], As3[BF16 ? A_FLOATS : 4];
+    __shared__ __attribute__((aligned(16))) float Bs2[BF16 ? BN * DN_BK : 4], Bs3[BF16 ? BN * DN_BK : 4];
+#define A_BUF(b) ((b) == 0 ? As0 : (b) == 1 ? As1 : (b) == 2 ? As2 : As3)
+#define B_BUF(b) ((b) == 0 ? Bs0 : (b) == 1 ? Bs1 : (b) == 2 ? Bs2 : Bs3)
 
     /* XCD-aware tile order: workgroup id -> (xcd, slot) -> linear tile with tile_m fastest. */
     const int bid = blockIdx.x;
@@ -325,7 +334,7 @@ __global__ __launch_bounds__(DN_THREADS, (BM == 128 ? 3 : 2)) void conv_mfma_ker
     const int HW = a.H * a.W;
 
     const __amdgpu_buffer_rsrc_t w_rsrc = __builtin_amdgcn_make_buffer_rsrc(
-        (void *)a.wp, 0, (int)a.wp_records, 0x00020000);
+        (void *)(BF16 ? a.wp16 : (const void *)a.wp), 0, (int)(BF16 ? a.wp16_records : a.wp_records), 0x00020000);
     const int bias = (TAPB && KS == 3) ? a.W + 1 : 0;
     const __amdgpu_buffer_rsrc_t in_rsrc = __builtin_amdgcn_make_buffer_rsrc(
         (void *)(a.in - bias), 0, (int)a.in_records, 0x00020000);
@@ -371,6 +380,31 @@ __global__ __launch_bounds__(DN_THREADS, (BM == 128 ? 3 : 2)) void conv_mfma_ker
 
     auto load_chunk = [&](int kc, int buf) {
         /* A */
+        if constexpr (BF16) {
+            /* bf16 copy: [chunk][k half][Mpad16 rows][8 bf16]; LDS image [k half][BM][16 bytes].
+             * A wave-load moves 64 consecutive 16-byte rows of one k half (both halves of the 32
+             * rows when BM == 32). */
+            constexpr int WL = BM / 32;                  /* wave-loads per chunk: 8, 4, 2, 1 */
+            constexpr int PER_WAVE = (WL + 3) / 4;
+#pragma unroll
+            for (int i = 0; i < PER_WAVE; ++i) {
+                const int wl = wave * PER_WAVE + i;
+                if (WL >= 4 || wl < WL) {
+                    if (BM >= 64) {
+                        constexpr int RB = BM / 64;
+                        const int h = wl / RB, rb = wl - h * RB;
+                        const unsigned soff = (unsigned)((((long)kc * 2 + h) * a.Mpad16 + m0 + rb * 64) * 16);
+                        __builtin_amdgcn_raw_ptr_buffer_load_lds(w_rsrc, (lds_ptr)&A_BUF(buf)[(h * BM + rb * 64) * 4], 16,
+                                                                 lane * 16, soff, 0, 0);
+                    } else {
+                        const unsigned voff = (unsigned)((((long)(lane >> 5) * a.Mpad16) + (lane & 31)) * 16);
+                        const unsigned soff = a.grouped ? (unsigned)(((long)(tile_m * a.KCH + kc) * 2 * 32) * 16)
+                                                        : (unsigned)(((long)kc * 2 * a.Mpad16 + m0) * 16);
+                        __builtin_amdgcn_raw_ptr_buffer_load_lds(w_rsrc, (lds_ptr)&A_BUF(buf)[0], 16, voff, soff, 0, 0);
+                    }
+                }
+            }
+        } else {
 #pragma unroll
         for (int i = 0; i < A_PER_WAVE; ++i) {
             const int wl = wave * A_PER_WAVE + i;        /* wave-load index: slot q, 64-row block rb */
@@ -380,7 +414,7 @@ __global__ __launch_bounds__(DN_THREADS, (BM == 128 ? 3 : 2)) void conv_mfma_ker
                 const int rb = BM >= 64 ? wl - q * RB : 0;
                 if (BM >= 64) {
                     const unsigned soff = (unsigned)((((long)kc * 4 + q) * a.Mpad + m0 + rb * 64) * 16);
-                    __builtin_amdgcn_raw_ptr_buffer_load_lds(w_rsrc, (lds_ptr)&(buf ? As1 : As0)[(q * BM + rb * 64) * 4], 16,
+                    __builtin_amdgcn_raw_ptr_buffer_load_lds(w_rsrc, (lds_ptr)&A_BUF(buf)[(q * BM + rb * 64) * 4], 16,
                                                              lane * 16, soff, 0, 0);
                 } else {
                     /* BM == 32: one wave-load covers two slots of 32 rows each */
@@ -389,10 +423,11 @@ __global__ __launch_bounds__(DN_THREADS, (BM == 128 ? 3 : 2)) void conv_mfma_ker
                     /* grouped: Mpad == 32 and the tile's chunks follow each other */
                     const unsigned soff = a.grouped ? (unsigned)(((long)(tile_m * a.KCH + kc) * 4 * 32) * 16)
                                                     : (unsigned)(((long)kc * 4 * a.Mpad + m0) * 16);
-                    __builtin_amdgcn_raw_ptr_buffer_load_lds(w_rsrc, (lds_ptr)&(buf ? As1 : As0)[(wl * 2 * BM) * 4], 16, voff,
+                    __builtin_amdgcn_raw_ptr_buffer_load_lds(w_rsrc, (lds_ptr)&A_BUF(buf)[(wl * 2 * BM) * 4], 16, voff,
                                                              soff, 0, 0);
                 }
             }
+        }
         }
         /* B */
         if (TAPB) {
@@ -405,7 +440,7 @@ __global__ __launch_bounds__(DN_THREADS, (BM == 128 ? 3 : 2)) void conv_mfma_ker
                 const int ng = wave * NG_PER_WAVE + g;
 #pragma unroll
                 for (int q = 0; q < 4; ++q)
-                    __builtin_amdgcn_raw_ptr_buffer_load_lds(in_rsrc, (lds_ptr)&(buf ? Bs1 : Bs0)[(q * BN + ng * 16) * 4], 4,
+                    __builtin_amdgcn_raw_ptr_buffer_load_lds(in_rsrc, (lds_ptr)&B_BUF(buf)[(q * BN + ng * 16) * 4], 4,
                                                              voff, soff0 + (unsigned)(q * 4 * HW * 4), 0, 0);
             }
             if (++ld_tap == TAPS) {
@@ -432,7 +467,7 @@ __global__ __launch_bounds__(DN_THREADS, (BM == 128 ? 3 : 2)) void conv_mfma_ker
                     const int ky = kyx[q] >> 16, kx = kyx[q] & 0xffff;
                     const bool ok = ((unsigned)(iy0[g] + ky) < (unsigned)a.H) & ((unsigned)(ix0[g] + kx) < (unsigned)a.W);
                     const unsigned voff = ok ? voff_px[g] + (unsigned)koff[q] : 0xFFFFFFFCu;
-                    __builtin_amdgcn_raw_ptr_buffer_load_lds(in_rsrc, (lds_ptr)&(buf ? Bs1 : Bs0)[(q * BN + ng * 16) * 4], 4,
+                    __builtin_amdgcn_raw_ptr_buffer_load_lds(in_rsrc, (lds_ptr)&B_BUF(buf)[(q * BN + ng * 16) * 4], 4,
                                                              voff, 0, 0, 0);
                 }
             }
@@ -450,21 +485,51 @@ __global__ __launch_bounds__(DN_THREADS, (BM == 128 ? 3 : 2)) void conv_mfma_ker
     const int li = lane & 31; /* row of A / column of B inside a 32x32 block */
     const int kh = lane >> 5; /* which half of the k pair this lane feeds */
 
-    load_chunk(kc_begin, 0);
-    __builtin_amdgcn_s_waitcnt(0);
-    __syncthreads();
+    /* loads one wave issues per chunk, for the s_waitcnt immediates of the bf16 pipeline (the A
+     * loads are left out where not every wave issues them: those waves wait for one load more
+     * than they must) */
+    constexpr int LPC = (BF16 && BM >= 128 ? BM / 128 : 0) + 4 * NG_PER_WAVE;
+    /* s_waitcnt on vmcnt alone: simm16 = vmcnt[3:0] | expcnt(7) << 4 | lgkmcnt(15) << 8 | vmcnt[5:4] << 14 */
+#define DN_WAIT_VM(n) __builtin_amdgcn_s_waitcnt(((n) & 15) | (7 << 4) | (15 << 8) | (((n) >> 4) << 14))
+    static_assert(2 * LPC < 64, "vmcnt is a 6-bit counter");
+
+    if constexpr (BF16) {
+        const int nch = kc_end - kc_begin;
+        load_chunk(kc_begin, 0);
+        if (nch > 1) load_chunk(kc_begin + 1, 1);
+        if (nch > 2) load_chunk(kc_begin + 2, 2);
+        if (nch > 2)
+            DN_WAIT_VM(2 * LPC);
+        else if (nch > 1)
+            DN_WAIT_VM(LPC);
+        else
+            __builtin_amdgcn_s_waitcnt(0);
+        __builtin_amdgcn_s_barrier();
+    } else {
+        load_chunk(kc_begin, 0);
+        __builtin_amdgcn_s_waitcnt(0);
+        __syncthreads();
+    }
 
     float4 av[2][TM], bv[2][TN]; /* MFMA operands of the current chunk: [k half][32-row block] */
+    bf16x8 a8[BF16 ? TM : 1];                /* bf16 mode: a row's eight k of this lane's half */
 
     auto read_operands = [&](int buf) {
 #pragma unroll
         for (int hb = 0; hb < 2; ++hb) {
+            if constexpr (!BF16) {
 #pragma unroll
-            for (int i = 0; i < TM; ++i)
-                av[hb][i] = *(const float4 *)&(buf ? As1 : As0)[((hb * 2 + kh) * BM + wm0 + i * 32 + li) * 4];
+                for (int i = 0; i < TM; ++i)
+                    av[hb][i] = *(const float4 *)&A_BUF(buf)[((hb * 2 + kh) * BM + wm0 + i * 32 + li) * 4];
+            }
 #pragma unroll
             for (int j = 0; j < TN; ++j)
-                bv[hb][j] = *(const float4 *)&(buf ? Bs1 : Bs0)[((hb * 2 + kh) * BN + wn0 + j * 32 + li) * 4];
+                bv[hb][j] = *(const float4 *)&B_BUF(buf)[((hb * 2 + kh) * BN + wn0 + j * 32 + li) * 4];
+        }
+        if constexpr (BF16) {
+#pragma unroll
+            for (int i = 0; i < TM; ++i)
+                a8[i] = *(const bf16x8 *)&A_BUF(buf)[(kh * BM + wm0 + i * 32 + li) * 4];
         }
     };
 
@@ -483,20 +548,14 @@ __global__ __launch_bounds__(DN_THREADS, (BM == 128 ? 3 : 2)) void conv_mfma_ker
         }
     };
 
-    /* Reduced-precision variant: the same fp32 tiles in LDS, each lane's eight k values of a row
-     * (two slots) rounded to bf16 (round to nearest even) on the way into one
-     * v_mfma_f32_32x32x16_bf16, which contracts all 16 k of the chunk at once; products and
-     * sums stay fp32, so does everything after the accumulators.  Which k sits in which lane half
-     * and position does not matter as long as A and B agree, and they share the slot layout. */
+    /* Reduced-precision variant: the weights come from their bf16 copy, whose rows hold the eight k
+     * of a lane half in the order the activation slots give them (slot kh, then slot 2 + kh);
+     * the activations stay fp32 tiles in LDS and are rounded to bf16 (nearest even) on the way
+     * into one v_mfma_f32_32x32x16_bf16, which contracts all 16 k of the chunk at once.
+     * Products and sums stay fp32, so does everything after the accumulators. */
     auto mfma_chunk = [&]() {
         if constexpr (BF16) {
-            bf16x8 a8[TM], b8[TN];
-#pragma unroll
-            for (int i = 0; i < TM; ++i) {
-                const f32x8 f = {av[0][i].x, av[0][i].y, av[0][i].z, av[0][i].w,
-                                 av[1][i].x, av[1][i].y, av[1][i].z, av[1][i].w};
-                a8[i] = __builtin_convertvector(f, bf16x8);
-            }
+            bf16x8 b8[TN];
 #pragma unroll
             for (int j = 0; j < TN; ++j) {
                 const f32x8 f = {bv[0][j].x, bv[0][j].y, bv[0][j].z, bv[0][j].w,
@@ -534,6 +593,38 @@ __global__ __launch_bounds__(DN_THREADS, (BM == 128 ? 3 : 2)) void conv_mfma_ker
         mfma_chunk();
     };
 
+    if constexpr (BF16) {
+        /* Four LDS stages, prefetch distance three: a bf16 chunk is 8 (or 4, 2) MFMAs, far shorter
+         * than a round trip to memory, so chunks kc+1 and kc+2 are already in flight when chunk
+         * kc+3 is requested, and a step waits only until kc+1 has landed (vmcnt counts loads, which
+         * complete in order).  __syncthreads() would drain every load (its fences wait for
+         * vmcnt(0) because direct-to-LDS loads count as LDS writes), so the barrier is the bare
+         * instruction: the explicit vmcnt wait before it covers the loads, and every LDS read of
+         * a stage has been consumed by MFMAs before the wave reaches the barrier after which the
+         * stage is overwritten. */
+        auto bstep = [&](int kcur, int buf) {
+            const int rem = kc_end - 1 - kcur; /* chunks after this one (wave-uniform) */
+            if (rem >= 3) load_chunk(kcur + 3, (buf + 3) & 3);
+            __builtin_amdgcn_sched_barrier(0);
+            read_operands(buf);
+            __builtin_amdgcn_sched_barrier(0);
+            mfma_chunk();
+            __builtin_amdgcn_sched_barrier(0);
+            if (rem >= 3)
+                DN_WAIT_VM(2 * LPC);
+            else if (rem == 2)
+                DN_WAIT_VM(LPC);
+            else
+                __builtin_amdgcn_s_waitcnt(0);
+            if (rem >= 1) __builtin_amdgcn_s_barrier();
+        };
+        for (int kc = kc_begin; kc < kc_end; kc += 4) {
+            bstep(kc, 0);
+            if (kc + 1 < kc_end) bstep(kc + 1, 1);
+            if (kc + 2 < kc_end) bstep(kc + 2, 2);
+            if (kc + 3 < kc_end) bstep(kc + 3, 3);
+        }
+    } else {
     int kc = kc_begin;
     /* two chunks per trip so the LDS buffer index is a compile-time constant in each half */
     for (; kc + 2 < kc_end; kc += 2) {
@@ -545,6 +636,8 @@ __global__ __launch_bounds__(DN_THREADS, (BM == 128 ? 3 : 2)) void conv_mfma_ker
         last(1);
     } else {
         last(0);
+    }
+
     }
 
     if (slice_id >= 0) {
@@ -559,7 +652,8 @@ __global__ __launch_bounds__(DN_THREADS, (BM == 128 ? 3 : 2)) void conv_mfma_ker
                     ws[((wave * TM * TN + i * TN + j) * 16 + r) * 64 + lane] = acc[i][j][r];
     } else {
         __syncthreads(); /* every wave has read its last operands: the LDS buffers are free */
-        float *E = BM == 128 ? (wave == 0 ? As0 : wave == 1 ? As1 : wave == 2 ? Bs0 : Bs1)
+        float *E = BM >= 128 ? (BF16 ? (wave == 0 ? Bs2 : wave == 1 ? Bs3 : wave == 2 ? Bs0 : Bs1)
+                                     : (wave == 0 ? As0 : wave == 1 ? As1 : wave == 2 ? Bs0 : Bs1))
                              : (wave < 2 ? Bs0 : Bs1) + (wave & 1) * 2048;
         conv_epilogue<TM, TN>(a, acc, E, m0, n0, wm0, wn0, lane);
     }
@@ -687,7 +781,8 @@ static inline int tap_blocked_taps(int c, int groups, int size)
     return 0;
 }
 
-extern "C" size_t conv_packed_floats(int n, int c, int groups, int size)
+/* fp32 part of the packed buffer */
+static size_t conv_packed_f32_floats(int n, int c, int groups, int size)
 {
     const int gt = conv_grouped_tile(n, c, groups, size);
     if (gt) return (size_t)(n / 32) * (size_t)(2 * gt) * DN_BK * 32;
@@ -698,25 +793,99 @@ extern "C" size_t conv_packed_floats(int n, int c, int groups, int size)
     return (size_t)(kch * mpad * DN_BK);
 }
 
+/* Rows of the bf16 copy: whole 256-row tiles for layers that use them, else as the fp32 part. */
+static int conv_mpad16(int n)
+{
+    const int unit = n > 128 ? 256 : DN_MPAD;
+    return (n + unit - 1) / unit * unit;
+}
+
+/* bf16 part (tap-blocked and grouped layers only), counted in floats: it follows the fp32 part in
+ * the same buffer so that one pointer still stands for a layer's packed weights */
+static size_t conv_packed_bf16_floats(int n, int c, int groups, int size)
+{
+    const int gt = conv_grouped_tile(n, c, groups, size);
+    if (gt) return conv_packed_f32_floats(n, c, groups, size) / 2;
+    const int taps = tap_blocked_taps(c, groups, size);
+    if (!taps) return 0;
+    const long kch = (long)c * taps / DN_BK;
+    return (size_t)(kch * conv_mpad16(n) * DN_BK / 2);
+}
+
+extern "C" size_t conv_packed_floats(int n, int c, int groups, int size)
+{
+    return conv_packed_f32_floats(n, c, groups, size) + conv_packed_bf16_floats(n, c, groups, size);
+}
+
+/* bf16 copy of a tap-blocked layer: element ((chunk*2 + h)*Mpad16 + m)*8 + p is the weight that the
+ * fp32 layout keeps at slot (p < 4 ? h : 2 + h), position p % 4 of the same chunk and row, rounded
+ * to nearest even. */
+__global__ void pack_weights_bf16_kernel(const float *w, __bf16 *packed, int M, int K, int Mpad16, long total, int taps)
+{
+    for (long i = blockIdx.x * (long)blockDim.x + threadIdx.x; i < total; i += (long)gridDim.x * blockDim.x) {
+        const int pp = (int)(i & 7);
+        long t = i >> 3;
+        const int m = (int)(t % Mpad16);
+        t /= Mpad16;
+        const int h = (int)(t & 1);
+        const int kc = (int)(t >> 1);
+        const int kk = (pp < 4 ? h : 2 + h) * 4 + (pp & 3);
+        const int cb = kc / taps, tap = kc - cb * taps;
+        const int k = (cb * DN_BK + kk) * taps + tap;
+        packed[i] = (__bf16)((m < M && k < K) ? w[(long)m * K + k] : 0.f);
+    }
+}
+
+/* bf16 copy of a grouped layer: ((tile*KCH + chunk)*2 + h)*32 + r rows of 8, as above */
+__global__ void pack_grouped_bf16_kernel(const float *w, __bf16 *packed, int cg, int taps, long total)
+{
+    const int kch = 2 * taps;
+    for (long i = blockIdx.x * (long)blockDim.x + threadIdx.x; i < total; i += (long)gridDim.x * blockDim.x) {
+        const int pp = (int)(i & 7);
+        long t = i >> 3;
+        const int r = (int)(t & 31);
+        t >>= 5;
+        const int h = (int)(t & 1);
+        t >>= 1;
+        const int kc = (int)(t % kch);
+        const int tile = (int)(t / kch);
+        const int cb = kc / taps, tap = kc - cb * taps;
+        const int ch = cb * DN_BK + (pp < 4 ? h : 2 + h) * 4 + (pp & 3);
+        const int f = tile * 32 + r;
+        const bool same_group = (r / cg) == (ch / cg);
+        packed[i] = (__bf16)(same_group ? w[((long)f * cg + (ch % cg)) * taps + tap] : 0.f);
+    }
+}
+
+static inline int pack_blocks(size_t total)
+{
+    const size_t b = (total + 255) / 256;
+    return (int)(b > 8192 ? 8192 : b);
+}
+
 extern "C" void conv_pack_weights_gpu(const float *weights, float *packed, int n, int c, int groups, int size)
 {
-    const size_t total = conv_packed_floats(n, c, groups, size);
+    const size_t total = conv_packed_f32_floats(n, c, groups, size);
     if (!total) return;
+    const size_t total16 = conv_packed_bf16_floats(n, c, groups, size) * 2; /* bf16 elements */
+    __bf16 *packed16 = (__bf16 *)(packed + total);
     const int gt = conv_grouped_tile(n, c, groups, size);
     if (gt) {
-        long gb = (long)((total + 255) / 256);
-        if (gb > 8192) gb = 8192;
-        hipLaunchKernelGGL(pack_grouped_kernel, dim3((int)gb), dim3(256), 0, dn_stream(), weights, packed,
+        hipLaunchKernelGGL(pack_grouped_kernel, dim3(pack_blocks(total)), dim3(256), 0, dn_stream(), weights, packed,
                            c / groups, gt, (long)total);
+        hipLaunchKernelGGL(pack_grouped_bf16_kernel, dim3(pack_blocks(total16)), dim3(256), 0, dn_stream(), weights,
+                           packed16, c / groups, gt, (long)total16);
         dn_check_launch("conv_pack_weights_gpu");
         return;
     }
     const int K = c * size * size;
     const int mpad = (n + DN_MPAD - 1) / DN_MPAD * DN_MPAD;
-    long blocks = (long)((total + 255) / 256);
-    if (blocks > 8192) blocks = 8192;
-    hipLaunchKernelGGL(pack_weights_kernel, dim3((int)blocks), dim3(256), 0, dn_stream(), weights, packed, n,
-                       K, mpad, (long)total, tap_blocked_taps(c, groups, size));
+    const int taps = tap_blocked_taps(c, groups, size);
+    hipLaunchKernelGGL(pack_weights_kernel, dim3(pack_blocks(total)), dim3(256), 0, dn_stream(), weights, packed, n,
+                       K, mpad, (long)total, taps);
+    if (total16)
+        hipLaunchKernelGGL(pack_weights_bf16_kernel, dim3(pack_blocks(total16)), dim3(256), 0, dn_stream(), weights,
+                           packed16, n, K, conv_mpad16(n), (long)total16, taps);
     dn_check_launch("conv_pack_weights_gpu");
 }
 
@@ -757,8 +926,10 @@ extern "C" const char *conv_kernel_name(int n, int c, int groups, int size)
         bm = 32;
     }
     if (mode < 0) return "conv_direct_kernel";
-    snprintf(name, sizeof name, "conv_mfma_kernel<%d,%d,%d,64,%d%s>", bm, bm == 128 ? 128 : 256, bm == 32 ? 32 : 64,
-             mode, (g_precision == 1 && mode >= 10) ? ",true" : "");
+    const int bf16 = g_precision == 1 && mode >= 10;
+    if (bf16 && bm == 128 && n > 128) bm = 256;
+    snprintf(name, sizeof name, "conv_mfma_kernel<%d,%d,%d,64,%d%s>", bm, bm >= 128 ? 128 : 256,
+             bm == 32 ? 32 : bm == 256 ? 128 : 64, mode, bf16 ? ",true" : "");
     return name;
 }
 
@@ -773,7 +944,7 @@ static int g_cus = 0;
  * a remainder that would leave most CUs idle for a whole tile time (or, at batch 1, a grid far
  * smaller than the chip) is cut along K into `split` slices each, reduced afterwards.
  * Returns the number of whole tiles; *split = 1 means no tail. */
-static long plan_split(long tiles, int kch, int cus, int *split)
+static long plan_split(long tiles, int kch, int cus, int *split, double fixed_scale)
 {
     *split = 1;
     if (g_algo == 3 || cus <= 0) return tiles;
@@ -782,7 +953,7 @@ static long plan_split(long tiles, int kch, int cus, int *split)
     if (tail == 0 || tail * 10 >= (long)cus * 9) return tiles; /* a nearly full round: leave it */
     /* Time in units of one 16-wide K chunk.  A workgroup costs its chunks plus a fixed part
      * (first load latency, epilogue or partial store); the reduce pass costs a little more. */
-    const double fixed_whole = 5.0, fixed_slice = 8.0, reduce = 4.0;
+    const double fixed_whole = 5.0 * fixed_scale, fixed_slice = 8.0 * fixed_scale, reduce = 4.0 * fixed_scale;
     double best = (double)kch + fixed_whole;                   /* the tail as whole tiles */
     const int max_s = kch / 4 < 32 ? kch / 4 : 32;             /* at least 4 chunks per slice */
     for (int s = 2; s <= max_s; ++s) {
@@ -818,7 +989,9 @@ static void launch_tile(const mfma_args &a0, int mode)
         g_cus = prop.multiProcessorCount;
     }
     int split = 1;
-    const long whole = plan_split(total, a.KCH, g_cus, &split);
+    /* a bf16 chunk takes a small fraction of an fp32 chunk's time; the fixed costs do not shrink */
+    const int bf16 = g_precision == 1 && mode >= 10;
+    const long whole = plan_split(total, a.KCH, g_cus, &split, bf16 ? 6.0 : 1.0);
     const long tail = total - whole;
     a.whole_tiles = (int)whole;
     a.split = split;
@@ -834,18 +1007,18 @@ static void launch_tile(const mfma_args &a0, int mode)
         a.partial = g_partial;
     }
     const dim3 grid((unsigned)(a.per_xcd * 8 + tail * split));
-    if (BM > 128 && mode != 11 && mode != 13) dn_fatal("conv dispatch: the 256-row tile is only built for the tap-blocked modes");
+    if (BM > 128 && !bf16) dn_fatal("conv dispatch: the 256-row tile is only built for the bf16-operand mode");
     switch (mode) {
     case 11:
-        if (g_precision == 1)
+        if (bf16)
             DN_LAUNCH((conv_mfma_kernel<BM, BN, WM, WN, 11, true>));
-        else
+        else if constexpr (BM <= 128)
             DN_LAUNCH((conv_mfma_kernel<BM, BN, WM, WN, 11>));
         break;
     case 13:
-        if (g_precision == 1)
+        if (bf16)
             DN_LAUNCH((conv_mfma_kernel<BM, BN, WM, WN, 13, true>));
-        else
+        else if constexpr (BM <= 128)
             DN_LAUNCH((conv_mfma_kernel<BM, BN, WM, WN, 13>));
         break;
     default:
@@ -984,9 +1157,14 @@ static void conv_forward(const float *input, const float *weights, const float *
     a.sum_slope_hi = conv_split(sum_slope).hi;
     a.sum_slope_lo = conv_split(sum_slope).lo;
     a.in_records = (unsigned)((long)batch * c * h * w * 4 + (long)(w + 1) * 4);
-    a.wp_records = (unsigned)(conv_packed_floats(n, c, groups, size) * 4);
+    a.wp_records = (unsigned)(conv_packed_f32_floats(n, c, groups, size) * 4);
+    a.wp16 = packed + conv_packed_f32_floats(n, c, groups, size);
+    a.wp16_records = (unsigned)(conv_packed_bf16_floats(n, c, groups, size) * 4);
+    a.Mpad16 = a.grouped ? 32 : conv_mpad16(n);
     if (n <= 32 || a.grouped)
         launch_tile<32, 256, 32, 64>(a, mode);
+    else if (n > 128 && g_precision == 1 && mode >= 10)
+        launch_tile<256, 128, 128, 64>(a, mode);
     else if (n <= 64)
         launch_tile<64, 256, 64, 64>(a, mode);
     else
