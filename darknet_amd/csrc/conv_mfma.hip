@@ -65,6 +65,8 @@ struct mfma_args {
     const void *wp16; /* the bf16 copy of the packed weights (bf16-operand mode) */
     unsigned wp16_records;
     int Mpad16;
+    const void *in16; /* staged bf16 copy of the input, [image][C/8][H*W][8] (bf16 mode, 3x3 layers) */
+    unsigned in16_records;
     const float *biases, *scales, *mean, *var;
     float *out;
     int C, H, W, M, K, KCH, Mpad;
@@ -270,7 +272,11 @@ __device__ __forceinline__ void conv_epilogue(const mfma_args &a, f32x16 (&acc)[
     }
 }
 
-template <int BM, int BN, int WM, int WN, int MODE, bool BF16 = false>
+/* BF16: 0 = fp32 operands; 1 = bf16 weights from their packed copy, fp32 activation tiles rounded
+ * on the way into the MFMA (1x1 layers: the input is read once, straight from the fp32 tensor);
+ * 2 = both operands bf16 in LDS, the activations gathered from a staged bf16 copy of the input
+ * (3x3 layers, which read every input element nine times). */
+template <int BM, int BN, int WM, int WN, int MODE, int BF16 = 0>
 __global__ __launch_bounds__(DN_THREADS, (BM == 128 ? 3 : 2)) void conv_mfma_kernel(mfma_args a)
 {
     constexpr int TM = WM / 32, TN = WN / 32;
@@ -283,14 +289,23 @@ __global__ __launch_bounds__(DN_THREADS, (BM == 128 ? 3 : 2)) void conv_mfma_ker
     /* Four separate LDS objects rather than two [2][...] arrays: the compiler makes every LDS read
      * wait (vmcnt) for direct-to-LDS loads it cannot prove disjoint from it, and it can only
      * prove that for distinct objects. */
+    constexpr bool V3 = BF16 == 2;
+    static_assert(!V3 || (TAPB && KS == 3), "the staged-input variant serves the tap-blocked 3x3 layers");
     constexpr int A_FLOATS = BF16 ? BM * DN_BK / 2 : BM * DN_BK; /* bf16 rows are 32 bytes */
-    __shared__ __attribute__((aligned(16))) float As0[A_FLOATS], As1[A_FLOATS];
-    __shared__ __attribute__((aligned(16))) float Bs0[BN * DN_BK], Bs1[BN * DN_BK];
-    /* the bf16 variant keeps three chunks in flight: four stages */
-    __shared__ __attribute__((aligned(16))) float As2[BF16 ? A_FLOATS : 4], As3[BF16 ? A_FLOATS : 4];
-    __shared__ __attribute__((aligned(16))) float Bs2[BF16 ? BN * DN_BK : 4], Bs3[BF16 ? BN * DN_BK : 4];
-#define A_BUF(b) ((b) == 0 ? As0 : (b) == 1 ? As1 : (b) == 2 ? As2 : As3)
-#define B_BUF(b) ((b) == 0 ? Bs0 : (b) == 1 ? Bs1 : (b) == 2 ? Bs2 : Bs3)
+    constexpr int B_FLOATS = V3 ? BN * DN_BK / 2 : BN * DN_BK;
+    __shared__ __attribute__((aligned(16))) float As0[V3 ? 4 : A_FLOATS], As1[V3 ? 4 : A_FLOATS];
+    __shared__ __attribute__((aligned(16))) float Bs0[V3 ? 4 : B_FLOATS], Bs1[V3 ? 4 : B_FLOATS];
+    /* the bf16 variants keep three chunks in flight: four stages */
+    __shared__ __attribute__((aligned(16))) float As2[BF16 == 1 ? A_FLOATS : 4], As3[BF16 == 1 ? A_FLOATS : 4];
+    __shared__ __attribute__((aligned(16))) float Bs2[BF16 == 1 ? B_FLOATS : 4], Bs3[BF16 == 1 ? B_FLOATS : 4];
+    /* staged-input variant: one object per stage, [A | B], each at least the 8 KB a wave's
+     * epilogue turn needs */
+    constexpr int S_FLOATS = V3 ? A_FLOATS + B_FLOATS : 4;
+    static_assert(!V3 || S_FLOATS >= 2048, "a stage doubles as one wave's epilogue buffer");
+    __shared__ __attribute__((aligned(16))) float S0[S_FLOATS], S1[S_FLOATS], S2[S_FLOATS], S3[S_FLOATS];
+#define S_BUF(b) ((b) == 0 ? S0 : (b) == 1 ? S1 : (b) == 2 ? S2 : S3)
+#define A_BUF(b) (V3 ? S_BUF(b) : ((b) == 0 ? As0 : (b) == 1 ? As1 : (b) == 2 ? As2 : As3))
+#define B_BUF(b) (V3 ? S_BUF(b) + A_FLOATS : ((b) == 0 ? Bs0 : (b) == 1 ? Bs1 : (b) == 2 ? Bs2 : Bs3))
 
     /* XCD-aware tile order: workgroup id -> (xcd, slot) -> linear tile with tile_m fastest. */
     const int bid = blockIdx.x;
@@ -336,14 +351,42 @@ __global__ __launch_bounds__(DN_THREADS, (BM == 128 ? 3 : 2)) void conv_mfma_ker
     const __amdgpu_buffer_rsrc_t w_rsrc = __builtin_amdgcn_make_buffer_rsrc(
         (void *)(BF16 ? a.wp16 : (const void *)a.wp), 0, (int)(BF16 ? a.wp16_records : a.wp_records), 0x00020000);
     const int bias = (TAPB && KS == 3) ? a.W + 1 : 0;
-    const __amdgpu_buffer_rsrc_t in_rsrc = __builtin_amdgcn_make_buffer_rsrc(
-        (void *)(a.in - bias), 0, (int)a.in_records, 0x00020000);
+    const __amdgpu_buffer_rsrc_t in_rsrc =
+        V3 ? __builtin_amdgcn_make_buffer_rsrc((void *)((const char *)a.in16 - (long)bias * 16), 0, (int)a.in16_records,
+                                               0x00020000)
+           : __builtin_amdgcn_make_buffer_rsrc((void *)(a.in - bias), 0, (int)a.in_records, 0x00020000);
 
     /* per column group handled by this wave: the lane's pixel */
     unsigned voff_px[NG_PER_WAVE]; /* byte offset of (image, channel kk [tap-blocked] or 0, oy*s, ox*s) */
     unsigned vmask[NG_PER_WAVE];   /* tap-blocked: bit t set when tap t lies inside the image */
     int iy0[NG_PER_WAVE], ix0[NG_PER_WAVE]; /* reference order: top-left input pixel of the window;
                                              * a column beyond N gets iy0 far outside the image */
+    /* staged-input variant: the input is [image][C/8][H*W] rows of eight bf16 channels, so a lane
+     * fetches a column's eight k of one half with one 16-byte load: a wave-load is 64 consecutive
+     * columns of one k half, and this wave serves half `lkh`, 64-column blocks lblk0 .. */
+    constexpr int NBW = V3 ? BN / 128 : 1;       /* 64-column blocks per wave */
+    const int lkh = wave >> 1, lblk0 = (wave & 1) * NBW;
+    unsigned c_voff[NBW], c_mask[NBW];
+    if constexpr (V3) {
+#pragma unroll
+        for (int g = 0; g < NBW; ++g) {
+            const long ncol = n0 + (lblk0 + g) * 64 + lane;
+            const bool col_ok = ncol < a.Ntotal;
+            const unsigned nn = col_ok ? (unsigned)ncol : 0u;
+            const int b = (int)(nn / (unsigned)a.P);
+            const int p = (int)nn - b * a.P;
+            const int oy = (int)((unsigned)p / (unsigned)a.OW);
+            const int ox = p - oy * a.OW;
+            const int y0 = oy * a.stride - 1, x0 = ox * a.stride - 1; /* pad == 1 */
+            c_voff[g] = (unsigned)((((long)b * (a.C >> 3) + lkh) * HW + (long)(oy * a.stride) * a.W + ox * a.stride) * 16);
+            c_mask[g] = 0;
+            if (col_ok) {
+#pragma unroll
+                for (int t = 0; t < 9; ++t)
+                    if ((unsigned)(y0 + t / 3) < (unsigned)a.H && (unsigned)(x0 + t % 3) < (unsigned)a.W) c_mask[g] |= 1u << t;
+            }
+        }
+    }
 #pragma unroll
     for (int g = 0; g < NG_PER_WAVE; ++g) {
         const long ncol = n0 + (wave * NG_PER_WAVE + g) * 16 + nl;
@@ -430,7 +473,21 @@ __global__ __launch_bounds__(DN_THREADS, (BM == 128 ? 3 : 2)) void conv_mfma_ker
         }
         }
         /* B */
-        if (TAPB) {
+        if constexpr (V3) {
+            const int ky = (ld_tap * 11) >> 5, kx = ld_tap - 3 * ((ld_tap * 11) >> 5); /* tap/3, tap%3 */
+            const int shift = (ky - 1) * a.W + (kx - 1);
+            const unsigned soff0 = (unsigned)(((long)2 * ld_cb * HW + shift + bias) * 16); /* wave-uniform */
+#pragma unroll
+            for (int g = 0; g < NBW; ++g) {
+                const unsigned voff = ((c_mask[g] >> ld_tap) & 1u) ? c_voff[g] : 0xFFFFFFF0u;
+                __builtin_amdgcn_raw_ptr_buffer_load_lds(in_rsrc, (lds_ptr)&B_BUF(buf)[(lkh * BN + (lblk0 + g) * 64) * 4], 16,
+                                                         voff, soff0, 0, 0);
+            }
+            if (++ld_tap == TAPS) {
+                ld_tap = 0;
+                ++ld_cb;
+            }
+        } else if (TAPB) {
             const int ky = (ld_tap * 11) >> 5, kx = ld_tap - 3 * ((ld_tap * 11) >> 5); /* tap/3, tap%3 */
             const int shift = KS == 1 ? 0 : (ky - 1) * a.W + (kx - 1);       /* pad == 1 for 3x3 */
             const unsigned soff0 = (unsigned)((ld_cb * 16 * HW + shift + bias) * 4); /* wave-uniform */
@@ -488,33 +545,16 @@ __global__ __launch_bounds__(DN_THREADS, (BM == 128 ? 3 : 2)) void conv_mfma_ker
     /* loads one wave issues per chunk, for the s_waitcnt immediates of the bf16 pipeline (the A
      * loads are left out where not every wave issues them: those waves wait for one load more
      * than they must) */
-    constexpr int LPC = (BF16 && BM >= 128 ? BM / 128 : 0) + 4 * NG_PER_WAVE;
+    constexpr int LPC = (BF16 && BM >= 128 ? BM / 128 : 0) + (V3 ? NBW : 4 * NG_PER_WAVE);
     /* s_waitcnt on vmcnt alone: simm16 = vmcnt[3:0] | expcnt(7) << 4 | lgkmcnt(15) << 8 | vmcnt[5:4] << 14 */
 #define DN_WAIT_VM(n) __builtin_amdgcn_s_waitcnt(((n) & 15) | (7 << 4) | (15 << 8) | (((n) >> 4) << 14))
     static_assert(2 * LPC < 64, "vmcnt is a 6-bit counter");
 
-    if constexpr (BF16) {
-        const int nch = kc_end - kc_begin;
-        load_chunk(kc_begin, 0);
-        if (nch > 1) load_chunk(kc_begin + 1, 1);
-        if (nch > 2) load_chunk(kc_begin + 2, 2);
-        if (nch > 2)
-            DN_WAIT_VM(2 * LPC);
-        else if (nch > 1)
-            DN_WAIT_VM(LPC);
-        else
-            __builtin_amdgcn_s_waitcnt(0);
-        __builtin_amdgcn_s_barrier();
-    } else {
-        load_chunk(kc_begin, 0);
-        __builtin_amdgcn_s_waitcnt(0);
-        __syncthreads();
-    }
+    float4 av[2][TM], bv[BF16 == 1 ? 2 : 1][2][TN]; /* MFMA operands of a chunk: [k half][32-row block] */
+    bf16x8 a8[2][BF16 ? TM : 1];             /* bf16 modes: a row's eight k of this lane's half, two register sets */
+    bf16x8 b8s[2][V3 ? TN : 1];              /* staged input: a column's eight k likewise */
 
-    float4 av[2][TM], bv[2][TN]; /* MFMA operands of the current chunk: [k half][32-row block] */
-    bf16x8 a8[BF16 ? TM : 1];                /* bf16 mode: a row's eight k of this lane's half */
-
-    auto read_operands = [&](int buf) {
+    auto read_operands = [&](int buf, int r) {
 #pragma unroll
         for (int hb = 0; hb < 2; ++hb) {
             if constexpr (!BF16) {
@@ -522,16 +562,41 @@ __global__ __launch_bounds__(DN_THREADS, (BM == 128 ? 3 : 2)) void conv_mfma_ker
                 for (int i = 0; i < TM; ++i)
                     av[hb][i] = *(const float4 *)&A_BUF(buf)[((hb * 2 + kh) * BM + wm0 + i * 32 + li) * 4];
             }
+            if constexpr (!V3) {
 #pragma unroll
-            for (int j = 0; j < TN; ++j)
-                bv[hb][j] = *(const float4 *)&B_BUF(buf)[((hb * 2 + kh) * BN + wn0 + j * 32 + li) * 4];
+                for (int j = 0; j < TN; ++j)
+                    bv[BF16 == 1 ? r : 0][hb][j] = *(const float4 *)&B_BUF(buf)[((hb * 2 + kh) * BN + wn0 + j * 32 + li) * 4];
+            }
         }
         if constexpr (BF16) {
 #pragma unroll
             for (int i = 0; i < TM; ++i)
-                a8[i] = *(const bf16x8 *)&A_BUF(buf)[(kh * BM + wm0 + i * 32 + li) * 4];
+                a8[r][i] = *(const bf16x8 *)&A_BUF(buf)[(kh * BM + wm0 + i * 32 + li) * 4];
+        }
+        if constexpr (V3) {
+#pragma unroll
+            for (int j = 0; j < TN; ++j)
+                b8s[r][j] = *(const bf16x8 *)&B_BUF(buf)[(kh * BN + wn0 + j * 32 + li) * 4];
         }
     };
+
+    if constexpr (BF16) {
+        /* chunks 0..2 requested; chunks 0 and 1 must have landed before the first step */
+        const int nch = kc_end - kc_begin;
+        load_chunk(kc_begin, 0);
+        if (nch > 1) load_chunk(kc_begin + 1, 1);
+        if (nch > 2) load_chunk(kc_begin + 2, 2);
+        if (nch > 2)
+            DN_WAIT_VM(LPC);
+        else
+            __builtin_amdgcn_s_waitcnt(0);
+        __builtin_amdgcn_s_barrier();
+        read_operands(0, 0);
+    } else {
+        load_chunk(kc_begin, 0);
+        __builtin_amdgcn_s_waitcnt(0);
+        __syncthreads();
+    }
 
     auto mfma_half = [&](int hb) {
 #pragma unroll
@@ -541,32 +606,38 @@ __global__ __launch_bounds__(DN_THREADS, (BM == 128 ? 3 : 2)) void conv_mfma_ker
                 const float ae = s == 0 ? av[hb][i].x : s == 1 ? av[hb][i].y : s == 2 ? av[hb][i].z : av[hb][i].w;
 #pragma unroll
                 for (int j = 0; j < TN; ++j) {
-                    const float be = s == 0 ? bv[hb][j].x : s == 1 ? bv[hb][j].y : s == 2 ? bv[hb][j].z : bv[hb][j].w;
+                    const float4 b4 = bv[0][hb][j];
+                    const float be = s == 0 ? b4.x : s == 1 ? b4.y : s == 2 ? b4.z : b4.w;
                     acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(be, ae, acc[i][j], 0, 0, 0);
                 }
             }
         }
     };
 
-    /* Reduced-precision variant: the weights come from their bf16 copy, whose rows hold the eight k
-     * of a lane half in the order the activation slots give them (slot kh, then slot 2 + kh);
-     * the activations stay fp32 tiles in LDS and are rounded to bf16 (nearest even) on the way
-     * into one v_mfma_f32_32x32x16_bf16, which contracts all 16 k of the chunk at once.
-     * Products and sums stay fp32, so does everything after the accumulators. */
-    auto mfma_chunk = [&]() {
+    /* Reduced-precision variants: the weights come from their bf16 copy, whose rows hold the eight
+     * k of a lane half in the order the activations give them.  Variant 1 keeps the activations
+     * as fp32 tiles in LDS and rounds them to bf16 (nearest even) on the way into the MFMA;
+     * variant 2 reads them already rounded from the staged copy.  One v_mfma_f32_32x32x16_bf16
+     * contracts all 16 k of the chunk; products and sums stay fp32, so does everything after the
+     * accumulators. */
+    auto mfma_chunk = [&](int r) {
         if constexpr (BF16) {
             bf16x8 b8[TN];
 #pragma unroll
             for (int j = 0; j < TN; ++j) {
-                const f32x8 f = {bv[0][j].x, bv[0][j].y, bv[0][j].z, bv[0][j].w,
-                                 bv[1][j].x, bv[1][j].y, bv[1][j].z, bv[1][j].w};
-                b8[j] = __builtin_convertvector(f, bf16x8);
+                if constexpr (V3) {
+                    b8[j] = b8s[r][j];
+                } else {
+                    const float4 lo = bv[BF16 == 1 ? r : 0][0][j], hi = bv[BF16 == 1 ? r : 0][1][j];
+                    const f32x8 f = {lo.x, lo.y, lo.z, lo.w, hi.x, hi.y, hi.z, hi.w};
+                    b8[j] = __builtin_convertvector(f, bf16x8);
+                }
             }
 #pragma unroll
             for (int i = 0; i < TM; ++i)
 #pragma unroll
                 for (int j = 0; j < TN; ++j)
-                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(b8[j], a8[i], acc[i][j], 0, 0, 0);
+                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(b8[j], a8[r][i], acc[i][j], 0, 0, 0);
         } else {
             mfma_half(0);
             mfma_half(1);
@@ -581,48 +652,47 @@ __global__ __launch_bounds__(DN_THREADS, (BM == 128 ? 3 : 2)) void conv_mfma_ker
     auto step = [&](int kc_next, int buf) {
         load_chunk(kc_next, buf ^ 1);
         __builtin_amdgcn_sched_barrier(0);
-        read_operands(buf);
+        read_operands(buf, 0);
         __builtin_amdgcn_sched_barrier(0);
-        mfma_chunk();
+        mfma_chunk(0);
         __builtin_amdgcn_sched_barrier(0);
         __builtin_amdgcn_s_waitcnt(0);
         __syncthreads();
     };
     auto last = [&](int buf) {
-        read_operands(buf);
-        mfma_chunk();
+        read_operands(buf, 0);
+        mfma_chunk(0);
     };
 
     if constexpr (BF16) {
-        /* Four LDS stages, prefetch distance three: a bf16 chunk is 8 (or 4, 2) MFMAs, far shorter
-         * than a round trip to memory, so chunks kc+1 and kc+2 are already in flight when chunk
-         * kc+3 is requested, and a step waits only until kc+1 has landed (vmcnt counts loads, which
-         * complete in order).  __syncthreads() would drain every load (its fences wait for
-         * vmcnt(0) because direct-to-LDS loads count as LDS writes), so the barrier is the bare
-         * instruction: the explicit vmcnt wait before it covers the loads, and every LDS read of
-         * a stage has been consumed by MFMAs before the wave reaches the barrier after which the
-         * stage is overwritten. */
-        auto bstep = [&](int kcur, int buf) {
+        /* Four LDS stages and two register sets.  A bf16 chunk is 8 (or 4, 2) MFMAs, far shorter
+         * than a trip to memory or even to LDS, so a step overlaps three things: the LDS reads of
+         * chunk kc+1 into the other register set, the request for chunk kc+3, and the MFMAs of
+         * chunk kc from registers read one step earlier.  On entry chunks up to kc+1 are in LDS
+         * and visible, chunk kc+2 is in flight; the step ends when kc+2 has landed for every wave
+         * (vmcnt counts this wave's loads, which complete in order; the barrier publishes them).
+         * The stage requested into is the one of chunk kc-1, last read two steps ago.
+         * __syncthreads() would drain every load (its fences wait for vmcnt(0) because
+         * direct-to-LDS loads count as LDS writes), so the barrier is the bare instruction. */
+        auto bstep = [&](int kcur, int buf, int r) {
             const int rem = kc_end - 1 - kcur; /* chunks after this one (wave-uniform) */
+            if (rem >= 1) read_operands((buf + 1) & 3, r ^ 1);
+            __builtin_amdgcn_sched_barrier(0);
             if (rem >= 3) load_chunk(kcur + 3, (buf + 3) & 3);
             __builtin_amdgcn_sched_barrier(0);
-            read_operands(buf);
-            __builtin_amdgcn_sched_barrier(0);
-            mfma_chunk();
+            mfma_chunk(r);
             __builtin_amdgcn_sched_barrier(0);
             if (rem >= 3)
-                DN_WAIT_VM(2 * LPC);
-            else if (rem == 2)
                 DN_WAIT_VM(LPC);
             else
-                __builtin_amdgcn_s_waitcnt(0);
-            if (rem >= 1) __builtin_amdgcn_s_barrier();
+                DN_WAIT_VM(0);
+            if (rem >= 2) __builtin_amdgcn_s_barrier();
         };
         for (int kc = kc_begin; kc < kc_end; kc += 4) {
-            bstep(kc, 0);
-            if (kc + 1 < kc_end) bstep(kc + 1, 1);
-            if (kc + 2 < kc_end) bstep(kc + 2, 2);
-            if (kc + 3 < kc_end) bstep(kc + 3, 3);
+            bstep(kc, 0, 0);
+            if (kc + 1 < kc_end) bstep(kc + 1, 1, 1);
+            if (kc + 2 < kc_end) bstep(kc + 2, 2, 0);
+            if (kc + 3 < kc_end) bstep(kc + 3, 3, 1);
         }
     } else {
     int kc = kc_begin;
@@ -652,9 +722,10 @@ __global__ __launch_bounds__(DN_THREADS, (BM == 128 ? 3 : 2)) void conv_mfma_ker
                     ws[((wave * TM * TN + i * TN + j) * 16 + r) * 64 + lane] = acc[i][j][r];
     } else {
         __syncthreads(); /* every wave has read its last operands: the LDS buffers are free */
-        float *E = BM >= 128 ? (BF16 ? (wave == 0 ? Bs2 : wave == 1 ? Bs3 : wave == 2 ? Bs0 : Bs1)
-                                     : (wave == 0 ? As0 : wave == 1 ? As1 : wave == 2 ? Bs0 : Bs1))
-                             : (wave < 2 ? Bs0 : Bs1) + (wave & 1) * 2048;
+        float *E = V3 ? S_BUF(wave)
+                   : BM >= 128 ? (BF16 ? (wave == 0 ? Bs2 : wave == 1 ? Bs3 : wave == 2 ? Bs0 : Bs1)
+                                       : (wave == 0 ? As0 : wave == 1 ? As1 : wave == 2 ? Bs0 : Bs1))
+                               : (wave < 2 ? Bs0 : Bs1) + (wave & 1) * 2048;
         conv_epilogue<TM, TN>(a, acc, E, m0, n0, wm0, wn0, lane);
     }
 }
@@ -818,8 +889,8 @@ extern "C" size_t conv_packed_floats(int n, int c, int groups, int size)
 }
 
 /* bf16 copy of a tap-blocked layer: element ((chunk*2 + h)*Mpad16 + m)*8 + p is the weight that the
- * fp32 layout keeps at slot (p < 4 ? h : 2 + h), position p % 4 of the same chunk and row, rounded
- * to nearest even. */
+ * fp32 layout keeps at slot (p < 4 ? h : 2 + h), position p % 4 of the same chunk and row (1x1
+ * layers) or at position 8*h + p of the chunk (3x3 layers), rounded to nearest even. */
 __global__ void pack_weights_bf16_kernel(const float *w, __bf16 *packed, int M, int K, int Mpad16, long total, int taps)
 {
     for (long i = blockIdx.x * (long)blockDim.x + threadIdx.x; i < total; i += (long)gridDim.x * blockDim.x) {
@@ -829,7 +900,9 @@ __global__ void pack_weights_bf16_kernel(const float *w, __bf16 *packed, int M, 
         t /= Mpad16;
         const int h = (int)(t & 1);
         const int kc = (int)(t >> 1);
-        const int kk = (pp < 4 ? h : 2 + h) * 4 + (pp & 3);
+        /* 1x1: the order the fp32 activation slots give (slot h, then slot 2 + h); 3x3: the staged
+         * input's, eight consecutive channels per half */
+        const int kk = taps == 1 ? (pp < 4 ? h : 2 + h) * 4 + (pp & 3) : 8 * h + pp;
         const int cb = kc / taps, tap = kc - cb * taps;
         const int k = (cb * DN_BK + kk) * taps + tap;
         packed[i] = (__bf16)((m < M && k < K) ? w[(long)m * K + k] : 0.f);
@@ -850,7 +923,7 @@ __global__ void pack_grouped_bf16_kernel(const float *w, __bf16 *packed, int cg,
         const int kc = (int)(t % kch);
         const int tile = (int)(t / kch);
         const int cb = kc / taps, tap = kc - cb * taps;
-        const int ch = cb * DN_BK + (pp < 4 ? h : 2 + h) * 4 + (pp & 3);
+        const int ch = cb * DN_BK + (taps == 1 ? (pp < 4 ? h : 2 + h) * 4 + (pp & 3) : 8 * h + pp);
         const int f = tile * 32 + r;
         const bool same_group = (r / cg) == (ch / cg);
         packed[i] = (__bf16)(same_group ? w[((long)f * cg + (ch % cg)) * taps + tap] : 0.f);
@@ -888,6 +961,26 @@ extern "C" void conv_pack_weights_gpu(const float *weights, float *packed, int n
                            packed16, n, K, conv_mpad16(n), (long)total16, taps);
     dn_check_launch("conv_pack_weights_gpu");
 }
+
+/* ---- bf16 staging of a 3x3 layer's input -------------------------------------------------- */
+/* [image][C][H*W] fp32 -> [image][C/8][H*W] rows of eight bf16 (nearest even): one thread per
+ * output row; for each of its eight channels consecutive threads read consecutive pixels, and
+ * they write consecutive 16-byte rows. */
+__global__ void stage_bf16_kernel(const float *in, bf16x8 *out, int cblocks, int HW, long total)
+{
+    const long i = blockIdx.x * (long)blockDim.x + threadIdx.x;
+    if (i >= total) return;
+    const long img_blk = i / HW;                 /* image * cblocks + block */
+    const int pix = (int)(i - img_blk * HW);
+    const float *src = in + img_blk * 8 * HW + pix;
+    f32x8 f;
+#pragma unroll
+    for (int j = 0; j < 8; ++j) f[j] = src[(long)j * HW];
+    out[i] = __builtin_convertvector(f, bf16x8);
+}
+
+static float *g_stage = 0; /* staged input of the bf16 3x3 path, grown on demand */
+static size_t g_stage_floats = 0;
 
 /* ---- dispatch ---------------------------------------------------------------------------- */
 /* One-shot kernel timing: the next MFMA convolution launches its main kernel with these two
@@ -929,7 +1022,7 @@ extern "C" const char *conv_kernel_name(int n, int c, int groups, int size)
     const int bf16 = g_precision == 1 && mode >= 10;
     if (bf16 && bm == 128 && n > 128) bm = 256;
     snprintf(name, sizeof name, "conv_mfma_kernel<%d,%d,%d,64,%d%s>", bm, bm >= 128 ? 128 : 256,
-             bm == 32 ? 32 : bm == 256 ? 128 : 64, mode, bf16 ? ",true" : "");
+             bm == 32 ? 32 : bm == 256 ? 128 : 64, mode, !bf16 ? "" : mode == 13 ? ",2" : ",1");
     return name;
 }
 
@@ -1011,13 +1104,13 @@ static void launch_tile(const mfma_args &a0, int mode)
     switch (mode) {
     case 11:
         if (bf16)
-            DN_LAUNCH((conv_mfma_kernel<BM, BN, WM, WN, 11, true>));
+            DN_LAUNCH((conv_mfma_kernel<BM, BN, WM, WN, 11, 1>));
         else if constexpr (BM <= 128)
             DN_LAUNCH((conv_mfma_kernel<BM, BN, WM, WN, 11>));
         break;
     case 13:
         if (bf16)
-            DN_LAUNCH((conv_mfma_kernel<BM, BN, WM, WN, 13, true>));
+            DN_LAUNCH((conv_mfma_kernel<BM, BN, WM, WN, 13, 2>));
         else if constexpr (BM <= 128)
             DN_LAUNCH((conv_mfma_kernel<BM, BN, WM, WN, 13>));
         break;
@@ -1161,6 +1254,22 @@ static void conv_forward(const float *input, const float *weights, const float *
     a.wp16 = packed + conv_packed_f32_floats(n, c, groups, size);
     a.wp16_records = (unsigned)(conv_packed_bf16_floats(n, c, groups, size) * 4);
     a.Mpad16 = a.grouped ? 32 : conv_mpad16(n);
+    a.in16 = 0;
+    a.in16_records = 0;
+    if (g_precision == 1 && mode == 13) {
+        /* the 3x3 bf16 kernel gathers from a bf16 copy of the input, eight channels per 16 bytes */
+        const long rows = (long)batch * (c / 8) * h * w;
+        const size_t need = (size_t)rows * 4 + 64;
+        if (need > g_stage_floats) {
+            if (g_stage) hip_free(g_stage);
+            g_stage = hip_make_array(0, need);
+            g_stage_floats = need;
+        }
+        hipLaunchKernelGGL(stage_bf16_kernel, dim3((unsigned)((rows + 255) / 256)), dim3(256), 0, dn_stream(), input,
+                           (bf16x8 *)g_stage, c / 8, h * w, rows);
+        a.in16 = g_stage;
+        a.in16_records = (unsigned)(rows * 16 + (long)(w + 1) * 16);
+    }
     if (n <= 32 || a.grouped)
         launch_tile<32, 256, 32, 64>(a, mode);
     else if (n > 128 && g_precision == 1 && mode >= 10)
