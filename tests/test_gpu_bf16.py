@@ -49,6 +49,11 @@ BF16_SHAPES = [  # b, c, h, w, n, size, stride, pad, groups, act
     (1, 64, 19, 19, 32, 1, 1, 0, 1, "linear"),      # 32-row tile
     (2, 1024, 13, 13, 255, 1, 1, 0, 1, "linear"),   # ragged M, K-split at this size
     (2, 128, 14, 14, 128, 3, 1, 1, 32, "leaky"),    # grouped 32-filter tiles
+    (5, 16, 7, 9, 130, 3, 1, 1, 1, "logistic"),     # one chunk per tap, tiny images, ragged M on the 128-row tile
+    (3, 64, 10, 10, 300, 3, 1, 1, 1, "leaky"),      # 256-row tiles, the second one ragged; N below one tile
+    (1, 32, 20, 21, 32, 3, 2, 1, 1, "relu"),        # 32-row tile on the staged-input variant, stride 2, odd width
+    (2, 48, 13, 13, 200, 1, 1, 0, 1, "leaky"),      # 1x1, 3 chunks (shorter than the pipeline), 169 pixels per image
+    (2, 16, 6, 6, 256, 1, 1, 0, 1, "linear"),       # a single chunk
 ]
 
 
