@@ -10,16 +10,22 @@
  * straight from the NCHW input (the index map of src/im2col.c:26-35) into LDS.
  *
  * Tiling (64-wide wavefronts, 4 waves per workgroup):
- *   workgroup tile BM x BN x 16; wave tile WM x WN built from 32x32 accumulators of
- *   v_mfma_f32_32x32x2_f32 (TM x TN of them).  LDS holds A as [BM][16] and B as [BN][16] floats
- *   (k contiguous, 16-byte slots XOR-swizzled by row instead of padded), double buffered; one ds_read_b128 per operand
- *   row feeds four MFMA k-steps.  Within a 16-wide chunk the k index a lane uses at step s of
- *   half hb is hb*8 + (lane/32)*4 + s for A and B alike, a bijection of the chunk, so the
- *   result is the plain sum over k.
+ *   workgroup tile BM x BN x 16 (128x128; 64x256 / 32x256 for layers with few filters); wave
+ *   tile WM x WN built from 32x32 accumulators of v_mfma_f32_32x32x2_f32 (TM x TN of them).
+ *   LDS holds a chunk of A as [4 slots][BM][4 floats] and of B as [4 slots][BN][4 floats]
+ *   (k = 4*slot + j), written by direct-to-LDS buffer loads and double buffered; one
+ *   ds_read_b128 per operand row feeds four MFMA k-steps.  Within a 16-wide chunk the k index a
+ *   lane uses at step s of half hb is 4*(2*hb + lane/32) + s for A and B alike, a bijection of
+ *   the chunk, so the result is the plain sum over k.
  *   Global loads for chunk i+1 are issued before the MFMAs of chunk i and land in LDS after
  *   them (one barrier per chunk).
- * Weights are pre-packed to [K/16][Mpad][16] (zero padded, Mpad multiple of 128) so the A tile
- * is one contiguous, 16-byte aligned block for any BM.
+ * Weights are pre-packed to [K/16][4 slots][Mpad][4] (zero padded, Mpad multiple of 128) so a
+ * wave-load of A is one contiguous kilobyte for any BM; a bf16 copy for the reduced-precision
+ * variants follows in the same buffer.
+ * The last partial round of tiles is cut along K into slices that park raw accumulators and are
+ * summed in slice order by conv_reduce_kernel (deterministic).
+ * Epilogue: batch-norm, bias and activation in the accumulator layout, a turn through LDS, then
+ * 256-byte row stores; a same-geometry residual add (shortcut layer) can ride along.
  *
  * Order of K.  The sum over k does not care about the order as long as A and B agree, and the
  * packing step can permute K for free, so two orders are used:

@@ -138,7 +138,9 @@ void forward_convolutional_shortcut_gpu(const float *input, const float *weights
 
 /* Weight repack for the MFMA kernel (the natural hook is push_convolutional_layer,
  * src/convolutional_kernels.cu:286-297).  conv_packed_floats() == 0 means the layer does not
- * use a packed copy (grouped convolutions). */
+ * use a packed copy (grouped convolutions outside the 32-filter block-diagonal scheme).  The
+ * buffer holds the fp32 layout and, for layers the bf16-operand mode can serve, a bf16 copy
+ * behind it (half as many bytes again), so conv_set_precision() needs no repacking. */
 size_t conv_packed_floats(int n, int c, int groups, int size);
 void conv_pack_weights_gpu(const float *weights, float *packed, int n, int c, int groups, int size);
 
