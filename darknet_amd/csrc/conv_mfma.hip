@@ -945,7 +945,7 @@ static inline int pack_blocks(size_t total)
 extern "C" void conv_pack_weights_gpu(const float *weights, float *packed, int n, int c, int groups, int size)
 {
     const size_t total = conv_packed_f32_floats(n, c, groups, size);
-    if (!total) return;
+    if (!total || hip_parse_only()) return;
     const size_t total16 = conv_packed_bf16_floats(n, c, groups, size) * 2; /* bf16 elements */
     __bf16 *packed16 = (__bf16 *)(packed + total);
     const int gt = conv_grouped_tile(n, c, groups, size);

@@ -50,9 +50,25 @@ void dn_check_launch(const char *what)
     }
 }
 
+/* Parse-only mode: cfg parsing, layer tables and weights-file reading/writing work on host memory
+ * alone (a machine without a GPU can inspect a network); nothing is allocated on or copied to a
+ * device, and every entry point that would launch work ends the process instead of computing
+ * anything on the host. */
+static int g_parse_only = 0;
+void hip_set_parse_only(int on) { g_parse_only = on ? 1 : 0; }
+int hip_parse_only(void) { return g_parse_only; }
+void hip_require_device(const char *what)
+{
+    if (g_parse_only) {
+        fprintf(stderr, "%s: the library is in parse-only mode, no device work is possible\n", what);
+        exit(-1);
+    }
+}
+
 void hip_set_device(int n)
 {
     gpu_index = n;
+    if (g_parse_only) return;
     hip_check_error(hipSetDevice(n));
 }
 
@@ -83,6 +99,7 @@ float *hip_make_array(float *x, size_t n)
 {
     float *x_gpu = 0;
     size_t size = sizeof(float) * (n ? n : 1);
+    if (g_parse_only) return 0;
     hip_check_error(hipMalloc((void **)&x_gpu, size));
     if (!x_gpu) dn_fatal("hipMalloc returned a null pointer");
     if (x) {
@@ -97,6 +114,7 @@ int *hip_make_int_array(int *x, size_t n)
 {
     int *x_gpu = 0;
     size_t size = sizeof(int) * (n ? n : 1);
+    if (g_parse_only) return 0;
     hip_check_error(hipMalloc((void **)&x_gpu, size));
     if (!x_gpu) dn_fatal("hipMalloc returned a null pointer");
     if (x) hip_check_error(hipMemcpy(x_gpu, x, sizeof(int) * n, hipMemcpyHostToDevice));
@@ -106,6 +124,7 @@ int *hip_make_int_array(int *x, size_t n)
 
 void hip_free(float *x_gpu)
 {
+    if (g_parse_only) return;
     hip_check_error(hipFree(x_gpu));
 }
 
@@ -176,6 +195,7 @@ static void staged_copy(char *dev, char *host, size_t bytes, int to_device)
  * queued on a non-null stream is drained first so the copy sees it. */
 void hip_push_array(float *x_gpu, float *x, size_t n)
 {
+    if (g_parse_only) return; /* the host copy is the only copy */
     if (sizeof(float) * n >= DN_STAGE_MIN) {
         staged_copy((char *)x_gpu, (char *)x, sizeof(float) * n, 1);
         return;
@@ -186,6 +206,7 @@ void hip_push_array(float *x_gpu, float *x, size_t n)
 
 void hip_pull_array(float *x_gpu, float *x, size_t n)
 {
+    if (g_parse_only) return;
     if (sizeof(float) * n >= DN_STAGE_MIN) {
         staged_copy((char *)x_gpu, (char *)x, sizeof(float) * n, 0);
         return;
@@ -196,12 +217,14 @@ void hip_pull_array(float *x_gpu, float *x, size_t n)
 
 void hip_push_int_array(int *x_gpu, int *x, size_t n)
 {
+    if (g_parse_only) return;
     if (g_stream) hip_check_error(hipStreamSynchronize(g_stream));
     hip_check_error(hipMemcpy(x_gpu, x, sizeof(int) * n, hipMemcpyHostToDevice));
 }
 
 void hip_pull_int_array(int *x_gpu, int *x, size_t n)
 {
+    if (g_parse_only) return;
     if (g_stream) hip_check_error(hipStreamSynchronize(g_stream));
     hip_check_error(hipMemcpy(x, x_gpu, sizeof(int) * n, hipMemcpyDeviceToHost));
 }

@@ -17,6 +17,10 @@ void dn_fatal(const char *msg);
 /* Checks the sticky launch error after a kernel launch (check_error(cudaPeekAtLastError())
  * follows every launch in the reference, e.g. src/blas_kernels.cu:27). */
 void dn_check_launch(const char *what);
+/* Ends the process with a message naming `what` when the library is in parse-only mode
+ * (hip_set_parse_only in darknet_hip.h). */
+void hip_require_device(const char *what);
+int hip_parse_only(void);
 
 #ifdef __cplusplus
 }

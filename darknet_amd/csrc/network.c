@@ -7,6 +7,10 @@
 #include <string.h>
 
 #include "host.h"
+#include "hip.h"
+
+/* written as a declaration so that it can stand before the function's own declarations */
+#define DN_NEED_DEVICE(what) const int need_device_ = (hip_require_device(what), 0); (void)need_device_
 
 /* src/network.c:177-186 */
 network *make_network(int n)
@@ -88,6 +92,7 @@ static int forward_conv_shortcut_pair(network net, int i)
 /* The layer loop of src/network.c:773-785 without the copies around it. */
 void forward_network_device(network *netp)
 {
+    DN_NEED_DEVICE("forward_network_device");
     network net = *netp;
     int i;
     net.train = 0;
@@ -112,6 +117,7 @@ void forward_network_device(network *netp)
  * milliseconds.  Events are created once per network size and reused. */
 float forward_network_profiled_kernels(network *netp, float *layer_ms, float *kernel_ms)
 {
+    DN_NEED_DEVICE("forward_network_profiled_kernels");
     static void **ev = 0, **ks = 0, **ke = 0;
     static int nev = 0;
     network net = *netp;
@@ -195,6 +201,7 @@ void network_pull_outputs(network *netp)
 /* src/network.c:762-788 */
 void forward_network_gpu(network *netp)
 {
+    DN_NEED_DEVICE("forward_network_gpu");
     network net = *netp;
     int i;
     hip_set_device(net.gpu_index);
@@ -214,6 +221,7 @@ void forward_network(network *net)
 /* src/network.c:497-508 */
 float *network_predict(network *net, float *input)
 {
+    DN_NEED_DEVICE("network_predict");
     network orig = *net;
     float *out;
     net->input = input;

@@ -93,6 +93,7 @@ __global__ void xnor_clear_pad_kernel(unsigned *wbits, int n, int npad, long row
 extern "C" void xnor_pack_weights_gpu(const float *weights, unsigned *wbits, float *wmean, int n, int c,
                                       int size)
 {
+    if (hip_parse_only()) return;
     const int npad = xnor_npad(n);
     const long rows = (long)size * size * ((c + 31) / 32);
     int *wpop = (int *)(wbits + rows * npad);

@@ -48,6 +48,13 @@ float  hip_compare(float *x_gpu, float *x, size_t n, char *s); /* cuda_compare  
 void   hip_pull_int_array(int *x_gpu, int *x, size_t n);/* (maxpool indexes; no reference twin) */
 void   hip_push_int_array(int *x_gpu, int *x, size_t n);/* (counters; no reference twin)        */
 void   hip_synchronize(void);                           /* hipStreamSynchronize on the stream  */
+/* Parse-only mode (no reference twin): after hip_set_parse_only(1) the cfg parser, the layer-table
+ * queries and the weights-file reader/writer work on host memory alone, on a machine with or
+ * without a GPU: nothing is allocated on or copied to a device (device pointers stay NULL).  It
+ * computes nothing: network_predict, forward_network* and every other call that needs the device
+ * print a message and exit(-1). */
+void   hip_set_parse_only(int on);
+int    hip_parse_only(void);
 void  *hip_get_stream(void);                            /* hipStream_t the library launches on */
 void   hip_set_stream(void *stream);                    /* 0 selects the null stream           */
 const char *hip_device_name(void);

