@@ -63,7 +63,8 @@ def test_bf16_mode_is_fp32_conv_of_rounded_operands(bf16, orc, b, c, h, w, n, si
     wt = synth.conv_weights(12, n, c // groups, size)
     bias, sc, mu, var = synth.bn_random(13, n)
     kw = dict(n=n, size=size, stride=stride, pad=pad, groups=groups)
-    assert bf16.conv_kernel_name(n, c, groups, size).decode().endswith(",2>" if size == 3 else ",1>")
+    name = bf16.conv_kernel_name(n, c, groups, size).decode()
+    assert name.count(",") == 5 and name.endswith(",2>" if size == 3 else ",1>")     # <BM,BN,WM,WN,mode,variant>
     got = run_conv(bf16, x, wt, bias, sc, mu, var, bn=1, act=act, **kw)
     want = orc.conv(round_bf16(x), round_bf16(wt), bias, sc, mu, var, batch_normalize=1, activation=act, **kw)
     assert norm_err(got, want) <= REL_TOL
@@ -73,13 +74,34 @@ def test_bf16_mode_is_fp32_conv_of_rounded_operands(bf16, orc, b, c, h, w, n, si
     assert 1e-5 < err < 2e-2          # really reduced precision, and no worse than bf16 rounding explains
 
 
+@pytest.mark.parametrize("b,c,h,w,n,size,stride,pad,groups,act,bn", __import__("test_gpu_conv").random_geometries(777, 32))
+def test_bf16_mode_random_geometries(bf16, orc, b, c, h, w, n, size, stride, pad, groups, act, bn):
+    """Whatever kernel a geometry lands on with the switch on - bf16 variants or untouched fp32
+    ones - the result is the fp32 convolution of operands rounded (or not) accordingly."""
+    x = synth.uniform(41, b * c * h * w).reshape(b, c, h, w)
+    wt = synth.conv_weights(42, n, c // groups, size)
+    bias, sc, mu, var = synth.bn_random(43, n)
+    if not bn:
+        sc = mu = var = None
+    kw = dict(n=n, size=size, stride=stride, pad=pad, groups=groups)
+    name = bf16.conv_kernel_name(n, c, groups, size).decode()
+    # a 3x3 layer packed tap-blocked but with padding other than 1 runs on the direct kernel
+    reduced = name.count(",") == 5 and not (size == 3 and pad != 1)    # <BM,BN,WM,WN,mode,variant>
+    got = run_conv(bf16, x, wt, bias, sc, mu, var, bn=bn, act=act, **kw)
+    if reduced:
+        want = orc.conv(round_bf16(x), round_bf16(wt), bias, sc, mu, var, batch_normalize=bn, activation=act, **kw)
+    else:
+        want = orc.conv(x, wt, bias, sc, mu, var, batch_normalize=bn, activation=act, **kw)
+    assert norm_err(got, want) <= REL_TOL, (name, reduced)
+
+
 def test_layers_on_other_kernels_stay_fp32(bf16, orc):
     """3 input channels -> reference-order kernel: the switch must not touch it."""
     b, c, h, w, n = 2, 3, 33, 35, 32
     x = synth.uniform(14, b * c * h * w).reshape(b, c, h, w)
     wt = synth.conv_weights(15, n, c, 3)
     bias, sc, mu, var = synth.bn_random(16, n)
-    assert bf16.conv_kernel_name(n, c, 1, 3).decode().endswith(",3>")
+    assert bf16.conv_kernel_name(n, c, 1, 3).decode().count(",") == 4
     got1 = run_conv(bf16, x, wt, bias, sc, mu, var, n=n, size=3, stride=1, pad=1, groups=1, bn=1, act="leaky")
     bf16.conv_set_precision(0)
     got0 = run_conv(bf16, x, wt, bias, sc, mu, var, n=n, size=3, stride=1, pad=1, groups=1, bn=1, act="leaky")

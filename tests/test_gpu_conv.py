@@ -96,6 +96,46 @@ def test_conv_exact_on_small_integers(dn, orc):
     assert np.array_equal(got, want)
 
 
+def random_geometries(seed, count):
+    """Seeded draw of legal layer geometries over every dispatch branch: 1x1 / 3x3 / 5x5 / 7x7,
+    strides 1-3, any padding up to the kernel size, channel counts on and off the 16-multiple that
+    selects the tap-blocked order, groups (equal, unequal, depthwise), filters around the tile
+    sizes, images smaller than the kernel window allows to skip."""
+    rng = np.random.default_rng(seed)
+    out = []
+    while len(out) < count:
+        size = int(rng.choice([1, 3, 3, 3, 5, 7]))
+        stride = 1 if size == 1 else int(rng.choice([1, 1, 2, 3]))
+        pad = 0 if size == 1 else int(rng.integers(0, size // 2 + 2))
+        groups = int(rng.choice([1, 1, 1, 2, 4, 8, 32]))
+        cg = int(rng.choice([1, 2, 3, 4, 8, 16, 20, 32, 48]))
+        fg = cg if (groups > 1 and rng.random() < 0.6) else int(rng.choice([1, 3, 8, 16, 31, 40, 65, 130, 260]))
+        c, n = cg * groups, fg * groups
+        if c > 512 or n > 600:
+            continue
+        h, w = int(rng.integers(1, 30)), int(rng.integers(1, 30))
+        if (h + 2 * pad - size) // stride + 1 <= 0 or (w + 2 * pad - size) // stride + 1 <= 0:
+            continue
+        b = int(rng.integers(1, 4))
+        act = str(rng.choice(["leaky", "linear", "relu", "logistic"]))
+        out.append((b, c, h, w, n, size, stride, pad, groups, act, int(rng.integers(0, 2))))
+    return out
+
+
+@pytest.mark.parametrize("b,c,h,w,n,size,stride,pad,groups,act,bn", random_geometries(20241, 48))
+def test_conv_random_geometries(dn, orc, b, c, h, w, n, size, stride, pad, groups, act, bn):
+    x = synth.uniform(31, b * c * h * w).reshape(b, c, h, w)
+    wt = synth.conv_weights(32, n, c // groups, size)
+    bias, sc, mu, var = synth.bn_random(33, n)
+    if not bn:
+        sc = mu = var = None
+    kw = dict(n=n, size=size, stride=stride, pad=pad, groups=groups)
+    want = orc.conv(x, wt, bias, sc, mu, var, batch_normalize=bn, activation=act, **kw)
+    got = run_conv(dn, x, wt, bias, sc, mu, var, bn=bn, act=act, **kw)
+    assert got.shape == want.shape
+    assert norm_err(got, want) <= REL_TOL, dn.conv_kernel_name(n, c, groups, size)
+
+
 def test_mfma_kernel_agrees_with_direct_kernel_and_unpacked_call(dn):
     b, c, h, w, n = 2, 64, 20, 20, 96
     x = synth.uniform(1, b * c * h * w).reshape(b, c, h, w)
