@@ -737,9 +737,11 @@ __global__ __launch_bounds__(DN_THREADS, (BM == 128 ? 3 : 2)) void conv_mfma_ker
 }
 
 /* Sums the K-slices of the tail tiles in slice order (deterministic) and applies the epilogue.
- * A thread owns four consecutive lanes' worth of one accumulator register: one 16-byte read per
- * slice, four consecutive output columns of one filter row.  Many small workgroups, because a
- * handful of tail tiles must still spread over the whole chip. */
+ * A thread owns four accumulator registers of one lane (r = 4g .. 4g+3): four consecutive pixels
+ * of one filter row (see conv_epilogue for the register map), so every read instruction of a
+ * wave covers 256 contiguous bytes of a slice and the result leaves as one 16-byte store.
+ * Threads whose filter or pixels lie outside the layer read nothing.  Many small workgroups,
+ * because a handful of tail tiles must still spread over the whole chip. */
 template <int BM, int BN, int WM, int WN>
 __global__ __launch_bounds__(DN_THREADS) void conv_reduce_kernel(mfma_args a)
 {
@@ -747,44 +749,61 @@ __global__ __launch_bounds__(DN_THREADS) void conv_reduce_kernel(mfma_args a)
     constexpr int WAVES_N = BN / WN;
     constexpr int GROUPS_PER_TILE = BM * BN / 4 / DN_THREADS; /* workgroups per tile */
     const int t = blockIdx.x / GROUPS_PER_TILE;
-    const int e = ((blockIdx.x - t * GROUPS_PER_TILE) * DN_THREADS + threadIdx.x) * 4; /* first element */
+    const int u = (blockIdx.x - t * GROUPS_PER_TILE) * DN_THREADS + threadIdx.x;
     const int lin = a.whole_tiles + t;
     const int m0 = (lin % a.tiles_m) * BM;
     const long n0 = (long)(lin / a.tiles_m) * BN;
-    /* e = ((wave*TM*TN + i*TN + j)*16 + r)*64 + lane; four consecutive e are four consecutive
-     * lanes = four consecutive FILTERS at one pixel (see conv_epilogue for the register map) */
-    const int lane = e & 63;
-    int q = e >> 6;
-    const int r = q & 15;
-    q >>= 4;
+    /* u = ((wave*TM*TN + i*TN + j)*4 + g)*64 + lane */
+    const int lane = u & 63;
+    const int g = (u >> 6) & 3;
+    int q = u >> 8;
     const int j = q % TN;
     q /= TN;
     const int i = q % TM;
     const int wave = q / TM;
-    const int mbase = m0 + (wave / WAVES_N) * WM + i * 32 + (lane & 31);
-    const long n = n0 + (wave % WAVES_N) * WN + j * 32 + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
-    float4 sum = make_float4(0.f, 0.f, 0.f, 0.f);
-    const float4 *ws = (const float4 *)(a.partial + (long)t * a.split * (BM * BN) + e);
+    const int m = m0 + (wave / WAVES_N) * WM + i * 32 + (lane & 31);
+    const long n = n0 + (wave % WAVES_N) * WN + j * 32 + 8 * g + 4 * (lane >> 5);
+    if (m >= a.M || n >= a.Ntotal) return;
+    /* element ((wave*TM*TN + i*TN + j)*16 + 4g + rr)*64 + lane of each slice */
+    const float *ws = a.partial + (long)t * a.split * (BM * BN) + ((u >> 8) * 16 + 4 * g) * 64 + lane;
+    float sum[4] = {0.f, 0.f, 0.f, 0.f};
     for (int sl = 0; sl < a.split; ++sl) {
-        const float4 v = ws[(long)sl * (BM * BN / 4)];
-        sum.x += v.x;
-        sum.y += v.y;
-        sum.z += v.z;
-        sum.w += v.w;
-    }
-    if (n >= a.Ntotal) return;
-    const int b = (int)((unsigned)n / (unsigned)a.P);
-    const int p = (int)n - b * a.P;
-    const float vals[4] = {sum.x, sum.y, sum.z, sum.w};
+        const float *p = ws + (long)sl * (BM * BN);
 #pragma unroll
-    for (int c = 0; c < 4; ++c) {
-        const int m = mbase + c;
-        if (m >= a.M) break;
-        const conv_row_t row = conv_row(a, m);
-        const long off = ((long)b * a.M + m) * a.P + p;
-        const float y = conv_tail_one(vals[c], row, conv_f2{a.slope_hi, a.slope_lo});
-        a.out[off] = y;
-        if (a.sum) a.sum[off] = conv_residual_one(a, y, a.add[off]);
+        for (int rr = 0; rr < 4; ++rr) sum[rr] += p[rr * 64];
+    }
+    const int b = (int)((unsigned)n / (unsigned)a.P);
+    const int px = (int)n - b * a.P;
+    const conv_row_t row = conv_row(a, m);
+    const long off = ((long)b * a.M + m) * a.P + px;
+    float y[4];
+#pragma unroll
+    for (int rr = 0; rr < 4; ++rr) y[rr] = conv_tail_one(sum[rr], row, conv_f2{a.slope_hi, a.slope_lo});
+    if (px + 3 < a.P) { /* the four pixels lie in one image (then n + 3 < Ntotal too) */
+        *(float4u *)(a.out + off) = (float4u){y[0], y[1], y[2], y[3]};
+        if (a.sum) {
+            const float4u r4 = *(const float4u *)(a.add + off);
+            float4u s4;
+            s4.x = conv_residual_one(a, y[0], r4.x);
+            s4.y = conv_residual_one(a, y[1], r4.y);
+            s4.z = conv_residual_one(a, y[2], r4.z);
+            s4.w = conv_residual_one(a, y[3], r4.w);
+            *(float4u *)(a.sum + off) = s4;
+        }
+    } else { /* image boundary or end of N inside the four: element by element */
+        int pc = px;
+        long offc = off;
+        const long wrap = (long)(a.M - 1) * a.P; /* what the offset gains when the pixel index wraps */
+        for (int rr = 0; rr < 4 && n + rr < a.Ntotal; ++rr) {
+            while (pc >= a.P) {
+                pc -= a.P;
+                offc += wrap;
+            }
+            a.out[offc] = y[rr];
+            if (a.sum) a.sum[offc] = conv_residual_one(a, y[rr], a.add[offc]);
+            ++pc;
+            ++offc;
+        }
     }
 }
 
