@@ -49,6 +49,15 @@ __global__ __launch_bounds__(DN_DIRECT_BLOCK) void conv_direct_kernel(direct_arg
     const int ix0 = ox * a.stride - a.pad;
     const float *img = a.in + ((long)b * a.c + (long)g * cg) * a.h * a.wd;
 
+    /* batch-norm constants of the workgroup's filters, once per workgroup (a double square root
+     * and division each); visible to all threads after the first barrier of the K loop */
+    __shared__ dn_bn_row rows[DN_FPB];
+    if ((int)threadIdx.x < nf) {
+        const int f = f0 + threadIdx.x;
+        rows[threadIdx.x] = dn_bn_make(a.bn, a.biases[f], a.bn ? a.scales[f] : 1.f, a.bn ? a.mean[f] : 0.f,
+                                       a.bn ? a.var[f] : 1.f);
+    }
+
     float acc[DN_FPB];
 #pragma unroll
     for (int j = 0; j < DN_FPB; ++j) acc[j] = 0.f;
@@ -82,9 +91,7 @@ __global__ __launch_bounds__(DN_DIRECT_BLOCK) void conv_direct_kernel(direct_arg
     for (int j = 0; j < DN_FPB; ++j) {
         if (j >= nf) continue;
         const int f = f0 + j;
-        const dn_bn_row row = dn_bn_make(a.bn, a.biases[f], a.bn ? a.scales[f] : 1.f,
-                                         a.bn ? a.mean[f] : 0.f, a.bn ? a.var[f] : 1.f);
-        const float y = dn_activate(dn_bn_apply(acc[j], row, a.bn), a.act);
+        const float y = dn_activate(dn_bn_apply(acc[j], rows[j], a.bn), a.act);
         a.out[((long)b * a.n + f) * P + p] = y;
     }
 }

@@ -147,6 +147,17 @@ __global__ __launch_bounds__(XN_BLOCK) void xnor_conv_kernel(const unsigned *__r
     const int ss = a.size * a.size;
     const int f0 = blockIdx.y * XN_FPB;
     const int P = a.oh * a.ow;
+    /* the batch-norm constants of the workgroup's filters (a double square root and division
+     * each) are the same for every pixel: computed once, by one lane per filter */
+    __shared__ dn_bn_row rows[XN_FPB];
+    __shared__ float wmeans[XN_FPB];
+    if (threadIdx.x < XN_FPB && f0 + (int)threadIdx.x < a.n) {
+        const int f = f0 + threadIdx.x;
+        rows[threadIdx.x] = dn_bn_make(a.bn, a.biases[f], a.bn ? a.scales[f] : 1.f, a.bn ? a.mean[f] : 0.f,
+                                       a.bn ? a.var[f] : 1.f);
+        wmeans[threadIdx.x] = a.wmean[f];
+    }
+    __syncthreads();
     const long col = blockIdx.x * (long)XN_BLOCK + threadIdx.x;
     const bool col_ok = col < a.ntotal;
     const long cc = col_ok ? col : 0;
@@ -186,10 +197,8 @@ __global__ __launch_bounds__(XN_BLOCK) void xnor_conv_kernel(const unsigned *__r
         int m = mism[j];
         for (unsigned o = outside; o; o &= o - 1) m -= wpop[f * ss + (__ffs(o) - 1)];
         const int dot = taps_inside * a.c - 2 * m;
-        const float acc = __fmul_rn(a.wmean[f], (float)dot);
-        const dn_bn_row r = dn_bn_make(a.bn, a.biases[f], a.bn ? a.scales[f] : 1.f, a.bn ? a.mean[f] : 0.f,
-                                       a.bn ? a.var[f] : 1.f);
-        a.out[((long)b * a.n + f) * P + p] = dn_activate(dn_bn_apply(acc, r, a.bn), a.act);
+        const float acc = __fmul_rn(wmeans[j], (float)dot);
+        a.out[((long)b * a.n + f) * P + p] = dn_activate(dn_bn_apply(acc, rows[j], a.bn), a.act);
     }
 }
 
