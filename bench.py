@@ -168,7 +168,7 @@ def main():
     ap.add_argument("--workload", default="yolov3-416", choices=sorted(WORKLOADS))
     ap.add_argument("--batch", type=int, default=64)
     ap.add_argument("--per-layer", default="")
-    ap.add_argument("--precision", default="fp32", choices=["fp32", "bf16"],
+    ap.add_argument("--precision", default="fp32", choices=["fp32", "bf16", "bf16x3"],
                     help="bf16: the tap-blocked MFMA kernels round their operands to bf16 (opt-in, not the "
                          "headline configuration; its error against fp32 is reported by the tests)")
     ap.add_argument("--no-cpu", action="store_true")
@@ -188,8 +188,11 @@ def main():
     L = api._lib.load()
     dev = L.hip_device_name().decode()
     log("device:", dev)
-    L.conv_set_precision(1 if args.precision == "bf16" else 0)
-    peak = PEAK_BF16_MFMA_TFLOPS if args.precision == "bf16" else PEAK_FP32_MFMA_TFLOPS
+    L.conv_set_precision({"fp32": 0, "bf16": 1, "bf16x3": 2}[args.precision])
+    # bf16x3 issues six bf16 MFMAs per fp32-equivalent multiply-add: its algorithmic FLOPs are priced
+    # against a sixth of the bf16 peak
+    peak = {"fp32": PEAK_FP32_MFMA_TFLOPS, "bf16": PEAK_BF16_MFMA_TFLOPS,
+            "bf16x3": PEAK_BF16_MFMA_TFLOPS / 6}[args.precision]
     net = api.Network(cfg_text=text)
     fill_params(net.set_conv, net.layers)
     x = synth.uniform01(7, net.inputs * net.batch)
@@ -312,7 +315,8 @@ def main():
         "metric": "images/sec", "value": round(value, 2), "unit": "images/s", "n_gpus": 1,
         "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(ms_per_step, 4),
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
-        "dtype": "f32" if args.precision == "fp32" else "bf16 operands, f32 accumulate and storage",
+        "dtype": {"fp32": "f32", "bf16": "bf16 operands, f32 accumulate and storage",
+                  "bf16x3": "f32 emulated with three bf16 pieces per operand, f32 accumulate and storage"}[args.precision],
         "data": "synthetic",
         "config": {"workload": f"{args.workload} forward, batch {args.batch}, {args.precision}, input uniform[0,1), "
                                f"weights uniform(-1,1)*sqrt(2/(k*k*c)), BN mean 0 var 1 scale 1",

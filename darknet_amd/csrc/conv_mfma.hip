@@ -70,6 +70,7 @@ struct mfma_args {
     const float *wp; /* packed weights */
     const void *wp16; /* the bf16 copy of the packed weights (bf16-operand mode) */
     unsigned wp16_records;
+    unsigned plane16; /* bytes of one bf16 copy; the mid and lo copies of the three-piece mode follow the first */
     int Mpad16;
     const void *in16; /* staged bf16 copy of the input, [image][C/8][H*W][8] (bf16 mode, 3x3 layers) */
     unsigned in16_records;
@@ -281,9 +282,14 @@ __device__ __forceinline__ void conv_epilogue(const mfma_args &a, f32x16 (&acc)[
 /* BF16: 0 = fp32 operands; 1 = bf16 weights from their packed copy, fp32 activation tiles rounded
  * on the way into the MFMA (1x1 layers: the input is read once, straight from the fp32 tensor);
  * 2 = both operands bf16 in LDS, the activations gathered from a staged bf16 copy of the input
- * (3x3 layers, which read every input element nine times). */
+ * (3x3 layers, which read every input element nine times);
+ * 3 = fp32 emulated on the bf16 matrix cores: every operand is the exact sum of three bf16 pieces
+ * (x = hi + mid + lo, each the nearest-even rounding of what the previous ones left), the weights
+ * pre-split into three packed copies, the activations split in registers from the fp32 LDS tile,
+ * and a product is the six piece-products down to 2^-16 relative (hi*hi, hi*mid, mid*hi, hi*lo,
+ * lo*hi, mid*mid; the three dropped ones are below 2^-24), accumulated in fp32. */
 template <int BM, int BN, int WM, int WN, int MODE, int BF16 = 0>
-__global__ __launch_bounds__(DN_THREADS, (BM == 128 ? 3 : 2)) void conv_mfma_kernel(mfma_args a)
+__global__ __launch_bounds__(DN_THREADS, ((BM == 128 && BF16 != 3) ? 3 : 2)) void conv_mfma_kernel(mfma_args a)
 {
     constexpr int TM = WM / 32, TN = WN / 32;
     constexpr int WAVES_N = BN / WN;
@@ -296,8 +302,10 @@ __global__ __launch_bounds__(DN_THREADS, (BM == 128 ? 3 : 2)) void conv_mfma_ker
      * wait (vmcnt) for direct-to-LDS loads it cannot prove disjoint from it, and it can only
      * prove that for distinct objects. */
     constexpr bool V3 = BF16 == 2;
+    constexpr bool X3 = BF16 == 3;                 /* three-piece emulation: fp32-style pipeline */
+    constexpr bool BFP = BF16 == 1 || BF16 == 2;    /* the deep-pipelined bf16 variants */
     static_assert(!V3 || (TAPB && KS == 3), "the staged-input variant serves the tap-blocked 3x3 layers");
-    constexpr int A_FLOATS = BF16 ? BM * DN_BK / 2 : BM * DN_BK; /* bf16 rows are 32 bytes */
+    constexpr int A_FLOATS = X3 ? 3 * BM * DN_BK / 2 : BF16 ? BM * DN_BK / 2 : BM * DN_BK; /* bf16 rows are 32 bytes */
     constexpr int B_FLOATS = V3 ? BN * DN_BK / 2 : BN * DN_BK;
     __shared__ __attribute__((aligned(16))) float As0[V3 ? 4 : A_FLOATS], As1[V3 ? 4 : A_FLOATS];
     __shared__ __attribute__((aligned(16))) float Bs0[V3 ? 4 : B_FLOATS], Bs1[V3 ? 4 : B_FLOATS];
@@ -435,21 +443,28 @@ __global__ __launch_bounds__(DN_THREADS, (BM == 128 ? 3 : 2)) void conv_mfma_ker
              * rows when BM == 32). */
             constexpr int WL = BM / 32;                  /* wave-loads per chunk: 8, 4, 2, 1 */
             constexpr int PER_WAVE = (WL + 3) / 4;
+            constexpr int PLANES = X3 ? 3 : 1;           /* hi (, mid, lo) copies, a.plane16 bytes apart */
 #pragma unroll
-            for (int i = 0; i < PER_WAVE; ++i) {
-                const int wl = wave * PER_WAVE + i;
-                if (WL >= 4 || wl < WL) {
-                    if (BM >= 64) {
-                        constexpr int RB = BM / 64;
-                        const int h = wl / RB, rb = wl - h * RB;
-                        const unsigned soff = (unsigned)((((long)kc * 2 + h) * a.Mpad16 + m0 + rb * 64) * 16);
-                        __builtin_amdgcn_raw_ptr_buffer_load_lds(w_rsrc, (lds_ptr)&A_BUF(buf)[(h * BM + rb * 64) * 4], 16,
-                                                                 lane * 16, soff, 0, 0);
-                    } else {
-                        const unsigned voff = (unsigned)((((long)(lane >> 5) * a.Mpad16) + (lane & 31)) * 16);
-                        const unsigned soff = a.grouped ? (unsigned)(((long)(tile_m * a.KCH + kc) * 2 * 32) * 16)
-                                                        : (unsigned)(((long)kc * 2 * a.Mpad16 + m0) * 16);
-                        __builtin_amdgcn_raw_ptr_buffer_load_lds(w_rsrc, (lds_ptr)&A_BUF(buf)[0], 16, voff, soff, 0, 0);
+            for (int pl = 0; pl < PLANES; ++pl) {
+#pragma unroll
+                for (int i = 0; i < PER_WAVE; ++i) {
+                    const int wl = wave * PER_WAVE + i;
+                    if (WL >= 4 || wl < WL) {
+                        if (BM >= 64) {
+                            constexpr int RB = BM / 64;
+                            const int h = wl / RB, rb = wl - h * RB;
+                            const unsigned soff =
+                                (unsigned)((((long)kc * 2 + h) * a.Mpad16 + m0 + rb * 64) * 16) + pl * a.plane16;
+                            __builtin_amdgcn_raw_ptr_buffer_load_lds(
+                                w_rsrc, (lds_ptr)&A_BUF(buf)[pl * BM * 8 + (h * BM + rb * 64) * 4], 16, lane * 16, soff, 0, 0);
+                        } else {
+                            const unsigned voff = (unsigned)((((long)(lane >> 5) * a.Mpad16) + (lane & 31)) * 16);
+                            const unsigned soff = (a.grouped ? (unsigned)(((long)(tile_m * a.KCH + kc) * 2 * 32) * 16)
+                                                             : (unsigned)(((long)kc * 2 * a.Mpad16 + m0) * 16)) +
+                                                  pl * a.plane16;
+                            __builtin_amdgcn_raw_ptr_buffer_load_lds(w_rsrc, (lds_ptr)&A_BUF(buf)[pl * BM * 8], 16, voff, soff,
+                                                                     0, 0);
+                        }
                     }
                 }
             }
@@ -551,13 +566,14 @@ __global__ __launch_bounds__(DN_THREADS, (BM == 128 ? 3 : 2)) void conv_mfma_ker
     /* loads one wave issues per chunk, for the s_waitcnt immediates of the bf16 pipeline (the A
      * loads are left out where not every wave issues them: those waves wait for one load more
      * than they must) */
-    constexpr int LPC = (BF16 && BM >= 128 ? BM / 128 : 0) + (V3 ? NBW : 4 * NG_PER_WAVE);
+    constexpr int LPC = (BFP && BM >= 128 ? BM / 128 : 0) + (V3 ? NBW : 4 * NG_PER_WAVE);
     /* s_waitcnt on vmcnt alone: simm16 = vmcnt[3:0] | expcnt(7) << 4 | lgkmcnt(15) << 8 | vmcnt[5:4] << 14 */
 #define DN_WAIT_VM(n) __builtin_amdgcn_s_waitcnt(((n) & 15) | (7 << 4) | (15 << 8) | (((n) >> 4) << 14))
     static_assert(2 * LPC < 64, "vmcnt is a 6-bit counter");
 
     float4 av[2][TM], bv[BF16 == 1 ? 2 : 1][2][TN]; /* MFMA operands of a chunk: [k half][32-row block] */
-    bf16x8 a8[2][BF16 ? TM : 1];             /* bf16 modes: a row's eight k of this lane's half, two register sets */
+    bf16x8 a8[2][BFP ? TM : 1];              /* bf16 modes: a row's eight k of this lane's half, two register sets */
+    bf16x8 a3[3][X3 ? TM : 1];               /* three-piece mode: hi, mid, lo of the same */
     bf16x8 b8s[2][V3 ? TN : 1];              /* staged input: a column's eight k likewise */
 
     auto read_operands = [&](int buf, int r) {
@@ -571,13 +587,23 @@ __global__ __launch_bounds__(DN_THREADS, (BM == 128 ? 3 : 2)) void conv_mfma_ker
             if constexpr (!V3) {
 #pragma unroll
                 for (int j = 0; j < TN; ++j)
-                    bv[BF16 == 1 ? r : 0][hb][j] = *(const float4 *)&B_BUF(buf)[((hb * 2 + kh) * BN + wn0 + j * 32 + li) * 4];
+                    /* which two slots hold this lane's eight k: (kh, 2 + kh) as the fp32 layout pairs them,
+                     * or (2kh, 2kh + 1) where the bf16 copy of a 3x3 layer is packed eight channels per half */
+                    bv[BF16 == 1 ? r : 0][hb][j] =
+                        *(const float4 *)&B_BUF(buf)[(((X3 && KS == 3) ? 2 * kh + hb : hb * 2 + kh) * BN + wn0 + j * 32 + li) * 4];
             }
         }
-        if constexpr (BF16) {
+        if constexpr (BFP) {
 #pragma unroll
             for (int i = 0; i < TM; ++i)
                 a8[r][i] = *(const bf16x8 *)&A_BUF(buf)[(kh * BM + wm0 + i * 32 + li) * 4];
+        }
+        if constexpr (X3) {
+#pragma unroll
+            for (int pl = 0; pl < 3; ++pl)
+#pragma unroll
+                for (int i = 0; i < TM; ++i)
+                    a3[pl][i] = *(const bf16x8 *)&A_BUF(buf)[pl * BM * 8 + (kh * BM + wm0 + i * 32 + li) * 4];
         }
         if constexpr (V3) {
 #pragma unroll
@@ -586,7 +612,7 @@ __global__ __launch_bounds__(DN_THREADS, (BM == 128 ? 3 : 2)) void conv_mfma_ker
         }
     };
 
-    if constexpr (BF16) {
+    if constexpr (BFP) {
         /* chunks 0..2 requested; chunks 0 and 1 must have landed before the first step */
         const int nch = kc_end - kc_begin;
         load_chunk(kc_begin, 0);
@@ -627,7 +653,32 @@ __global__ __launch_bounds__(DN_THREADS, (BM == 128 ? 3 : 2)) void conv_mfma_ker
      * contracts all 16 k of the chunk; products and sums stay fp32, so does everything after the
      * accumulators. */
     auto mfma_chunk = [&](int r) {
-        if constexpr (BF16) {
+        if constexpr (X3) {
+            /* x = hi + mid + lo: hi = bf16(x), mid = bf16(x - hi), lo = bf16(x - hi - mid); both
+             * subtractions are exact in fp32.  Small terms first. */
+            bf16x8 bh[TN], bm[TN], bl[TN];
+#pragma unroll
+            for (int j = 0; j < TN; ++j) {
+                const float4 q0 = bv[0][0][j], q1 = bv[0][1][j];
+                const f32x8 f = {q0.x, q0.y, q0.z, q0.w, q1.x, q1.y, q1.z, q1.w};
+                bh[j] = __builtin_convertvector(f, bf16x8);
+                const f32x8 r1 = f - __builtin_convertvector(bh[j], f32x8);
+                bm[j] = __builtin_convertvector(r1, bf16x8);
+                const f32x8 r2 = r1 - __builtin_convertvector(bm[j], f32x8);
+                bl[j] = __builtin_convertvector(r2, bf16x8);
+            }
+            /* term by term over all accumulators, so that consecutive MFMAs are independent */
+#define DN_X3_TERM(BOP, APL)                                                                        \
+    _Pragma("unroll") for (int i = 0; i < TM; ++i) _Pragma("unroll") for (int j = 0; j < TN; ++j)  \
+        acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(BOP[j], a3[APL][i], acc[i][j], 0, 0, 0)
+            DN_X3_TERM(bl, 0); /* lo  * hi  */
+            DN_X3_TERM(bh, 2); /* hi  * lo  */
+            DN_X3_TERM(bm, 1); /* mid * mid */
+            DN_X3_TERM(bm, 0); /* mid * hi  */
+            DN_X3_TERM(bh, 1); /* hi  * mid */
+            DN_X3_TERM(bh, 0); /* hi  * hi  */
+#undef DN_X3_TERM
+        } else if constexpr (BF16) {
             bf16x8 b8[TN];
 #pragma unroll
             for (int j = 0; j < TN; ++j) {
@@ -670,7 +721,7 @@ __global__ __launch_bounds__(DN_THREADS, (BM == 128 ? 3 : 2)) void conv_mfma_ker
         mfma_chunk(0);
     };
 
-    if constexpr (BF16) {
+    if constexpr (BFP) {
         /* Four LDS stages and two register sets.  A bf16 chunk is 8 (or 4, 2) MFMAs, far shorter
          * than a trip to memory or even to LDS, so a step overlaps three things: the LDS reads of
          * chunk kc+1 into the other register set, the request for chunk kc+3, and the MFMAs of
@@ -729,7 +780,7 @@ __global__ __launch_bounds__(DN_THREADS, (BM == 128 ? 3 : 2)) void conv_mfma_ker
     } else {
         __syncthreads(); /* every wave has read its last operands: the LDS buffers are free */
         float *E = V3 ? S_BUF(wave)
-                   : BM >= 128 ? (BF16 ? (wave == 0 ? Bs2 : wave == 1 ? Bs3 : wave == 2 ? Bs0 : Bs1)
+                   : BM >= 128 ? (BFP ? (wave == 0 ? Bs2 : wave == 1 ? Bs3 : wave == 2 ? Bs0 : Bs1)
                                        : (wave == 0 ? As0 : wave == 1 ? As1 : wave == 2 ? Bs0 : Bs1))
                                : (wave < 2 ? Bs0 : Bs1) + (wave & 1) * 2048;
         conv_epilogue<TM, TN>(a, acc, E, m0, n0, wm0, wn0, lane);
@@ -908,15 +959,31 @@ static size_t conv_packed_bf16_floats(int n, int c, int groups, int size)
     return (size_t)(kch * conv_mpad16(n) * DN_BK / 2);
 }
 
+/* three bf16 copies follow the fp32 part: hi (the bf16 mode's operand), then mid and lo, which the
+ * three-piece emulation adds */
+#define DN_BF16_PLANES 3
+
 extern "C" size_t conv_packed_floats(int n, int c, int groups, int size)
 {
-    return conv_packed_f32_floats(n, c, groups, size) + conv_packed_bf16_floats(n, c, groups, size);
+    return conv_packed_f32_floats(n, c, groups, size) + DN_BF16_PLANES * conv_packed_bf16_floats(n, c, groups, size);
+}
+
+/* piece `plane` of w = hi + mid + lo, each the nearest-even bf16 of what the previous ones left */
+__device__ __forceinline__ __bf16 conv_bf16_piece(float w, int plane)
+{
+    __bf16 p = (__bf16)w;
+    for (int i = 0; i < plane; ++i) {
+        w -= (float)p; /* exact */
+        p = (__bf16)w;
+    }
+    return p;
 }
 
 /* bf16 copy of a tap-blocked layer: element ((chunk*2 + h)*Mpad16 + m)*8 + p is the weight that the
  * fp32 layout keeps at slot (p < 4 ? h : 2 + h), position p % 4 of the same chunk and row (1x1
  * layers) or at position 8*h + p of the chunk (3x3 layers), rounded to nearest even. */
-__global__ void pack_weights_bf16_kernel(const float *w, __bf16 *packed, int M, int K, int Mpad16, long total, int taps)
+__global__ void pack_weights_bf16_kernel(const float *w, __bf16 *packed, int M, int K, int Mpad16, long total, int taps,
+                                         int plane)
 {
     for (long i = blockIdx.x * (long)blockDim.x + threadIdx.x; i < total; i += (long)gridDim.x * blockDim.x) {
         const int pp = (int)(i & 7);
@@ -930,12 +997,12 @@ __global__ void pack_weights_bf16_kernel(const float *w, __bf16 *packed, int M, 
         const int kk = taps == 1 ? (pp < 4 ? h : 2 + h) * 4 + (pp & 3) : 8 * h + pp;
         const int cb = kc / taps, tap = kc - cb * taps;
         const int k = (cb * DN_BK + kk) * taps + tap;
-        packed[i] = (__bf16)((m < M && k < K) ? w[(long)m * K + k] : 0.f);
+        packed[i] = conv_bf16_piece((m < M && k < K) ? w[(long)m * K + k] : 0.f, plane);
     }
 }
 
 /* bf16 copy of a grouped layer: ((tile*KCH + chunk)*2 + h)*32 + r rows of 8, as above */
-__global__ void pack_grouped_bf16_kernel(const float *w, __bf16 *packed, int cg, int taps, long total)
+__global__ void pack_grouped_bf16_kernel(const float *w, __bf16 *packed, int cg, int taps, long total, int plane)
 {
     const int kch = 2 * taps;
     for (long i = blockIdx.x * (long)blockDim.x + threadIdx.x; i < total; i += (long)gridDim.x * blockDim.x) {
@@ -951,7 +1018,7 @@ __global__ void pack_grouped_bf16_kernel(const float *w, __bf16 *packed, int cg,
         const int ch = cb * DN_BK + (taps == 1 ? (pp < 4 ? h : 2 + h) * 4 + (pp & 3) : 8 * h + pp);
         const int f = tile * 32 + r;
         const bool same_group = (r / cg) == (ch / cg);
-        packed[i] = (__bf16)(same_group ? w[((long)f * cg + (ch % cg)) * taps + tap] : 0.f);
+        packed[i] = conv_bf16_piece(same_group ? w[((long)f * cg + (ch % cg)) * taps + tap] : 0.f, plane);
     }
 }
 
@@ -971,8 +1038,9 @@ extern "C" void conv_pack_weights_gpu(const float *weights, float *packed, int n
     if (gt) {
         hipLaunchKernelGGL(pack_grouped_kernel, dim3(pack_blocks(total)), dim3(256), 0, dn_stream(), weights, packed,
                            c / groups, gt, (long)total);
-        hipLaunchKernelGGL(pack_grouped_bf16_kernel, dim3(pack_blocks(total16)), dim3(256), 0, dn_stream(), weights,
-                           packed16, c / groups, gt, (long)total16);
+        for (int pl = 0; pl < DN_BF16_PLANES; ++pl)
+            hipLaunchKernelGGL(pack_grouped_bf16_kernel, dim3(pack_blocks(total16)), dim3(256), 0, dn_stream(), weights,
+                               packed16 + (size_t)pl * total16, c / groups, gt, (long)total16, pl);
         dn_check_launch("conv_pack_weights_gpu");
         return;
     }
@@ -981,9 +1049,9 @@ extern "C" void conv_pack_weights_gpu(const float *weights, float *packed, int n
     const int taps = tap_blocked_taps(c, groups, size);
     hipLaunchKernelGGL(pack_weights_kernel, dim3(pack_blocks(total)), dim3(256), 0, dn_stream(), weights, packed, n,
                        K, mpad, (long)total, taps);
-    if (total16)
+    for (int pl = 0; total16 && pl < DN_BF16_PLANES; ++pl)
         hipLaunchKernelGGL(pack_weights_bf16_kernel, dim3(pack_blocks(total16)), dim3(256), 0, dn_stream(), weights,
-                           packed16, n, K, conv_mpad16(n), (long)total16, taps);
+                           packed16 + (size_t)pl * total16, n, K, conv_mpad16(n), (long)total16, taps, pl);
     dn_check_launch("conv_pack_weights_gpu");
 }
 
@@ -1023,11 +1091,14 @@ static int g_algo = 0;
 extern "C" void conv_set_algo(int algo) { g_algo = algo; }
 
 /* 0 = fp32 operands (default, the reference's arithmetic); 1 = the tap-blocked MFMA kernels round
- * both operands to bf16 and accumulate in fp32 (layers on other kernels stay fp32). */
+ * both operands to bf16 and accumulate in fp32; 2 = they split both operands into three bf16 pieces
+ * and sum six piece-products in fp32 (fp32-level accuracy on the bf16 matrix cores).  Layers on
+ * other kernels stay fp32. */
 static int g_precision = 0;
 extern "C" void conv_set_precision(int precision)
 {
-    if (precision != 0 && precision != 1) dn_fatal("conv_set_precision: 0 (fp32) or 1 (bf16 operands)");
+    if (precision < 0 || precision > 2)
+        dn_fatal("conv_set_precision: 0 (fp32), 1 (bf16 operands) or 2 (fp32 emulated with three bf16 pieces)");
     g_precision = precision;
 }
 extern "C" int conv_get_precision(void) { return g_precision; }
@@ -1045,9 +1116,10 @@ extern "C" const char *conv_kernel_name(int n, int c, int groups, int size)
     }
     if (mode < 0) return "conv_direct_kernel";
     const int bf16 = g_precision == 1 && mode >= 10;
+    const int x3 = g_precision == 2 && mode >= 10;
     if (bf16 && bm == 128 && n > 128) bm = 256;
     snprintf(name, sizeof name, "conv_mfma_kernel<%d,%d,%d,64,%d%s>", bm, bm >= 128 ? 128 : 256,
-             bm == 32 ? 32 : bm == 256 ? 128 : 64, mode, !bf16 ? "" : mode == 13 ? ",2" : ",1");
+             bm == 32 ? 32 : bm == 256 ? 128 : 64, mode, x3 ? ",3" : !bf16 ? "" : mode == 13 ? ",2" : ",1");
     return name;
 }
 
@@ -1109,7 +1181,8 @@ static void launch_tile(const mfma_args &a0, int mode)
     int split = 1;
     /* a bf16 chunk takes a small fraction of an fp32 chunk's time; the fixed costs do not shrink */
     const int bf16 = g_precision == 1 && mode >= 10;
-    const long whole = plan_split(total, a.KCH, g_cus, &split, bf16 ? 6.0 : 1.0);
+    const int x3 = g_precision == 2 && mode >= 10;
+    const long whole = plan_split(total, a.KCH, g_cus, &split, bf16 ? 6.0 : x3 ? 2.0 : 1.0);
     const long tail = total - whole;
     a.whole_tiles = (int)whole;
     a.split = split;
@@ -1128,16 +1201,24 @@ static void launch_tile(const mfma_args &a0, int mode)
     if (BM > 128 && !bf16) dn_fatal("conv dispatch: the 256-row tile is only built for the bf16-operand mode");
     switch (mode) {
     case 11:
-        if (bf16)
+        if (bf16) {
             DN_LAUNCH((conv_mfma_kernel<BM, BN, WM, WN, 11, 1>));
-        else if constexpr (BM <= 128)
-            DN_LAUNCH((conv_mfma_kernel<BM, BN, WM, WN, 11>));
+        } else if constexpr (BM <= 128) {
+            if (x3)
+                DN_LAUNCH((conv_mfma_kernel<BM, BN, WM, WN, 11, 3>));
+            else
+                DN_LAUNCH((conv_mfma_kernel<BM, BN, WM, WN, 11>));
+        }
         break;
     case 13:
-        if (bf16)
+        if (bf16) {
             DN_LAUNCH((conv_mfma_kernel<BM, BN, WM, WN, 13, 2>));
-        else if constexpr (BM <= 128)
-            DN_LAUNCH((conv_mfma_kernel<BM, BN, WM, WN, 13>));
+        } else if constexpr (BM <= 128) {
+            if (x3)
+                DN_LAUNCH((conv_mfma_kernel<BM, BN, WM, WN, 13, 3>));
+            else
+                DN_LAUNCH((conv_mfma_kernel<BM, BN, WM, WN, 13>));
+        }
         break;
     default:
         if constexpr (BM <= 128) {
@@ -1277,7 +1358,8 @@ static void conv_forward(const float *input, const float *weights, const float *
     a.in_records = (unsigned)((long)batch * c * h * w * 4 + (long)(w + 1) * 4);
     a.wp_records = (unsigned)(conv_packed_f32_floats(n, c, groups, size) * 4);
     a.wp16 = packed + conv_packed_f32_floats(n, c, groups, size);
-    a.wp16_records = (unsigned)(conv_packed_bf16_floats(n, c, groups, size) * 4);
+    a.plane16 = (unsigned)(conv_packed_bf16_floats(n, c, groups, size) * 4);
+    a.wp16_records = DN_BF16_PLANES * a.plane16;
     a.Mpad16 = a.grouped ? 32 : conv_mpad16(n);
     a.in16 = 0;
     a.in16_records = 0;

@@ -74,11 +74,11 @@ def main():
     ap.add_argument("--sweep", action="store_true")
     ap.add_argument("--algo", type=int, default=0)
     ap.add_argument("--data", default="random", choices=["random", "zeros"])
-    ap.add_argument("--precision", default="fp32", choices=["fp32", "bf16"])
+    ap.add_argument("--precision", default="fp32", choices=["fp32", "bf16", "bf16x3"])
     a = ap.parse_args()
     api.set_gpu(0)
     _lib.load().conv_set_algo(a.algo)
-    _lib.load().conv_set_precision(1 if a.precision == "bf16" else 0)
+    _lib.load().conv_set_precision({"fp32": 0, "bf16": 1, "bf16x3": 2}[a.precision])
     if a.sweep:
         for name, (c, h, w, n, size, stride) in cfgs.SWEEP.items():
             for batch in (1, 64):

@@ -169,10 +169,16 @@ int conv_profile_pending(void);
 void conv_set_algo(int algo);
 
 /* Operand precision of the tap-blocked MFMA convolution kernels (channels a multiple of 16, 1x1 or
- * 3x3 pad 1; grouped 32-filter tiles): 0 = fp32 (default; the reference's arithmetic, the parity
- * bar applies), 1 = both operands rounded to bf16 (nearest even) inside the kernel, products and
- * sums in fp32, epilogue unchanged.  Layers served by other kernels (first layer, direct, xnor)
- * stay fp32.  An opt-in speed/precision trade with no counterpart in the reference. */
+ * 3x3 pad 1; grouped 32-filter tiles):
+ *   0  fp32 (default; the reference's arithmetic on v_mfma_f32_32x32x2_f32);
+ *   1  both operands rounded to bf16 (nearest even) inside the kernel, products and sums in fp32,
+ *      epilogue unchanged: an opt-in speed/precision trade outside the parity bar;
+ *   2  fp32 emulated on the bf16 matrix cores: each operand is the exact sum of three bf16 pieces,
+ *      six piece-products per multiply-add summed in fp32 (the three dropped ones are below 2^-24
+ *      relative).  Meets the fp32 parity bar; measured closer to the fp64 convolution than the
+ *      fp32 CPU path is.
+ * Layers served by other kernels (first layer, direct, xnor) stay fp32.  No counterpart in the
+ * reference. */
 void conv_set_precision(int precision);
 int conv_get_precision(void);
 

@@ -95,6 +95,55 @@ def test_bf16_mode_random_geometries(bf16, orc, b, c, h, w, n, size, stride, pad
     assert norm_err(got, want) <= REL_TOL, (name, reduced)
 
 
+@pytest.fixture
+def bf16x3(dn):
+    dn.conv_set_precision(2)
+    yield dn
+    dn.conv_set_precision(0)
+
+
+@pytest.mark.parametrize("b,c,h,w,n,size,stride,pad,groups,act", BF16_SHAPES)
+def test_three_piece_mode_meets_the_fp32_bar(bf16x3, orc, b, c, h, w, n, size, stride, pad, groups, act):
+    """precision 2: operands split into three bf16 pieces, six piece-products summed in fp32.  No
+    rounding of the operands survives (x = hi + mid + lo exactly), so the fp32 parity bar applies
+    unchanged, with the fp64 convolution as referee: the mode must sit as close to it as the
+    fp32 checker does (within a factor that leaves room for the three dropped 2^-24 terms)."""
+    x = synth.uniform(11, b * c * h * w).reshape(b, c, h, w)
+    wt = synth.conv_weights(12, n, c // groups, size)
+    bias, sc, mu, var = synth.bn_random(13, n)
+    kw = dict(n=n, size=size, stride=stride, pad=pad, groups=groups)
+    name = bf16x3.conv_kernel_name(n, c, groups, size).decode()
+    assert name.count(",") == 5 and name.endswith(",3>")
+    got = run_conv(bf16x3, x, wt, bias, sc, mu, var, bn=1, act=act, **kw)
+    want = orc.conv(x, wt, bias, sc, mu, var, batch_normalize=1, activation=act, **kw)
+    ref64 = orc.conv_f64(x, wt, bias, sc, mu, var, batch_normalize=1, activation=act, **kw)
+    e_cpu, e_64, cpu_64 = norm_err(got, want), norm_err(got, ref64), norm_err(want, ref64)
+    print(f"three-piece mode {size}x{size}/{stride} {c}->{n} g{groups}: vs cpu {e_cpu:.2e}, vs fp64 {e_64:.2e}, "
+          f"cpu vs fp64 {cpu_64:.2e}")
+    assert e_cpu <= REL_TOL
+    assert e_64 <= max(4 * cpu_64, 2e-6)
+
+
+@pytest.mark.parametrize("b,c,h,w,n,size,stride,pad,groups,act,bn", __import__("test_gpu_conv").random_geometries(778, 24))
+def test_three_piece_mode_random_geometries(bf16x3, orc, b, c, h, w, n, size, stride, pad, groups, act, bn):
+    x = synth.uniform(51, b * c * h * w).reshape(b, c, h, w)
+    wt = synth.conv_weights(52, n, c // groups, size)
+    bias, sc, mu, var = synth.bn_random(53, n)
+    if not bn:
+        sc = mu = var = None
+    kw = dict(n=n, size=size, stride=stride, pad=pad, groups=groups)
+    got = run_conv(bf16x3, x, wt, bias, sc, mu, var, bn=bn, act=act, **kw)
+    want = orc.conv(x, wt, bias, sc, mu, var, batch_normalize=bn, activation=act, **kw)
+    assert norm_err(got, want) <= REL_TOL, bf16x3.conv_kernel_name(n, c, groups, size)
+
+
+def test_three_piece_mode_whole_network(bf16x3):
+    """yolov3 at 160 in the three-piece mode: per-layer <= 1e-4 and yolo heads <= 1e-3, the bar of
+    the fp32 mode."""
+    from test_gpu_network import check_network
+    assert check_network(cfgs.yolov3(1, 160)) <= REL_TOL
+
+
 def test_layers_on_other_kernels_stay_fp32(bf16, orc):
     """3 input channels -> reference-order kernel: the switch must not touch it."""
     b, c, h, w, n = 2, 3, 33, 35, 32
