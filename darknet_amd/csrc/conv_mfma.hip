@@ -212,9 +212,12 @@ template <int TM, int TN>
 __device__ __forceinline__ void conv_epilogue(const mfma_args &a, f32x16 (&acc)[TM][TN], float *E, int m0,
                                               long n0, int wm0, int wn0, int lane)
 {
-    static_assert(TN == 2, "a wave's tile is 64 columns wide");
+    static_assert(TN == 1 || TN == 2, "a wave's tile is 32 or 64 columns wide");
+    constexpr int QN = 8 * TN;  /* quads of four pixels per filter row of the turn buffer */
+    constexpr int RS = 32 * TN; /* its row stride in floats */
+    constexpr int RG = 64 / QN; /* filter rows one read instruction covers (4 or 8) */
     const int li = lane & 31, kh = lane >> 5;
-    const int q = lane & 15, fr = lane >> 4; /* after the turn: quad of 4 pixels, row within a group of 4 */
+    const int q = lane & (QN - 1), fr = lane / QN; /* after the turn: quad of 4 pixels, row within a group of RG */
     const int P = a.P;
     const int Nt = (int)a.Ntotal;            /* Ntotal < 2^31 on this path */
     const int n = (int)n0 + wn0 + 4 * q;
@@ -237,14 +240,14 @@ __device__ __forceinline__ void conv_epilogue(const mfma_args &a, f32x16 (&acc)[
                 o.z = conv_tail_one(acc[i][j][rg * 4 + 2], row, conv_f2{a.slope_hi, a.slope_lo});
                 o.w = conv_tail_one(acc[i][j][rg * 4 + 3], row, conv_f2{a.slope_hi, a.slope_lo});
                 const int qq = j * 8 + 2 * rg + kh;
-                *(float4 *)&E[li * 64 + ((qq ^ (li & 15)) << 2)] = o;
+                *(float4 *)&E[li * RS + ((qq ^ (li & (QN - 1))) << 2)] = o;
             }
         }
         __builtin_amdgcn_wave_barrier(); /* LDS operations of one wave complete in order */
 #pragma unroll
-        for (int t = 0; t < 8; ++t) {
-            const int f = fr + 4 * t;
-            const float4 o = *(const float4 *)&E[f * 64 + ((q ^ (f & 15)) << 2)];
+        for (int t = 0; t < 32 / RG; ++t) {
+            const int f = fr + RG * t;
+            const float4 o = *(const float4 *)&E[f * RS + ((q ^ (f & (QN - 1))) << 2)];
             const int m = mrow + f;
             if (m >= a.M || n >= Nt) continue;
             const long o_off = off + (long)m * P;
@@ -1118,8 +1121,11 @@ extern "C" const char *conv_kernel_name(int n, int c, int groups, int size)
     const int bf16 = g_precision == 1 && mode >= 10;
     const int x3 = g_precision == 2 && mode >= 10;
     if (bf16 && bm == 128 && n > 128) bm = 256;
-    snprintf(name, sizeof name, "conv_mfma_kernel<%d,%d,%d,64,%d%s>", bm, bm >= 128 ? 128 : 256,
-             bm == 32 ? 32 : bm == 256 ? 128 : 64, mode, x3 ? ",3" : !bf16 ? "" : mode == 13 ? ",2" : ",1");
+    if (x3 && bm == 128)
+        snprintf(name, sizeof name, "conv_mfma_kernel<128,128,128,32,%d,3>", mode);
+    else
+        snprintf(name, sizeof name, "conv_mfma_kernel<%d,%d,%d,64,%d%s>", bm, bm >= 128 ? 128 : 256,
+                 bm == 32 ? 32 : bm == 256 ? 128 : 64, mode, x3 ? ",3" : !bf16 ? "" : mode == 13 ? ",2" : ",1");
     return name;
 }
 
@@ -1199,9 +1205,13 @@ static void launch_tile(const mfma_args &a0, int mode)
     }
     const dim3 grid((unsigned)(a.per_xcd * 8 + tail * split));
     if (BM > 128 && !bf16) dn_fatal("conv dispatch: the 256-row tile is only built for the bf16-operand mode");
+    constexpr bool X3_ONLY = WN == 32; /* the 128x32 wave tile is built for the three-piece mode alone */
+    if (X3_ONLY && !x3) dn_fatal("conv dispatch: the 128x32 wave tile is only built for the three-piece mode");
     switch (mode) {
     case 11:
-        if (bf16) {
+        if constexpr (X3_ONLY) {
+            DN_LAUNCH((conv_mfma_kernel<BM, BN, WM, WN, 11, 3>));
+        } else if (bf16) {
             DN_LAUNCH((conv_mfma_kernel<BM, BN, WM, WN, 11, 1>));
         } else if constexpr (BM <= 128) {
             if (x3)
@@ -1211,7 +1221,9 @@ static void launch_tile(const mfma_args &a0, int mode)
         }
         break;
     case 13:
-        if (bf16) {
+        if constexpr (X3_ONLY) {
+            DN_LAUNCH((conv_mfma_kernel<BM, BN, WM, WN, 13, 3>));
+        } else if (bf16) {
             DN_LAUNCH((conv_mfma_kernel<BM, BN, WM, WN, 13, 2>));
         } else if constexpr (BM <= 128) {
             if (x3)
@@ -1221,7 +1233,7 @@ static void launch_tile(const mfma_args &a0, int mode)
         }
         break;
     default:
-        if constexpr (BM <= 128) {
+        if constexpr (BM <= 128 && !X3_ONLY) {
             if (mode == 1)
                 DN_LAUNCH((conv_mfma_kernel<BM, BN, WM, WN, 1>));
             else if (mode == 3)
@@ -1383,6 +1395,9 @@ static void conv_forward(const float *input, const float *weights, const float *
         launch_tile<256, 128, 128, 64>(a, mode);
     else if (n <= 64)
         launch_tile<64, 256, 64, 64>(a, mode);
+    else if (g_precision == 2 && mode >= 10)
+        /* four waves side by side, 128 rows x 32 columns each: no two waves split the same activations */
+        launch_tile<128, 128, 128, 32>(a, mode);
     else
         launch_tile<128, 128, 64, 64>(a, mode);
     dn_check_launch("forward_convolutional_gpu");
