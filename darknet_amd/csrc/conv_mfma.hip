@@ -1205,7 +1205,9 @@ static void launch_tile(const mfma_args &a0, int mode)
     }
     const dim3 grid((unsigned)(a.per_xcd * 8 + tail * split));
     if (BM > 128 && !bf16) dn_fatal("conv dispatch: the 256-row tile is only built for the bf16-operand mode");
-    constexpr bool X3_ONLY = WN == 32; /* the 128x32 wave tile is built for the three-piece mode alone */
+    constexpr bool X3_ONLY = WN == 32; /* the 128x32 wave tile is built for the three-piece mode alone ... */
+    constexpr bool NO_X3 = BM == 128 && WN == 64; /* ... which never runs the 128x128 tile with 64x64 wave tiles */
+    if (NO_X3 && x3) dn_fatal("conv dispatch: the three-piece mode runs 128x128 tiles with 128x32 wave tiles");
     if (X3_ONLY && !x3) dn_fatal("conv dispatch: the 128x32 wave tile is only built for the three-piece mode");
     switch (mode) {
     case 11:
@@ -1214,10 +1216,13 @@ static void launch_tile(const mfma_args &a0, int mode)
         } else if (bf16) {
             DN_LAUNCH((conv_mfma_kernel<BM, BN, WM, WN, 11, 1>));
         } else if constexpr (BM <= 128) {
-            if (x3)
-                DN_LAUNCH((conv_mfma_kernel<BM, BN, WM, WN, 11, 3>));
-            else
-                DN_LAUNCH((conv_mfma_kernel<BM, BN, WM, WN, 11>));
+            if constexpr (!NO_X3) {
+                if (x3) {
+                    DN_LAUNCH((conv_mfma_kernel<BM, BN, WM, WN, 11, 3>));
+                    break;
+                }
+            }
+            DN_LAUNCH((conv_mfma_kernel<BM, BN, WM, WN, 11>));
         }
         break;
     case 13:
@@ -1226,10 +1231,13 @@ static void launch_tile(const mfma_args &a0, int mode)
         } else if (bf16) {
             DN_LAUNCH((conv_mfma_kernel<BM, BN, WM, WN, 13, 2>));
         } else if constexpr (BM <= 128) {
-            if (x3)
-                DN_LAUNCH((conv_mfma_kernel<BM, BN, WM, WN, 13, 3>));
-            else
-                DN_LAUNCH((conv_mfma_kernel<BM, BN, WM, WN, 13>));
+            if constexpr (!NO_X3) {
+                if (x3) {
+                    DN_LAUNCH((conv_mfma_kernel<BM, BN, WM, WN, 13, 3>));
+                    break;
+                }
+            }
+            DN_LAUNCH((conv_mfma_kernel<BM, BN, WM, WN, 13>));
         }
         break;
     default:
