@@ -26,6 +26,10 @@
  * summed in slice order by conv_reduce_kernel (deterministic).
  * Epilogue: batch-norm, bias and activation in the accumulator layout, a turn through LDS, then
  * 256-byte row stores; a same-geometry residual add (shortcut layer) can ride along.
+ * Three opt-in variants of the same kernel run on the bf16 matrix cores (template parameter BF16,
+ * conv_set_precision): operands rounded to bf16 (1: fp32 activation tiles converted in registers,
+ * 2: 3x3 layers gathering from a staged bf16 copy of the input; both with bf16 weights, four LDS
+ * stages and 256x128 tiles), and fp32 emulated with three bf16 pieces per operand (3).
  *
  * Order of K.  The sum over k does not care about the order as long as A and B agree, and the
  * packing step can permute K for free, so two orders are used:

@@ -1,11 +1,14 @@
-"""The opt-in bf16-operand mode of the tap-blocked MFMA convolution kernels.
+"""The two opt-in modes of the tap-blocked MFMA convolution kernels that run on the bf16 matrix cores.
 
-What the mode computes is pinned exactly: the CPU checker run on operands rounded to bf16 (round
-to nearest even, done here in integer arithmetic) must agree with the kernel to the fp32 bar
-(<= 1e-4 max-normalised; the products of two bf16 numbers are exact in fp32, so only the
-summation order differs).  Against the unrounded fp32 checker the mode's error is measured and
-bounded loosely (it is a precision trade, not a parity claim), and the default fp32 mode must be
-untouched by a round trip through the switch."""
+bf16-operand mode (conv_set_precision(1)).  What it computes is pinned exactly: the CPU checker run
+on operands rounded to bf16 (round to nearest even, done here in integer arithmetic) must agree with
+the kernel to the fp32 bar (<= 1e-4 max-normalised; the products of two bf16 numbers are exact in
+fp32, so only the summation order differs).  Against the unrounded fp32 checker the mode's error is
+measured and bounded loosely (it is a precision trade, not a parity claim), and the default fp32
+mode must be untouched by a round trip through the switch.
+
+Three-piece mode (conv_set_precision(2)): fp32 emulated with three bf16 pieces per operand.  It is
+held to the fp32 parity bar itself, with the fp64 convolution as referee."""
 import numpy as np
 import pytest
 
