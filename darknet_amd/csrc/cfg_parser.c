@@ -457,7 +457,7 @@ network *parse_network_cfg(char *filename)
         net->truths = out->outputs;
         if (last->truths) net->truths = last->truths;
         if (!out->output) {
-            out->output = (float *)dn_calloc((size_t)out->outputs * out->batch, sizeof(float));
+            out->output = hip_host_alloc((size_t)out->outputs * out->batch);
             /* a dropout layer behind it shares the buffer (src/parser.c:831) */
             if (i + 1 < net->n && net->layers[i + 1].type == DROPOUT) net->layers[i + 1].output = out->output;
         }

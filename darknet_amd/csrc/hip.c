@@ -128,6 +128,56 @@ void hip_free(float *x_gpu)
     hip_check_error(hipFree(x_gpu));
 }
 
+/* Pinned host buffers for what network_predict hands back (yolo / region / last-layer outputs):
+ * a copy into pinned memory is one DMA at the link's rate, where pageable memory has to pass
+ * through the staging buffers below at the speed of a host memcpy.  The library remembers its own
+ * pinned blocks so that push/pull recognise them; anything else is treated as pageable. */
+static struct { char *p; size_t bytes; } *g_pinned = 0;
+static int g_npinned = 0, g_cap_pinned = 0;
+
+float *hip_host_alloc(size_t n)
+{
+    const size_t bytes = sizeof(float) * (n ? n : 1);
+    void *p = 0;
+    if (g_parse_only || hipHostMalloc(&p, bytes, hipHostMallocDefault) != hipSuccess || !p) {
+        (void)hipGetLastError(); /* the failed allocation must not surface at the next launch check */
+        p = calloc(1, bytes);
+        if (!p) dn_fatal("Malloc error");
+        return (float *)p;
+    }
+    memset(p, 0, bytes);
+    if (g_npinned == g_cap_pinned) {
+        g_cap_pinned = g_cap_pinned ? 2 * g_cap_pinned : 16;
+        g_pinned = realloc(g_pinned, sizeof(*g_pinned) * (size_t)g_cap_pinned);
+        if (!g_pinned) dn_fatal("Malloc error");
+    }
+    g_pinned[g_npinned].p = (char *)p;
+    g_pinned[g_npinned].bytes = bytes;
+    ++g_npinned;
+    return (float *)p;
+}
+
+void hip_host_free(float *x)
+{
+    int i;
+    if (!x) return;
+    for (i = 0; i < g_npinned; ++i)
+        if (g_pinned[i].p == (char *)x) {
+            hip_check_error(hipHostFree(x));
+            g_pinned[i] = g_pinned[--g_npinned];
+            return;
+        }
+    free(x);
+}
+
+static int host_is_pinned(const void *x, size_t bytes)
+{
+    int i;
+    for (i = 0; i < g_npinned; ++i)
+        if ((const char *)x >= g_pinned[i].p && (const char *)x + bytes <= g_pinned[i].p + g_pinned[i].bytes) return 1;
+    return 0;
+}
+
 /* Large copies between pageable host memory and the device go through two pinned staging
  * buffers on a stream of their own: the CPU copy of chunk i+1 into (out of) one buffer overlaps
  * the DMA of chunk i from (into) the other.  A plain hipMemcpy from pageable memory stages through
@@ -196,7 +246,7 @@ static void staged_copy(char *dev, char *host, size_t bytes, int to_device)
 void hip_push_array(float *x_gpu, float *x, size_t n)
 {
     if (g_parse_only) return; /* the host copy is the only copy */
-    if (sizeof(float) * n >= DN_STAGE_MIN) {
+    if (sizeof(float) * n >= DN_STAGE_MIN && !host_is_pinned(x, sizeof(float) * n)) {
         staged_copy((char *)x_gpu, (char *)x, sizeof(float) * n, 1);
         return;
     }
@@ -207,7 +257,7 @@ void hip_push_array(float *x_gpu, float *x, size_t n)
 void hip_pull_array(float *x_gpu, float *x, size_t n)
 {
     if (g_parse_only) return;
-    if (sizeof(float) * n >= DN_STAGE_MIN) {
+    if (sizeof(float) * n >= DN_STAGE_MIN && !host_is_pinned(x, sizeof(float) * n)) {
         staged_copy((char *)x_gpu, (char *)x, sizeof(float) * n, 0);
         return;
     }

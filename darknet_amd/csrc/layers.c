@@ -305,7 +305,7 @@ layer make_yolo_layer(int batch, int w, int h, int n, int total, int *mask, int 
     l.outputs = h * w * n * (classes + 4 + 1);
     l.inputs = l.outputs;
     l.truths = 90 * (4 + 1);
-    l.output = (float *)dn_calloc((size_t)batch * l.outputs, sizeof(float));
+    l.output = hip_host_alloc((size_t)batch * l.outputs); /* pinned: network_predict pulls it every call */
     for (i = 0; i < total * 2; ++i) l.biases[i] = .5f;
     l.forward_gpu = forward_yolo_layer_gpu;
     l.output_gpu = hip_make_array(0, (size_t)batch * l.outputs);
@@ -600,7 +600,7 @@ layer make_region_layer(int batch, int w, int h, int n, int classes, int coords)
     l.outputs = h * w * n * (classes + coords + 1);
     l.inputs = l.outputs;
     l.truths = 30 * (l.coords + 1);
-    l.output = (float *)dn_calloc((size_t)batch * l.outputs, sizeof(float));
+    l.output = hip_host_alloc((size_t)batch * l.outputs);
     for (i = 0; i < n * 2; ++i) l.biases[i] = .5f;
     l.forward_gpu = forward_region_layer_gpu;
     l.output_gpu = hip_make_array(0, (size_t)batch * l.outputs);
@@ -625,7 +625,7 @@ void free_layer(layer l)
     free(l.weights);
     free(l.rolling_mean);
     free(l.rolling_variance);
-    free(l.output);
+    hip_host_free(l.output);
     free(l.indexes);
     if (l.indexes_gpu) hip_free((float *)l.indexes_gpu);
     if (l.weights_gpu) hip_free(l.weights_gpu);

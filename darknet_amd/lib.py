@@ -87,6 +87,7 @@ SIGNATURES = {
     "network_set_fusion": (None, [i]),
     "forward_network_profiled_kernels": (f, [V, F, F]),
     "hip_set_parse_only": (None, [i]), "hip_parse_only": (i, []),
+    "hip_host_alloc": (F, [z]), "hip_host_free": (None, [F]),
     "conv_set_precision": (None, [i]), "conv_get_precision": (i, []),
     "conv_profile_next": (None, [V, V]), "conv_profile_pending": (i, []),
     "conv_kernel_name": (C.c_char_p, [i, i, i, i]), "layer_output_host": (F, [V, i]),

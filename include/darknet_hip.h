@@ -48,6 +48,12 @@ float  hip_compare(float *x_gpu, float *x, size_t n, char *s); /* cuda_compare  
 void   hip_pull_int_array(int *x_gpu, int *x, size_t n);/* (maxpool indexes; no reference twin) */
 void   hip_push_int_array(int *x_gpu, int *x, size_t n);/* (counters; no reference twin)        */
 void   hip_synchronize(void);                           /* hipStreamSynchronize on the stream  */
+/* Pinned host memory (zero-filled; no reference twin): hip_push_array / hip_pull_array move such a
+ * buffer with one DMA at the link's rate instead of staging it through a host memcpy.  The library
+ * uses it for the outputs network_predict returns; callers may use it for their input batches.
+ * hip_host_free also accepts (and free()s) ordinary malloc'ed pointers. */
+float *hip_host_alloc(size_t n);
+void   hip_host_free(float *x);
 /* Parse-only mode (no reference twin): after hip_set_parse_only(1) the cfg parser, the layer-table
  * queries and the weights-file reader/writer work on host memory alone, on a machine with or
  * without a GPU: nothing is allocated on or copied to a device (device pointers stay NULL).  It
