@@ -114,6 +114,17 @@ def do_nms_sort(rows: np.ndarray, classes: int, thresh: float) -> np.ndarray:
     return _rows_of(dets, n, classes)
 
 
+def pinned_array(n: int):
+    """A zero-filled float32 numpy array over pinned host memory (hip_host_alloc): push/pull and
+    network_predict move it with one DMA.  Release it with free_pinned_array."""
+    ptr = _lib.load().hip_host_alloc(n)
+    return np.ctypeslib.as_array(ptr, shape=(n,))
+
+
+def free_pinned_array(a):
+    _lib.load().hip_host_free(a.ctypes.data_as(C.POINTER(C.c_float)))
+
+
 def set_gpu(n: int = 0):
     _lib.load().cuda_set_device(n)
 
