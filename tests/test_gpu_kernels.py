@@ -8,10 +8,10 @@ import os
 import numpy as np
 import pytest
 
-from darknet_amd import api, synth
+from darknet_amd import api, cfgs, synth
 from oracle.cpu import ACTIVATIONS
 
-from util import norm_err
+from util import fill_params, norm_err
 
 pytestmark = pytest.mark.gpu
 GOLD = os.path.join(os.path.dirname(__file__), "golden")
@@ -221,3 +221,33 @@ def test_large_copies_round_trip_through_the_staging_buffers(dn, n):
     dn.fill_gpu(1000, 3.5, d.ptr, 1)
     dn.hip_pull_array(d.ptr, api._fp(back), n)
     assert np.all(back[:1000] == 3.5) and np.array_equal(back[1000:], y[1000:])
+
+
+def test_pinned_host_buffers_copy_directly_and_predict_the_same(dn):
+    """hip_host_alloc memory is zero-filled, moves with push/pull like any host buffer (also from the
+    middle of the block and across the staging threshold), and a batch built in it gives the bits
+    network_predict gives for the same batch in pageable memory."""
+    n = (8 << 20) // 4 + 77
+    a = api.pinned_array(n)
+    assert a.dtype == np.float32 and not a.any()
+    x = synth.uniform(5, n, -1, 1)
+    a[:] = x
+    d = D(n=n)
+    dn.hip_push_array(d.ptr, api._fp(a), n)
+    dn.fill_gpu(500, -2.0, d.ptr, 1)                # queued work is seen by the pull
+    b = api.pinned_array(n + 10)
+    dn.hip_pull_array(d.ptr, api._fp(b[10:]), n)    # inside the pinned block, offset start
+    assert np.all(b[10:510] == -2.0) and np.array_equal(b[510:], x[500:]) and not b[:10].any()
+    api.free_pinned_array(a)
+    api.free_pinned_array(b)
+
+    net = api.Network(cfg_text=cfgs.yolov3_tiny(2, 96))
+    fill_params(net.set_conv, net.layers)
+    xin = synth.uniform01(9, net.inputs * 2)
+    want = net.predict(xin)
+    p = api.pinned_array(xin.size)
+    p[:] = xin
+    got = net.predict(p)
+    assert np.array_equal(got, want)
+    api.free_pinned_array(p)
+    net.free()
