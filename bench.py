@@ -160,6 +160,78 @@ def cpu_baseline(kind_pref, cfg_name, size, budget_s=20.0):
                       f"-Ofast -fopenmp, OMP_NUM_THREADS={threads}, {dt:.3f} s/pass"}
 
 
+def post_bench(args):
+    """--post: latency of the steps either side of the forward pass for one 416x416 yolov3 image -
+    letterbox of a 1920x1080 frame into the network input and get_network_boxes + do_nms_sort on the
+    three yolo heads - on the device, and the compiled reference's CPU functions on the same data
+    (resize/letterbox_image, get_network_boxes, do_nms_sort).  Prints one JSON line of its own."""
+    import ctypes as C
+    import numpy as np
+    from darknet_amd import api, cfgs, synth
+    api.set_gpu(0)
+    L = api._lib.load()
+    text = cfgs.yolov3(1, 416)
+    net = api.Network(cfg_text=text)
+    fill_params(net.set_conv, net.layers)
+    frame = synth.uniform01(3, 3 * 1080 * 1920).reshape(3, 1080, 1920)
+    x = synth.uniform01(7, net.inputs)
+    net.predict(x)
+    heads = {i: net.layer_output(i) for i, Ly in enumerate(net.layers) if Ly["type"] == "yolo"}
+
+    def timed(fn, reps):
+        fn()
+        L.hip_synchronize()
+        t0 = time.perf_counter()
+        for _ in range(reps):
+            fn()
+        L.hip_synchronize()
+        return (time.perf_counter() - t0) * 1e3 / reps
+
+    out = {"metric": "post-processing latency", "unit": "ms", "workload": "yolov3-416, one 1920x1080 frame", "gpu": {},
+           "cpu_reference": {}}
+    out["gpu"]["letterbox_1080p_into_input_ms"] = round(timed(lambda: net.letterbox_input(0, frame), 20), 4)
+    obj = np.concatenate([h.reshape(3, 85, -1)[:, 4, :].ravel() for h in heads.values()])
+    num = C.c_int(0)
+    for want in (50, 500, 5000):
+        thresh = float(np.sort(obj)[-want])
+        def boxes():
+            d = L.get_network_boxes_image(net.net, 0, 1920, 1080, thresh, 1, 0.45, C.byref(num))
+            L.free_detections(d, num.value)
+        ms = timed(boxes, 20)
+        out["gpu"][f"boxes_nms_{want}_candidates_ms"] = round(ms, 4)
+        out["gpu"][f"boxes_nms_{want}_candidates_kept"] = int(num.value)
+    net.free()
+    try:
+        from oracle import ref
+        if ref.available("fast"):
+            with tempfile.NamedTemporaryFile("w", suffix=".cfg", delete=False) as f:
+                f.write(text)
+            devnull = os.open(os.devnull, os.O_WRONLY)
+            saved = os.dup(2)
+            os.dup2(devnull, 2)
+            try:
+                rnet = ref.RefNet(f.name, "fast")
+            finally:
+                os.dup2(saved, 2)
+                os.close(devnull)
+                os.close(saved)
+                os.unlink(f.name)
+            for i, h in heads.items():
+                rnet.set_output(i, h)
+            t0 = time.perf_counter()
+            ref.letterbox_image(frame, 416, 416, "fast")
+            out["cpu_reference"]["letterbox_1080p_ms"] = round((time.perf_counter() - t0) * 1e3, 3)
+            for want in (50, 500, 5000):
+                thresh = float(np.sort(obj)[-want])
+                t0 = time.perf_counter()
+                rows = rnet.get_boxes(1920, 1080, thresh, 1, 0.45)
+                out["cpu_reference"][f"boxes_nms_{want}_candidates_ms"] = round((time.perf_counter() - t0) * 1e3, 3)
+            out["cpu_reference"]["kind"] = "compiled reference, -Ofast -fopenmp"
+    except Exception as e:  # the CPU leg is a comparison only
+        log("cpu reference leg failed:", repr(e))
+    print(json.dumps(out), flush=True)
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -172,12 +244,18 @@ def main():
                     help="bf16: the tap-blocked MFMA kernels round their operands to bf16 (opt-in, not the "
                          "headline configuration; its error against fp32 is reported by the tests)")
     ap.add_argument("--no-cpu", action="store_true")
+    ap.add_argument("--post", action="store_true",
+                    help="time letterbox and detection decode + NMS around the forward pass instead")
     ap.add_argument("--cpu-kind", default="reference", choices=["reference", "port"])
     args = ap.parse_args()
     if args.gpus != 1:
         log("bench.py: this build runs on one GPU only (the forward path has no exchange step: it shards "
             "by batch, every GPU running the same forward on its share of the images). Use --gpus 1.")
         sys.exit(2)
+
+    if args.post:
+        post_bench(args)
+        return
 
     import numpy as np
     from darknet_amd import api, cfgs, synth
