@@ -8,8 +8,9 @@ Default workload: yolov3 at 416x416, batch 64, fp32 - the configuration the head
 quoted on.  Prints ONE JSON line on stdout; progress goes to stderr.
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload yolov3-416|yolov3-608|yolov3-tiny-416|
-                    yolov3-tiny-xnor-416|resnext50-224] [--batch B] [--precision fp32|bf16]
+                    yolov3-tiny-xnor-416|resnext50-224] [--batch B] [--precision fp32|bf16x3|bf16]
                     [--per-layer FILE] [--no-cpu]
+    python bench.py --post      (letterbox and detection decode + NMS latency instead of the forward pass)
 
 The line carries, besides the driver's fields:
   roofline      the dominant kernel's algorithmic FLOP/s against the fp32 MFMA peak, from HIP
