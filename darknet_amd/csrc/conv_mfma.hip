@@ -1303,6 +1303,24 @@ static void conv_forward(const float *input, const float *weights, const float *
     if ((long)batch * c * h * w >= (1L << 40) || (long)batch * n * oh * ow >= (1L << 40))
         dn_fatal("forward_convolutional_gpu: tensor too large");
 
+    /* The MFMA kernels address the input through 32-bit buffer offsets and count output columns in
+     * 32 bits.  A batch beyond that is processed in slices of whole images (images are independent),
+     * so only a single image of 4 GiB or 2^31 pixels ever falls back to the direct kernel. */
+    if (g_algo != 1 && batch > 1) {
+        const long in_img = (long)c * h * w * 4, out_img = (long)n * oh * ow;
+        const long by_bytes = ((1L << 32) - (2L << 20)) / in_img, by_cols = ((1L << 31) - 1024) / ((long)oh * ow);
+        const long per = by_bytes < by_cols ? by_bytes : by_cols;
+        if (per >= 1 && per < batch) {
+            for (long b0 = 0; b0 < batch; b0 += per) {
+                const int nb = (int)(batch - b0 < per ? batch - b0 : per);
+                conv_forward(input + b0 * (in_img / 4), weights, packed, biases, scales, rolling_mean, rolling_variance,
+                             output + b0 * out_img, nb, c, h, w, n, groups, size, stride, pad, batch_normalize,
+                             activation, add ? add + b0 * out_img : 0, sum ? sum + b0 * out_img : 0, s1, s2, sum_act);
+            }
+            return;
+        }
+    }
+
     const long K = (long)(c / groups) * size * size;
     int mode = conv_mode(c, groups, size, stride, pad, (long)batch * c * h * w * 4);
     /* grouped layers that fit the 32-filter block-diagonal scheme run on the tap-blocked kernel */

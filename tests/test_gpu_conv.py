@@ -246,3 +246,26 @@ def test_conv_shortcut_fused_equals_separate_calls(dn, b, c, h, w, n, size, stri
     assert np.array_equal(out_a.numpy((total,)), out_b.numpy((total,)))
     assert np.array_equal(sum_a.numpy((total,)), sum_b.numpy((total,)))
     assert np.abs(sum_b.numpy((total,))).max() > 0
+
+
+def test_batches_beyond_4_gib_run_in_slices_of_whole_images(dn):
+    """The MFMA kernels address their input with 32-bit offsets.  A batch whose input exceeds 4 GiB
+    is cut into slices of whole images on the host instead of falling back to the direct kernel:
+    every image must equal the result of convolving it alone (summation order aside)."""
+    b, c, h, w, n = 63, 16, 1040, 1040, 16          # 63 x 69.2 MB = 4.36 GB in, the same out
+    assert b * c * h * w * 4 > (1 << 32)
+    rng = np.random.default_rng(5)
+    x = rng.random((b, c, h, w), dtype=np.float32) - 0.5
+    wt = synth.conv_weights(61, n, c, 3)
+    bias, sc, mu, var = synth.bn_random(62, n)
+    kw = dict(n=n, size=3, stride=1, pad=1, groups=1, bn=1, act="leaky")
+    assert dn.conv_kernel_name(n, c, 1, 3).decode().startswith("conv_mfma_kernel")
+    ev = dn.hip_event_create(), dn.hip_event_create()
+    dn.conv_profile_next(ev[0], ev[1])         # only an MFMA launch takes the pair of events
+    got = run_conv(dn, x, wt, bias, sc, mu, var, **kw)
+    assert dn.conv_profile_pending() == 0 and dn.hip_event_elapsed_ms(ev[0], ev[1]) > 0
+    assert got.shape == (b, n, h, w)
+    per = ((1 << 32) - (2 << 20)) // (c * h * w * 4)      # images per slice
+    for i in (0, per - 1, per, b - 1):
+        alone = run_conv(dn, x[i:i + 1], wt, bias, sc, mu, var, **kw)
+        assert norm_err(got[i:i + 1], alone) <= 1e-5, i
