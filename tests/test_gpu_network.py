@@ -210,7 +210,7 @@ def test_kernel_stamped_timing(dn):
     for i, L in enumerate(net.layers):
         assert np.array_equal(net.layer_output(i), want[i]), i
         if L["type"] == "convolutional":
-            assert 0 < kernel_ms[i] <= layer_ms[i] + 0.05, (i, kernel_ms[i], layer_ms[i])
+            assert 0 < kernel_ms[i] <= layer_ms[i] + 0.25, (i, kernel_ms[i], layer_ms[i])   # slack: two timers
         else:
             assert kernel_ms[i] == -1.0, (i, L["type"], kernel_ms[i])
     assert sum(k for k in kernel_ms if k > 0) < total
