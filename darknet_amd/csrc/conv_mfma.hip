@@ -213,8 +213,8 @@ __device__ __forceinline__ float conv_residual_one(const mfma_args &a, float y, 
  * reads them back with 16 lanes per filter row: a store instruction then covers 4 rows of 256
  * contiguous bytes, and the residual of a fused shortcut is read the same way. */
 template <int TM, int TN>
-__device__ __forceinline__ void conv_epilogue(const mfma_args &a, f32x16 (&acc)[TM][TN], float *E, int m0,
-                                              long n0, int wm0, int wn0, int lane)
+__device__ __forceinline__ void conv_epilogue(const mfma_args &a, f32x16 (&acc)[TM][TN], float *E,
+                                              const conv_row_t *rows, int m0, long n0, int wm0, int wn0, int lane)
 {
     static_assert(TN == 1 || TN == 2, "a wave's tile is 32 or 64 columns wide");
     constexpr int QN = 8 * TN;  /* quads of four pixels per filter row of the turn buffer */
@@ -233,7 +233,7 @@ __device__ __forceinline__ void conv_epilogue(const mfma_args &a, f32x16 (&acc)[
 #pragma unroll
     for (int i = 0; i < TM; ++i) {
         const int mrow = m0 + wm0 + i * 32;
-        const conv_row_t row = conv_row(a, mrow + li < a.M ? mrow + li : a.M - 1);
+        const conv_row_t row = rows[wm0 + i * 32 + li]; /* computed once per workgroup */
 #pragma unroll
         for (int j = 0; j < TN; ++j) {
 #pragma unroll
@@ -325,6 +325,7 @@ __global__ __launch_bounds__(DN_THREADS, ((BM == 128 && BF16 != 3) ? 3 : 2)) voi
     static_assert(!V3 || S_FLOATS >= 2048, "a stage doubles as one wave's epilogue buffer");
     __shared__ __attribute__((aligned(16))) float S0[S_FLOATS], S1[S_FLOATS], S2[S_FLOATS], S3[S_FLOATS];
 #define S_BUF(b) ((b) == 0 ? S0 : (b) == 1 ? S1 : (b) == 2 ? S2 : S3)
+    __shared__ conv_row_t rows_s[BM]; /* batch-norm constants of the tile's filters, for the epilogue */
 #define A_BUF(b) (V3 ? S_BUF(b) : ((b) == 0 ? As0 : (b) == 1 ? As1 : (b) == 2 ? As2 : As3))
 #define B_BUF(b) (V3 ? S_BUF(b) + A_FLOATS : ((b) == 0 ? Bs0 : (b) == 1 ? Bs1 : (b) == 2 ? Bs2 : Bs3))
 
@@ -785,12 +786,16 @@ __global__ __launch_bounds__(DN_THREADS, ((BM == 128 && BF16 != 3) ? 3 : 2)) voi
                 for (int r = 0; r < 16; ++r)
                     ws[((wave * TM * TN + i * TN + j) * 16 + r) * 64 + lane] = acc[i][j][r];
     } else {
+        /* The per-filter constants cost a double-precision square root and division each: one lane
+         * per filter of the tile computes them once (every wave would otherwise repeat them for
+         * each of its 32-row blocks, on the vector ALU the fp32 MFMAs of the other waves need). */
+        if (tid < BM) rows_s[tid] = conv_row(a, m0 + tid < a.M ? m0 + tid : a.M - 1);
         __syncthreads(); /* every wave has read its last operands: the LDS buffers are free */
         float *E = V3 ? S_BUF(wave)
                    : BM >= 128 ? (BFP ? (wave == 0 ? Bs2 : wave == 1 ? Bs3 : wave == 2 ? Bs0 : Bs1)
                                        : (wave == 0 ? As0 : wave == 1 ? As1 : wave == 2 ? Bs0 : Bs1))
                                : (wave < 2 ? Bs0 : Bs1) + (wave & 1) * 2048;
-        conv_epilogue<TM, TN>(a, acc, E, m0, n0, wm0, wn0, lane);
+        conv_epilogue<TM, TN>(a, acc, E, rows_s, m0, n0, wm0, wn0, lane);
     }
 }
 
