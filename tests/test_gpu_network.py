@@ -261,3 +261,32 @@ def test_connected_layers_at_classifier_sizes(dn):
         assert norm_err(net.layer_output(i), want[i]) <= REL_TOL, i
     assert abs(net.conv_flops() - 2.0 * (9216 * 4096 + 4096 * 1000)) < 1
     net.free()
+
+
+def device_free_bytes():
+    """Free device memory as the HIP runtime (already loaded by the library) reports it."""
+    import ctypes
+    rt = ctypes.CDLL("libamdhip64.so")
+    free, total = ctypes.c_size_t(), ctypes.c_size_t()
+    assert rt.hipMemGetInfo(ctypes.byref(free), ctypes.byref(total)) == 0
+    return free.value
+
+
+def test_free_network_returns_its_device_memory(dn):
+    """A serving process that loads and frees networks must not grow: after a first cycle has
+    sized the library's process-wide work buffers, every later parse -> set weights -> predict ->
+    detect -> free cycle gives back all the device memory it took."""
+    def cycle(text):
+        net = api.Network(cfg_text=text)
+        fill_params(net.set_conv, net.layers, seed=5, bn="random")
+        net.predict(synth.uniform01(3, net.inputs * net.batch))
+        net.free()
+
+    texts = [cfgs.yolov3(2, 416), cfgs.yolov3_tiny(2, 416, xnor=True), cfgs.resnext50(2, 224)]
+    for t in texts:
+        cycle(t)
+    base = device_free_bytes()
+    for _ in range(3):
+        for t in texts:
+            cycle(t)
+    assert device_free_bytes() >= base - (4 << 20), (base, device_free_bytes())

@@ -1,0 +1,55 @@
+"""The library's host C files (cfg reader and parser, layer constructors, weights file reader and
+writer, network bookkeeping) built with AddressSanitizer and UndefinedBehaviorSanitizer and driven
+in parse-only mode by tests/host_driver.c: no bad access, no undefined behaviour, and every byte
+the parser allocates is given back by free_network (LeakSanitizer runs at exit).  The HIP objects
+are the uninstrumented ones the library build left in darknet_amd/build; nothing in them runs."""
+import glob
+import os
+import re
+import shutil
+import subprocess
+
+import pytest
+
+from darknet_amd import build as dbuild
+from oracle import cfg as ocfg
+
+from util import have_reference_tree
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+GOLD = os.path.join(HERE, "golden")
+SAN = ["-g", "-O1", "-fsanitize=address,undefined", "-fno-sanitize-recover=undefined", "-fno-omit-frame-pointer"]
+
+
+def test_host_code_under_address_and_ub_sanitizers(tmp_path):
+    hip_objs = [os.path.join(dbuild.OBJDIR, s + ".o") for s in dbuild.HIP_SOURCES]
+    if not all(os.path.exists(o) for o in hip_objs) or not shutil.which("gcc"):
+        pytest.skip("needs the object files of a library build in this tree")
+    flags = [f for f in dbuild.C_FLAGS if f != "-O2"] + SAN
+    objs = []
+    for s in dbuild.C_SOURCES + ["host_driver.c"]:
+        src = os.path.join(HERE if s == "host_driver.c" else dbuild.CSRC, s)
+        objs.append(str(tmp_path / (s + ".o")))
+        subprocess.run(["gcc"] + flags + ["-c", src, "-o", objs[-1]], check=True)
+    exe = str(tmp_path / "host_driver")
+    subprocess.run(["g++", "-fsanitize=address,undefined", "-o", exe] + objs + hip_objs +
+                   ["-L" + os.path.join(dbuild.ROCM, "lib"), "-Wl,-rpath," + os.path.join(dbuild.ROCM, "lib"),
+                    "-lamdhip64", "-lgomp", "-lm"], check=True)
+
+    again = str(tmp_path / "again.weights")
+    cases = [os.path.join(GOLD, "small_net2.cfg") + "@" + os.path.join(GOLD, "small_net2.weights"),
+             os.path.join(GOLD, "region_net.cfg"),
+             os.path.join(GOLD, "small_net.cfg") + "@" + os.path.join(GOLD, "small_net.weights")]
+    if have_reference_tree():
+        for path in sorted(glob.glob("/root/reference/cfg/*.cfg")):
+            text = open(path).read()
+            kinds = set(re.findall(r"(?m)^\s*(\[[a-z]+\])", text))
+            if kinds <= set(ocfg.SECTION_ALIASES) and not re.search(r"(?m)^\s*(tree|map)\s*=", text):
+                cases.append(path)
+    env = dict(os.environ, ASAN_OPTIONS="detect_leaks=1:halt_on_error=1", UBSAN_OPTIONS="print_stacktrace=1")
+    r = subprocess.run([exe, again] + cases, capture_output=True, text=True, timeout=600, env=env)
+    assert r.returncode == 0, r.stderr[-4000:]
+    assert r.stdout.count("ok ") == len(cases), r.stdout[-2000:]
+    assert "Sanitizer" not in r.stderr and "runtime error" not in r.stderr, r.stderr[-4000:]
+    # the last weights case written back is byte-identical to the file the reference saved
+    assert open(again, "rb").read() == open(os.path.join(GOLD, "small_net.weights"), "rb").read()
