@@ -8,7 +8,7 @@ Default workload: yolov3 at 416x416, batch 64, fp32 - the configuration the head
 quoted on.  Prints ONE JSON line on stdout; progress goes to stderr.
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload yolov3-416|yolov3-608|yolov3-tiny-416|
-                    yolov3-tiny-xnor-416|resnext50-224] [--batch B] [--precision fp32|bf16x3|bf16]
+                    yolov3-tiny-xnor-416|resnext50-224|yolov1-448|yolov1-tiny-448] [--batch B] [--precision fp32|bf16x3|bf16]
                     [--per-layer FILE] [--no-cpu]
     python bench.py --post      (letterbox and detection decode + NMS latency instead of the forward pass)
 
@@ -45,6 +45,8 @@ WORKLOADS = {
     "yolov3-tiny-416": ("yolov3_tiny", 416),
     "resnext50-224": ("resnext50", 224),
     "yolov3-tiny-xnor-416": ("yolov3_tiny_xnor", 416),
+    "yolov1-448": ("yolov1", 448),
+    "yolov1-tiny-448": ("yolov1_tiny", 448),
 }
 
 
@@ -61,8 +63,17 @@ def log(*a):
 
 def fill_params(setter, layers, seed=1000):
     """uniform(-1,1)*sqrt(2/(k*k*c/groups)) weights, biases 0, BN mean 0 / variance 1 / scale 1."""
+    import numpy as np
     from darknet_amd import synth
     for i, L in enumerate(layers):
+        if L["type"] == "local":         # one weight matrix per output location, one bias per output
+            setter(i, synth.conv_weights(seed + i, L["out_h"] * L["out_w"] * L["n"], L["c"], L["size"]),
+                   np.zeros(L["outputs"], np.float32), None, None, None)
+            continue
+        if L["type"] == "connected":
+            setter(i, synth.conv_weights(seed + i, L["outputs"], L["inputs"], 1), np.zeros(L["outputs"], np.float32),
+                   None, None, None)
+            continue
         if L["type"] != "convolutional":
             continue
         w = synth.conv_weights(seed + i, L["n"], L["c"] // L["groups"], L["size"])
@@ -80,6 +91,10 @@ def layer_bytes(L):
     if t == "convolutional":
         wbytes = 4 * L["nweights"] + (16 * L["n"] if L["batch_normalize"] else 4 * L["n"])
         return 4 * b * (L["inputs"] + L["outputs"]) + wbytes
+    if t == "local":
+        return 4 * b * (L["inputs"] + L["outputs"]) + 4 * (L["nweights"] + L["outputs"])
+    if t == "connected":
+        return 4 * b * (L["inputs"] + L["outputs"]) + 4 * (L["inputs"] * L["outputs"] + L["outputs"])
     if t == "maxpool":
         return 4 * b * (L["inputs"] + L["outputs"])  # inference leaves the argmax indexes out
     if t == "shortcut":

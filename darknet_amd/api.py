@@ -301,7 +301,7 @@ class Network:
         suppression of do_nms_sort when nms > 0 -> rows [n, 5 + classes]."""
         num = C.c_int(0)
         dets = self.L.get_network_boxes_image(self.net, image, w, h, thresh, relative, nms, C.byref(num))
-        classes = max([L["classes"] for L in self.layers if L["type"] in ("yolo", "region")] + [0])
+        classes = max([L["classes"] for L in self.layers if L["type"] in ("yolo", "region", "detection")] + [0])
         rows = _rows_of(C.cast(dets, C.POINTER(DETECTION)), num.value, classes)
         self.L.free_detections(dets, num.value)
         return rows
@@ -310,7 +310,7 @@ class Network:
         """The reference's own call (image 0, no suppression)."""
         num = C.c_int(0)
         dets = self.L.get_network_boxes(self.net, w, h, thresh, 0.5, None, relative, C.byref(num))
-        classes = max([L["classes"] for L in self.layers if L["type"] in ("yolo", "region")] + [0])
+        classes = max([L["classes"] for L in self.layers if L["type"] in ("yolo", "region", "detection")] + [0])
         rows = _rows_of(C.cast(dets, C.POINTER(DETECTION)), num.value, classes)
         self.L.free_detections(dets, num.value)
         return rows

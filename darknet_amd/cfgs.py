@@ -144,3 +144,42 @@ SWEEP = {
     "1x1_512to256_52": (512, 52, 52, 256, 1, 1),
     "3x3s2_128to256_104": (128, 104, 104, 256, 3, 2),
 }
+
+
+def _detection(num: int, side: int = 7, classes: int = 20) -> str:
+    return (f"[detection]\nclasses={classes}\ncoords=4\nrescore=1\nside={side}\nnum={num}\nsoftmax=0\nsqrt=1\n"
+            "jitter=.2\nobject_scale=1\nnoobject_scale=.5\nclass_scale=1\ncoord_scale=5\n")
+
+
+def yolov1_tiny(batch: int = 1, size: int = 448) -> str:
+    """cfg/yolov1-tiny.cfg: 8 conv / 6 maxpool, a connected layer onto the 7x7x(2*5+20) grid, detection.
+    The connected layer fixes the input size: side * 64 pixels."""
+    out = [_net(batch, size, size)]
+    for f in [16, 32, 64, 128, 256, 512]:
+        out.append(_conv(f, 3))
+        out.append("[maxpool]\nsize=2\nstride=2\n")
+    out.append(_conv(1024, 3))
+    out.append(_conv(256, 3))
+    out.append("[connected]\noutput=1470\nactivation=linear\n")
+    out.append(_detection(2))
+    return "\n".join(out)
+
+
+def yolov1(batch: int = 1, size: int = 448) -> str:
+    """cfg/yolov1.cfg: 24 conv / 4 maxpool, the locally connected layer on the 7x7x1024 map,
+    dropout, a connected layer onto the 7x7x(3*5+20) grid, detection."""
+    out = [_net(batch, size, size)]
+    pool = "[maxpool]\nsize=2\nstride=2\n"
+    out += [_conv(64, 7, 2), pool, _conv(192, 3), pool,
+            _conv(128, 1), _conv(256, 3), _conv(256, 1), _conv(512, 3), pool]
+    for _ in range(4):
+        out += [_conv(256, 1), _conv(512, 3)]
+    out += [_conv(512, 1), _conv(1024, 3), pool]
+    for _ in range(2):
+        out += [_conv(512, 1), _conv(1024, 3)]
+    out += [_conv(1024, 3), _conv(1024, 3, 2), _conv(1024, 3), _conv(1024, 3)]
+    out.append("[local]\nsize=3\nstride=1\npad=1\nfilters=256\nactivation=leaky\n")
+    out.append("[dropout]\nprobability=.5\n")
+    out.append("[connected]\noutput=1715\nactivation=linear\n")
+    out.append(_detection(3))
+    return "\n".join(out)

@@ -17,7 +17,7 @@ static int network_max_detections(network *net, int *classes)
     int i, s = 0, cl = -1;
     for (i = 0; i < net->n; ++i) {
         layer l = net->layers[i];
-        if (l.type != YOLO && l.type != REGION) continue;
+        if (l.type != YOLO && l.type != REGION && l.type != DETECTION) continue;
         s += l.w * l.h * l.n;
         if (cl >= 0 && cl != l.classes) dn_fatal("detections: heads disagree on the number of classes");
         cl = l.classes;
@@ -48,7 +48,11 @@ int network_decode_image_gpu(network *net, int b, int w, int h, float thresh, in
     for (i = 0; i < net->n; ++i) {
         layer l = net->layers[i];
         float anchors[32];
-        if (l.type == DETECTION) dn_fatal("detections: the yolov1 detection layer is not decoded");
+        if (l.type == DETECTION) { /* src/network.c:555-558 */
+            detection_decode_gpu(l.output_gpu + (size_t)b * l.outputs, l.side, l.n, l.classes, l.sqrt, w, h, thresh,
+                                 net->det_rows_gpu, net->det_max_rows, net->det_count_gpu);
+            continue;
+        }
         if (l.type != YOLO && l.type != REGION) continue;
         if (l.n > 16) dn_fatal("detections: more than 16 anchors per head");
         if (l.type == REGION) { /* src/network.c:553-556 */

@@ -42,6 +42,8 @@ static LAYER_TYPE section_type(const char *t)
     if (!strcmp(t, "[crop]")) return CROP;
     if (!strcmp(t, "[cost]")) return COST;
     if (!strcmp(t, "[region]")) return REGION;
+    if (!strcmp(t, "[local]")) return LOCAL;
+    if (!strcmp(t, "[detection]")) return DETECTION;
     return BLANK;
 }
 
@@ -83,6 +85,8 @@ char *get_layer_string(LAYER_TYPE a)
     case CROP: return "crop";
     case COST: return "cost";
     case REGION: return "region";
+    case LOCAL: return "local";
+    case DETECTION: return "detection";
     default: return "none";
     }
 }
@@ -286,6 +290,37 @@ static layer parse_cost(cfg_section *o, size_params p)
     return make_cost_layer(p.batch, p.inputs, 0, scale);
 }
 
+/* src/parser.c:161-177: pad is the number of zero pixels itself here, not a flag */
+static layer parse_local(cfg_section *o, size_params p)
+{
+    int n = cfg_find_int(o, "filters", 1);
+    int size = cfg_find_int(o, "size", 1);
+    int stride = cfg_find_int(o, "stride", 1);
+    int pad = cfg_find_int(o, "pad", 0);
+    ACTIVATION a = get_activation(cfg_find_str(o, "activation", "logistic"));
+    need_image(p, "local");
+    return make_local_layer(p.batch, p.h, p.w, p.c, n, size, stride, pad, a);
+}
+
+/* src/parser.c:405-428 */
+static layer parse_detection(cfg_section *o, size_params p)
+{
+    static const char *training_keys[] = {"coord_scale", "forced", "object_scale", "noobject_scale", "class_scale",
+                                          "jitter", "random", "reorg", 0};
+    int coords = cfg_find_int(o, "coords", 1);
+    int classes = cfg_find_int(o, "classes", 1);
+    int rescore = cfg_find_int(o, "rescore", 0);
+    int num = cfg_find_int(o, "num", 1);
+    int side = cfg_find_int(o, "side", 7);
+    int i;
+    layer l = make_detection_layer(p.batch, p.inputs, num, side, classes, coords, rescore);
+    l.softmax = cfg_find_int(o, "softmax", 0);
+    l.sqrt = cfg_find_int(o, "sqrt", 0);
+    l.max_boxes = cfg_find_int_quiet(o, "max", 90);
+    for (i = 0; training_keys[i]; ++i) (void)cfg_find(o, training_keys[i]);
+    return l;
+}
+
 /* src/parser.c:353-403 */
 static layer parse_region(cfg_section *o, size_params p)
 {
@@ -416,6 +451,8 @@ network *parse_network_cfg(char *filename)
         case CROP: l = parse_crop(o, p); break;
         case COST: l = parse_cost(o, p); break;
         case REGION: l = parse_region(o, p); break;
+        case LOCAL: l = parse_local(o, p); break;
+        case DETECTION: l = parse_detection(o, p); break;
         case DROPOUT:
             if (count == 0) dn_fatal("dropout cannot be the first layer");
             l = parse_dropout(o, p);

@@ -251,6 +251,70 @@ extern "C" void region_decode_gpu(const float *layer_output, int lw, int lh, int
     dn_check_launch("region_decode_gpu");
 }
 
+/* ---- yolov1 detection layer --------------------------------------------------------------- */
+struct detection_decode_args {
+    const float *pred; /* one image: [cells][classes] probabilities, [cells][n] scales, [cells][n][4] boxes */
+    float *rows;
+    int *count;
+    int max_rows;
+    int side, n, classes, sqrt, w, h;
+    float thresh;
+};
+
+/* get_detection_detections (src/detection_layer.c:225-252) in its own arithmetic: the centre in
+ * float, the extent through pow() in double (pow(x, 2) of a float is the exact product, pow(x, 1)
+ * is x).  The objectness is stored whatever the threshold, as there. */
+__global__ void detection_decode_kernel(detection_decode_args a)
+{
+    const int cells = a.side * a.side;
+    const int total = cells * a.n;
+    const int base = *a.count;
+    for (int idx = blockIdx.x * blockDim.x + threadIdx.x; idx < total; idx += gridDim.x * blockDim.x) {
+        if (base + idx >= a.max_rows) continue;
+        const int cell = idx / a.n;
+        const int row = cell / a.side, col = cell - row * a.side;
+        const float scale = a.pred[cells * a.classes + idx];
+        const float *bx = a.pred + cells * (a.classes + a.n) + idx * 4;
+        const double wd = (double)bx[2], hd = (double)bx[3];
+        float *r = a.rows + (long)(base + idx) * (5 + a.classes);
+        r[0] = __fmul_rn(__fdiv_rn(__fadd_rn(bx[0], (float)col), (float)a.side), (float)a.w);
+        r[1] = __fmul_rn(__fdiv_rn(__fadd_rn(bx[1], (float)row), (float)a.side), (float)a.h);
+        r[2] = (float)((a.sqrt ? wd * wd : wd) * (double)a.w);
+        r[3] = (float)((a.sqrt ? hd * hd : hd) * (double)a.h);
+        r[4] = scale;
+        const float *cls = a.pred + cell * a.classes;
+        for (int j = 0; j < a.classes; ++j) {
+            const float prob = __fmul_rn(scale, cls[j]);
+            r[5 + j] = (prob > a.thresh) ? prob : 0.f;
+        }
+    }
+}
+
+extern "C" void detection_decode_gpu(const float *layer_output, int side, int n, int classes, int sqrt, int w,
+                                     int h, float thresh, float *rows, int max_rows, int *count)
+{
+    if (!layer_output || !rows || !count) dn_fatal("detection_decode_gpu: null pointer");
+    if (side <= 0 || n <= 0 || classes < 0 || w <= 0 || h <= 0 || max_rows < 0 ||
+        (long)side * side * ((long)n * 5 + classes) > 0x7fffffffL)
+        dn_fatal("detection_decode_gpu: bad geometry");
+    detection_decode_args a;
+    a.pred = layer_output;
+    a.rows = rows;
+    a.count = count;
+    a.max_rows = max_rows;
+    a.side = side;
+    a.n = n;
+    a.classes = classes;
+    a.sqrt = sqrt;
+    a.w = w;
+    a.h = h;
+    a.thresh = thresh;
+    const int total = side * side * n;
+    hipLaunchKernelGGL(detection_decode_kernel, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, dn_stream(), a);
+    hipLaunchKernelGGL(add_count_kernel, dim3(1), dim3(1), 0, dn_stream(), count, total);
+    dn_check_launch("detection_decode_gpu");
+}
+
 /* ---- non-maximum suppression ------------------------------------------------------------- */
 /* box_iou of src/box.c:111-155 in the reference's float arithmetic */
 __device__ __forceinline__ float dn_overlap(float x1, float w1, float x2, float w2)

@@ -614,6 +614,104 @@ void forward_region_layer_gpu(layer l, network net)
                        l.softmax);
 }
 
+/* ---- local (yolov1): src/local_layer.c:26-89.  One weight matrix per output location, one bias
+ * per output element; the reference's random initial weights are left to the weights file. ----- */
+layer make_local_layer(int batch, int h, int w, int c, int n, int size, int stride, int pad, ACTIVATION activation)
+{
+    layer l;
+    long locations, nweights;
+    memset(&l, 0, sizeof l);
+    l.type = LOCAL;
+    l.h = h;
+    l.w = w;
+    l.c = c;
+    l.n = n;
+    l.batch = batch;
+    l.stride = stride;
+    l.size = size;
+    l.pad = pad;
+    if (size < 1 || stride < 1 || n < 1 || pad < 0) dn_fatal("local layer: bad size, stride, pad or filters");
+    if ((pad ? 1 : size) > h || (pad ? 1 : size) > w) dn_fatal("local layer: kernel larger than its input");
+    l.out_h = (h - (pad ? 1 : size)) / stride + 1; /* src/local_layer.c:10-24 */
+    l.out_w = (w - (pad ? 1 : size)) / stride + 1;
+    if ((h + 2 * pad - size) / stride + 1 != l.out_h || (w + 2 * pad - size) / stride + 1 != l.out_w)
+        dn_fatal("local layer: pad and size give im2col a different output size than the layer's");
+    l.out_c = n;
+    l.outputs = l.out_h * l.out_w * l.out_c;
+    l.inputs = l.w * l.h * l.c;
+    l.activation = activation;
+    locations = (long)l.out_h * l.out_w;
+    nweights = (long)c * n * size * size * locations;
+    if (nweights >= (1L << 31)) dn_fatal("local layer: too many weights");
+    l.nweights = (int)nweights;
+    l.nbiases = l.outputs;
+    l.weights = (float *)dn_calloc((size_t)nweights, sizeof(float));
+    l.biases = (float *)dn_calloc((size_t)l.outputs, sizeof(float));
+    l.workspace_size = (size_t)l.out_h * l.out_w * size * size * c; /* as src/local_layer.c:63 sets it; unused here */
+    l.forward_gpu = forward_local_layer_gpu;
+    if (gpu_index < 0) dn_fatal("this library has no CPU path: gpu_index must name a device");
+    l.weights_gpu = hip_make_array(l.weights, (size_t)nweights);
+    l.biases_gpu = hip_make_array(l.biases, (size_t)l.outputs);
+    l.output_gpu = hip_make_array(0, (size_t)batch * l.outputs);
+    if (dn_verbose)
+        fprintf(stderr, "Local Layer: %d x %d x %d image, %d filters -> %d x %d x %d image\n", h, w, c, n, l.out_h,
+                l.out_w, n);
+    return l;
+}
+
+void forward_local_layer_gpu(layer l, network net)
+{
+    forward_local_gpu(net.input_gpu, l.weights_gpu, l.biases_gpu, l.output_gpu, l.batch, l.c, l.h, l.w, l.n, l.size,
+                      l.stride, l.pad, (int)l.activation);
+}
+
+void push_local_layer(layer l)
+{
+    hip_push_array(l.weights_gpu, l.weights, (size_t)l.nweights);
+    hip_push_array(l.biases_gpu, l.biases, (size_t)l.outputs);
+}
+
+void pull_local_layer(layer l)
+{
+    hip_pull_array(l.weights_gpu, l.weights, (size_t)l.nweights);
+    hip_pull_array(l.biases_gpu, l.biases, (size_t)l.outputs);
+}
+
+/* ---- detection (yolov1 head): src/detection_layer.c:14-48.  At inference the layer is a copy
+ * of its input, with a softmax over each cell's class scores when `softmax` is set (:50-66; the
+ * reference's GPU forward :256-262 only copies, its CPU forward is followed here). -------------- */
+layer make_detection_layer(int batch, int inputs, int n, int side, int classes, int coords, int rescore)
+{
+    layer l;
+    memset(&l, 0, sizeof l);
+    l.type = DETECTION;
+    l.n = n;
+    l.batch = batch;
+    l.inputs = inputs;
+    l.classes = classes;
+    l.coords = coords;
+    l.rescore = rescore;
+    l.side = side;
+    l.w = side;
+    l.h = side;
+    if (side < 1 || n < 1 || classes < 0 || (long)side * side * ((long)(1 + coords) * n + classes) != inputs)
+        dn_fatal("detection layer: the layer before it must output side*side*((1+coords)*num+classes) values");
+    l.outputs = l.inputs;
+    l.truths = l.side * l.side * (1 + l.coords + l.classes);
+    l.output = hip_host_alloc((size_t)batch * l.outputs);
+    l.forward_gpu = forward_detection_layer_gpu;
+    l.output_gpu = hip_make_array(0, (size_t)batch * l.outputs);
+    if (dn_verbose) fprintf(stderr, "Detection Layer\n");
+    return l;
+}
+
+void forward_detection_layer_gpu(layer l, network net)
+{
+    copy_gpu(l.batch * l.inputs, net.input_gpu, 1, l.output_gpu, 1);
+    if (l.softmax) /* per image and cell, over the classes at the head of the vector */
+        softmax_gpu(net.input_gpu, l.classes, l.batch, l.inputs, l.side * l.side, l.classes, 1, 1.f, l.output_gpu);
+}
+
 void free_layer(layer l)
 {
     if (l.type == DROPOUT) return; /* its buffers belong to the layer before it (src/layer.c:8-14) */

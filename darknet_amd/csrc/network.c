@@ -276,8 +276,15 @@ void network_set_conv(network *net, int i, const float *weights, const float *bi
                       const float *rolling_mean, const float *rolling_variance)
 {
     layer l;
+    if (i >= 0 && i < net->n && net->layers[i].type == LOCAL) { /* weights[nweights], biases[outputs] */
+        l = net->layers[i];
+        if (weights) memcpy(l.weights, weights, sizeof(float) * (size_t)l.nweights);
+        if (biases) memcpy(l.biases, biases, sizeof(float) * (size_t)l.outputs);
+        push_local_layer(l);
+        return;
+    }
     if (i < 0 || i >= net->n || (net->layers[i].type != CONVOLUTIONAL && net->layers[i].type != CONNECTED))
-        dn_fatal("network_set_conv: not a convolutional or connected layer");
+        dn_fatal("network_set_conv: not a convolutional, connected or local layer");
     l = net->layers[i];
     if (weights) memcpy(l.weights, weights, sizeof(float) * (size_t)l.nweights);
     if (biases) memcpy(l.biases, biases, sizeof(float) * (size_t)l.n);

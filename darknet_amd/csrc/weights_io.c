@@ -6,7 +6,8 @@
  * else as int; then, per layer in order, for a convolutional layer: biases[n]; if
  * batch_normalize (and not dontloadscales) scales[n], rolling_mean[n], rolling_variance[n];
  * weights[nweights] (src/parser.c:958-977, :1164-1215); for a connected layer: biases[outputs],
- * weights[outputs*inputs], then the batch-norm vectors (:991-1005, :1098-1120).  Other layer
+ * weights[outputs*inputs], then the batch-norm vectors (:991-1005, :1098-1120); for a local
+ * layer: biases[outputs], weights[locations*n*size*size*c] (:1066-1077, :1292-1302).  Other layer
  * types on this path carry no parameters.  A load ends in push_convolutional_layer, which also refreshes the packed copy
  * the MFMA kernel reads.
  */
@@ -97,6 +98,11 @@ void load_weights_upto(network *net, char *filename, int start, int cutoff)
         if (l.dontload) continue;
         if (l.type == CONVOLUTIONAL) load_convolutional_weights(l, fp);
         if (l.type == CONNECTED) load_connected_weights(l, fp, transpose);
+        if (l.type == LOCAL) { /* src/parser.c:1292-1302 */
+            read_floats(l.biases, (size_t)l.outputs, fp, "local biases");
+            read_floats(l.weights, (size_t)l.nweights, fp, "local weights");
+            push_local_layer(l);
+        }
     }
     if (dn_verbose) fprintf(stderr, "Done!\n");
     fclose(fp);
@@ -130,6 +136,12 @@ void save_weights_upto(network *net, char *filename, int cutoff)
                 fwrite(l.rolling_mean, sizeof(float), (size_t)l.outputs, fp);
                 fwrite(l.rolling_variance, sizeof(float), (size_t)l.outputs, fp);
             }
+            continue;
+        }
+        if (l.type == LOCAL) { /* src/parser.c:1066-1077 */
+            pull_local_layer(l);
+            fwrite(l.biases, sizeof(float), (size_t)l.outputs, fp);
+            fwrite(l.weights, sizeof(float), (size_t)l.nweights, fp);
             continue;
         }
         if (l.type != CONVOLUTIONAL) continue;

@@ -73,6 +73,8 @@ SIGNATURES = {
     "nms_sort_gpu": (None, [V, i, i, f]),
     "region_decode_gpu": (None, [V, i, i, i, i, i, i, F, i, i, i, i, i, f, V, i, V]),
     "forward_region_gpu": (None, [V, V, i, i, i, i, i, i, i, i]),
+    "forward_local_gpu": (None, [V, V, V, V, i, i, i, i, i, i, i, i, i]),
+    "detection_decode_gpu": (None, [V, i, i, i, i, i, i, f, V, i, V]),
     "num_detections": (i, [V, f]), "make_network_boxes": (V, [V, f, I]),
     "fill_network_boxes": (None, [V, i, i, f, f, I, i, V]),
     "get_network_boxes": (V, [V, i, i, f, f, I, i, I]), "free_detections": (None, [V, i]),
@@ -110,6 +112,8 @@ STRUCT_BY_VALUE = [
     "forward_connected_layer_gpu", "forward_dropout_layer_gpu", "forward_reorg_layer_gpu",
     "forward_crop_layer_gpu", "forward_cost_layer_gpu", "push_connected_layer", "pull_connected_layer",
     "make_region_layer", "forward_region_layer_gpu",
+    "make_local_layer", "forward_local_layer_gpu", "push_local_layer", "pull_local_layer",
+    "make_detection_layer", "forward_detection_layer_gpu",
     "make_image", "make_empty_image", "free_image", "resize_image", "letterbox_image", "network_predict_image",
     "network_letterbox_input",
 ]

@@ -88,9 +88,12 @@ struct layer {
     float ignore_thresh;
     float truth_thresh;
     int random;
-    int coords;        /* region */
+    int coords;        /* region, detection */
     int background;
     int softmax;
+    int side;          /* detection */
+    int sqrt;
+    int rescore;
     int flatten;       /* reorg */
     int extra;
     int noadjust;      /* crop */
@@ -211,6 +214,10 @@ layer make_crop_layer(int batch, int h, int w, int c, int crop_height, int crop_
 layer make_cost_layer(int batch, int inputs, int cost_type, float scale); /* src/cost_layer.c:40 */
 layer make_region_layer(int batch, int w, int h, int n, int classes, int coords); /* src/region_layer.c:13 */
 layer make_softmax_layer(int batch, int inputs, int groups); /* src/softmax_layer.c:11 */
+layer make_local_layer(int batch, int h, int w, int c, int n, int size, int stride, int pad,
+                       ACTIVATION activation);                 /* src/local_layer.c:26 */
+layer make_detection_layer(int batch, int inputs, int n, int side, int classes, int coords,
+                           int rescore);                       /* src/detection_layer.c:14 */
 void free_layer(layer l);                                 /* src/layer.c:6 */
 
 /* ---- per-layer GPU forwards, the function-pointer targets (include/darknet.h:122) -------- */
@@ -228,6 +235,10 @@ void forward_reorg_layer_gpu(layer l, network net);         /* src/reorg_layer.c
 void forward_crop_layer_gpu(layer l, network net);          /* src/crop_layer_kernels.cu:183 */
 void forward_cost_layer_gpu(layer l, network net);          /* src/cost_layer.c:120 (no truth: nothing) */
 void forward_region_layer_gpu(layer l, network net);        /* src/region_layer.c:439 */
+void forward_local_layer_gpu(layer l, network net);         /* src/local_layer.c:186 */
+void forward_detection_layer_gpu(layer l, network net);     /* src/detection_layer.c:256 (inference) */
+void push_local_layer(layer l);                             /* src/local_layer.c:286 */
+void pull_local_layer(layer l);                             /* src/local_layer.c:278 */
 void push_connected_layer(layer l);                         /* src/connected_layer.c:268 */
 void pull_connected_layer(layer l);                         /* src/connected_layer.c:254 */
 void push_convolutional_layer(layer l);                     /* src/convolutional_kernels.cu:286 */
@@ -265,7 +276,7 @@ float *network_predict_image(network *net, image im);      /* src/network.c:579 
 void network_letterbox_input(network *net, int b, image im);
 void network_pull_outputs(network *net);
 
-/* ---- detections (yolo and region heads; the yolov1 detection layer is outside the path) ---- */
+/* ---- detections (yolo, region and yolov1 detection heads) ---- */
 int num_detections(network *net, float thresh);                       /* src/network.c:510 */
 detection *make_network_boxes(network *net, float thresh, int *num);  /* src/network.c:526 */
 void fill_network_boxes(network *net, int w, int h, float thresh, float hier, int *map, int relative,
@@ -301,6 +312,9 @@ void network_set_fusion(int on);
 float *layer_output_host(network *net, int i);
 int *layer_indexes_host(network *net, int i);
 void network_set_verbose(int on);
+/* Overwrites layer i's parameters (host and device copies); NULL leaves a vector as it is.
+ * Convolutional: weights[nweights], biases/scales/mean/variance[n]; connected: the same with
+ * n = outputs; local: weights[nweights], biases[outputs] (the other three are ignored). */
 void network_set_conv(network *net, int i, const float *weights, const float *biases,
                       const float *scales, const float *rolling_mean,
                       const float *rolling_variance);

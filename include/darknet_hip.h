@@ -245,6 +245,16 @@ void forward_yolo_gpu(const float *input, float *output, int batch, int w, int h
 void forward_region_gpu(const float *input, float *output, int batch, int w, int h, int n_anchors,
                         int classes, int coords, int background, int softmax);
 
+/* forward_local_layer_gpu (src/local_layer.c:186-215; the CPU form :91-120 defines the result):
+ * a convolution with one [n][size*size*c] weight matrix per output location (location-major) and
+ * one bias per output element, then the activation.  `pad` is the number of zero pixels on each
+ * side, as the reference hands it to im2col, not a flag.  Output [b][n][out_h][out_w] with
+ * out_h = (h - (pad ? 1 : size))/stride + 1 (src/local_layer.c:10-24); geometries for which im2col
+ * would produce a different count end the process. */
+void forward_local_gpu(const float *input, const float *weights, const float *biases, float *output,
+                       int batch, int c, int h, int w, int n, int size, int stride, int pad,
+                       int activation);
+
 /* forward_avgpool_layer_gpu (src/avgpool_layer_kernels.cu:46-54). */
 void forward_avgpool_gpu(const float *input, float *output, int batch, int c, int h, int w);
 
@@ -297,6 +307,15 @@ void yolo_decode_gpu(const float *layer_output, int lw, int lh, int n, int class
 void region_decode_gpu(const float *layer_output, int lw, int lh, int n, int classes, int coords,
                        int background, const float *anchors, int netw, int neth, int w, int h,
                        int relative, float thresh, float *rows, int max_rows, int *count);
+
+/* The same for the yolov1 detection layer, get_detection_detections src/detection_layer.c:225-252:
+ * all side*side*n rows are written, row cell*n + box after the `*count` rows already there; the
+ * objectness column holds the box's scale whatever the threshold, the class columns
+ * scale*probability where that exceeds `thresh`, else 0.  layer_output is one image of the
+ * layer: [cells][classes] probabilities, [cells][n] scales, [cells][n][4] boxes; the box is scaled
+ * to w x h as given (no letterbox correction, as in the reference). */
+void detection_decode_gpu(const float *layer_output, int side, int n, int classes, int sqrt, int w,
+                          int h, float thresh, float *rows, int max_rows, int *count);
 
 /* do_nms_sort (src/box.c:58-89) on device rows, in place: per class, in descending
  * probability (ties: lower row first), a row zeroes that class's probability in every later row

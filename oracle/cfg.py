@@ -7,7 +7,9 @@ convolutional_out_height/width src/convolutional_layer.c:66-74; parse_maxpool :4
 make_maxpool_layer src/maxpool_layer.c:21-36; parse_route :601-640; parse_shortcut :539-556
 with make_shortcut_layer src/shortcut_layer.c:9-24; parse_upsample :592-599 with
 make_upsample_layer src/upsample_layer.c:7-29; parse_yolo :306-342 with make_yolo_layer
-src/yolo_layer.c:13-32; parse_avgpool :500-511; parse_softmax :270-283.
+src/yolo_layer.c:13-32; parse_avgpool :500-511; parse_softmax :270-283; parse_local :161-177 with
+make_local_layer src/local_layer.c:10-47; parse_detection :405-428 with make_detection_layer
+src/detection_layer.c:14-33.
 
 Pinned by tests/test_oracle_cfg.py against the layer table of the compiled reference.
 """
@@ -23,6 +25,7 @@ SECTION_ALIASES = {
     "[route]": "route", "[shortcut]": "shortcut", "[upsample]": "upsample", "[yolo]": "yolo",
     "[conn]": "connected", "[connected]": "connected", "[dropout]": "dropout", "[reorg]": "reorg",
     "[crop]": "crop", "[cost]": "cost", "[region]": "region",
+    "[local]": "local", "[detection]": "detection",
     "[net]": "net", "[network]": "net",
 }
 
@@ -153,6 +156,23 @@ def parse(text: str) -> dict:
             L["outputs"] = h * w * L["out_c"]
             if L["outputs"] != inputs:
                 raise ValueError("region layer: outputs != inputs")
+        elif kind == "local":
+            # pad is the number of zero pixels itself; the output size is the layer's own rule
+            n, size, stride, pad = gi(o, "filters", 1), gi(o, "size", 1), gi(o, "stride", 1), gi(o, "pad", 0)
+            if not (h and w and c):
+                raise ValueError("Layer before local layer must output image.")
+            oh = (h - (1 if pad else size)) // stride + 1
+            ow = (w - (1 if pad else size)) // stride + 1
+            L.update(n=n, size=size, stride=stride, pad=pad, activation=o.get("activation", "logistic"),
+                     out_h=oh, out_w=ow, out_c=n, inputs=h * w * c)
+        elif kind == "detection":
+            coords, classes, num, side = gi(o, "coords", 1), gi(o, "classes", 1), gi(o, "num", 1), gi(o, "side", 7)
+            if side * side * ((1 + coords) * num + classes) != inputs:
+                raise ValueError("detection layer: side*side*((1+coords)*num+classes) != inputs")
+            L.update(n=num, classes=classes, coords=coords, side=side, rescore=gi(o, "rescore", 0),
+                     softmax=gi(o, "softmax", 0), sqrt=gi(o, "sqrt", 0), max_boxes=gi(o, "max", 90),
+                     truths=side * side * (1 + coords + classes),
+                     h=side, w=side, c=0, out_h=0, out_w=0, out_c=0, outputs=inputs)
         elif kind == "upsample":
             stride = gi(o, "stride", 2)
             L.update(stride=stride, scale=gf(o, "scale", 1.0),

@@ -243,6 +243,39 @@ class Oracle:
         self.lib.orc_region(_fp(x), _fp(out), b, w, h, n_anchors, classes, coords, background, softmax)
         return out
 
+    def local(self, x, weights, biases, *, n, size, stride=1, pad=0, activation="logistic"):
+        """forward_local_layer on x [b, c, h, w]; pad is the number of zero pixels per side."""
+        x = np.ascontiguousarray(x, np.float32)
+        b, c, h, w = x.shape
+        oh = (h - (1 if pad else size)) // stride + 1
+        ow = (w - (1 if pad else size)) // stride + 1
+        assert (h + 2 * pad - size) // stride + 1 == oh and (w + 2 * pad - size) // stride + 1 == ow
+        wt = np.ascontiguousarray(weights, np.float32)
+        bi = np.ascontiguousarray(biases, np.float32)
+        assert wt.size == oh * ow * n * size * size * c and bi.size == oh * ow * n
+        out = np.empty((b, n, oh, ow), np.float32)
+        work = np.empty(size * size * c * oh * ow, np.float32)
+        a = ACTIVATIONS.index(activation) if isinstance(activation, str) else activation
+        self.lib.orc_local_forward(_fp(x), _fp(wt), _fp(bi), _fp(out), b, c, h, w, n, size, stride, pad, a,
+                                   _fp(work))
+        return out
+
+    def detection(self, x, side, classes, softmax=0):
+        """forward_detection_layer at inference on x [b, inputs]."""
+        x = np.ascontiguousarray(x, np.float32)
+        out = np.empty_like(x)
+        self.lib.orc_detection_forward(_fp(x), _fp(out), x.shape[0], x.shape[1], side, classes, int(softmax))
+        return out
+
+    def detection_detections(self, pred, side, n, classes, sqrt, w, h, thresh):
+        """get_detection_detections on one image's layer output -> all side*side*n rows."""
+        pred = np.ascontiguousarray(pred, np.float32).reshape(-1)
+        assert pred.size == side * side * (5 * n + classes)
+        rows = np.zeros((side * side * n, 5 + classes), np.float32)
+        self.lib.orc_detection_detections(_fp(pred), side, n, classes, int(sqrt), w, h, C.c_float(thresh),
+                                          _fp(rows))
+        return rows
+
     def region_detections(self, pred, n_anchors, classes, coords, background, biases, netw, neth, w, h, relative,
                           thresh):
         """get_region_detections on image 0 of `pred` -> all lw*lh*n rows [*, 5 + classes]."""

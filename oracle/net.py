@@ -55,6 +55,12 @@ class OracleNet:
         if t == "region":
             return o.region(x.reshape(b, L["c"], L["h"], L["w"]), L["n"], L["classes"], L["coords"],
                             L["background"], L["softmax"])
+        if t == "local":
+            w, bi = self.params[i][:2]
+            return o.local(x.reshape(b, L["c"], L["h"], L["w"]), w, bi, n=L["n"], size=L["size"],
+                           stride=L["stride"], pad=L["pad"], activation=L["activation"])
+        if t == "detection":
+            return o.detection(x.reshape(b, -1), L["side"], L["classes"], L["softmax"])
         if t == "connected":
             w, bi, sc, mu, var = self.params[i]
             return o.connected(x.reshape(b, -1), w, bi, sc, mu, var, outputs=L["outputs"],
@@ -94,6 +100,11 @@ class OracleNet:
                 rows.append(self.orc.region_detections(pred, L["n"], classes, L["coords"], L["background"],
                                                        L["anchors"], self.net["w"], self.net["h"], w, h, relative,
                                                        thresh))
+                continue
+            if L["type"] == "detection":   # src/network.c:555-558: w, h as given, no letterbox correction
+                classes = L["classes"]
+                pred = np.asarray(outs[i], np.float32).reshape(L["batch"], -1)[image]
+                rows.append(self.orc.detection_detections(pred, L["side"], L["n"], classes, L["sqrt"], w, h, thresh))
                 continue
             if L["type"] != "yolo":
                 continue

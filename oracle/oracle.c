@@ -770,3 +770,69 @@ int orc_region_detections(const float *pred, int lw, int lh, int n, int classes,
     }
     return cells * n;
 }
+
+/* ---- forward_local_layer: src/local_layer.c:91-120.  Output starts as the per-element biases
+ * (:97-99); per image one im2col (pad is the pixel count here), then for every location j a
+ * [n x K] by [K x 1] gemm on column j of the im2col buffer, accumulated into out[., j] in the
+ * reference's k order (:101-117); then the activation.  Weights are location-major.
+ * workspace: K * locations floats. -------------------------------------------------------------- */
+void orc_local_forward(const float *input, const float *weights, const float *biases, float *output, int batch,
+                       int c, int h, int w, int n, int size, int stride, int pad, int activation, float *workspace)
+{
+    const int out_h = (h - (pad ? 1 : size)) / stride + 1; /* local_out_height :10-16 */
+    const int out_w = (w - (pad ? 1 : size)) / stride + 1;
+    const int locations = out_h * out_w;
+    const int K = size * size * c;
+    const long outputs = (long)locations * n;
+    for (int b = 0; b < batch; ++b) {
+        float *out = output + b * outputs;
+        for (long i = 0; i < outputs; ++i) out[i] = biases[i];
+        orc_im2col(input + (long)b * c * h * w, c, h, w, size, stride, pad, workspace);
+        for (int j = 0; j < locations; ++j)
+            orc_gemm_nn(n, 1, K, 1.f, weights + (long)j * K * n, K, workspace + j, locations, out + j, locations);
+    }
+    orc_activate_array(output, outputs * batch, activation);
+}
+
+/* ---- forward_detection_layer at inference: src/detection_layer.c:50-66: a copy, then softmax
+ * over each cell's classes when `softmax` is set. ---------------------------------------------- */
+void orc_detection_forward(const float *input, float *output, int batch, int inputs, int side, int classes,
+                           int softmax)
+{
+    memcpy(output, input, sizeof(float) * (size_t)inputs * batch);
+    if (!softmax) return;
+    for (int b = 0; b < batch; ++b)
+        for (int i = 0; i < side * side; ++i) {
+            const long o = (long)b * inputs + (long)i * classes;
+            orc_softmax(output + o, classes, 1, 0, 1, 0, 1, 1.f, output + o);
+        }
+}
+
+/* ---- get_detection_detections: src/detection_layer.c:225-252 on image 0 of `pred`; all
+ * side*side*n rows, row cell*n + box: x, y, w, h, objectness (the box scale, whatever the
+ * threshold), prob[classes]. -------------------------------------------------------------------- */
+int orc_detection_detections(const float *pred, int side, int n, int classes, int sqrt_flag, int w, int h,
+                             float thresh, float *rows)
+{
+    for (int i = 0; i < side * side; ++i) {
+        const int row = i / side;
+        const int col = i % side;
+        for (int k = 0; k < n; ++k) {
+            const int index = i * n + k;
+            const int p_index = side * side * classes + i * n + k;
+            const float scale = pred[p_index];
+            const int box_index = side * side * (classes + n) + (i * n + k) * 4;
+            float *r = rows + (long)index * (5 + classes);
+            r[0] = (pred[box_index + 0] + col) / side * w;
+            r[1] = (pred[box_index + 1] + row) / side * h;
+            r[2] = pow(pred[box_index + 2], (sqrt_flag ? 2 : 1)) * w;
+            r[3] = pow(pred[box_index + 3], (sqrt_flag ? 2 : 1)) * h;
+            r[4] = scale;
+            for (int j = 0; j < classes; ++j) {
+                const float prob = scale * pred[i * classes + j];
+                r[5 + j] = (prob > thresh) ? prob : 0;
+            }
+        }
+    }
+    return side * side * n;
+}

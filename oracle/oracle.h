@@ -87,6 +87,13 @@ int orc_region_detections(const float *pred, int lw, int lh, int n, int classes,
                           const float *biases, int netw, int neth, int w, int h, int relative, float thresh,
                           float *rows);
 
+void orc_local_forward(const float *input, const float *weights, const float *biases, float *output, int batch,
+                       int c, int h, int w, int n, int size, int stride, int pad, int activation, float *workspace);
+void orc_detection_forward(const float *input, float *output, int batch, int inputs, int side, int classes,
+                           int softmax);
+int orc_detection_detections(const float *pred, int side, int n, int classes, int sqrt_flag, int w, int h,
+                             float thresh, float *rows);
+
 /* detections (test infrastructure like everything here): see oracle.c */
 int orc_yolo_detections(const float *pred, int lw, int lh, int n, int classes, const float *biases,
                         const int *mask, int netw, int neth, int w, int h, int relative, float thresh,

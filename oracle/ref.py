@@ -82,6 +82,7 @@ class RefNet:
         H.refh_yolo_mask.argtypes = [C.c_void_p, C.c_int, _I, C.c_int, _F, C.c_int]
         H.refh_set_conv.argtypes = [C.c_void_p, C.c_int] + [_F] * 5
         H.refh_set_connected.argtypes = [C.c_void_p, C.c_int] + [_F] * 5
+        H.refh_set_local.argtypes = [C.c_void_p, C.c_int] + [_F] * 2
         H.refh_predict.restype = _F
         H.refh_predict.argtypes = [C.c_void_p, _F]
         for f in ("refh_layer_output", "refh_layer_weights", "refh_layer_binary_weights",
@@ -125,6 +126,9 @@ class RefNet:
 
     def set_conv(self, i, weights, biases, scales=None, mean=None, var=None):
         p = lambda a: None if a is None else np.ascontiguousarray(a, np.float32).ctypes.data_as(_F)
+        if self.layers[i]["type"] == "local":
+            self.h.refh_set_local(self.net, i, p(weights), p(biases))
+            return
         f = self.h.refh_set_connected if self.layers[i]["type"] == "connected" else self.h.refh_set_conv
         f(self.net, i, p(weights), p(biases), p(scales), p(mean), p(var))
 
@@ -137,7 +141,7 @@ class RefNet:
     def get_boxes(self, w, h, thresh, relative=1, nms=0.0):
         """get_network_boxes (+ do_nms_sort when nms > 0) -> rows [n, 5 + classes]."""
         classes = self.layers[-1]["classes"]
-        cap = sum(L["w"] * L["h"] * L["n"] for L in self.layers if L["type"] in ("yolo", "region"))
+        cap = sum(L["w"] * L["h"] * L["n"] for L in self.layers if L["type"] in ("yolo", "region", "detection"))
         rows = np.zeros((max(cap, 1), 5 + classes), np.float32)
         n = self.h.refh_get_boxes(self.net, w, h, thresh, relative, nms, rows.ctypes.data_as(_F), cap)
         return rows[:n].copy()

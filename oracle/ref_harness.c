@@ -121,6 +121,16 @@ void refh_set_connected(network *net, int i, const float *weights, const float *
     }
 }
 
+/* The same for a local layer: weights[locations*n*size*size*c], biases[outputs]
+ * (src/local_layer.c:48-52; the layer does not fill in nweights). */
+void refh_set_local(network *net, int i, const float *weights, const float *biases)
+{
+    layer l = net->layers[i];
+    size_t nw = (size_t)l.c * l.n * l.size * l.size * l.out_h * l.out_w;
+    if (weights) memcpy(l.weights, weights, sizeof(float) * nw);
+    if (biases) memcpy(l.biases, biases, sizeof(float) * (size_t)l.outputs);
+}
+
 float *refh_predict(network *net, float *input)
 {
     return network_predict(net, input);

@@ -20,10 +20,12 @@ seeded synthetic inputs; nothing from the reference's sources is stored.  Fixtur
                          extra), dropout, connected (with and without batch-norm), softmax, cost
   image_cases.npz        letterbox_image / resize_image of small images (down, up, both aspects)
   region_case.npz        a yolov2-style region head (region_net.cfg): layer input/output, boxes, NMS
+  yolov1_net.weights/yolov1_case.npz  a yolov1-style tail (yolov1_net.cfg): conv, local, dropout, connected,
+                         detection; every layer's output, the saved weights file, boxes, NMS
   detections_case.npz    the two yolo tensors of a yolov3-tiny forward at 96x96 and what
                          get_network_boxes / do_nms_sort make of them (rows x,y,w,h,obj,prob[80])
 
-`python tests/golden/make_golden.py detections|small_net2|images|region` rewrites only that fixture.
+`python tests/golden/make_golden.py detections|small_net2|images|region|yolov1` rewrites only that fixture.
 """
 import json
 import os
@@ -233,6 +235,39 @@ def region_fixture():
     np.savez_compressed(os.path.join(HERE, "region_case.npz"), **data)
 
 
+YOLOV1_CASES = {"square": (90, 90, 0.05, 1, 0.0), "wide": (200, 120, 0.1, 0, 0.0), "wide_nms": (200, 120, 0.05, 0, 0.4)}
+
+
+def yolov1_fixture():
+    """A yolov1-style tail (yolov1_net.cfg, written by hand next to this script): conv -> local ->
+    dropout -> connected -> detection.  Every layer's output, the weights file the reference saves
+    (it holds a local layer's block), the detection output with softmax=1, and what
+    get_network_boxes / do_nms_sort make of the head."""
+    path = os.path.join(HERE, "yolov1_net.cfg")
+    r = ref.RefNet(path)
+    fill_params(r.set_conv, r.layers, seed=77, bn="random")
+    import ctypes as C
+    lib = ref.raw()
+    lib.save_weights.argtypes = [C.c_void_p, C.c_char_p]
+    lib.save_weights(r.net, os.path.join(HERE, "yolov1_net.weights").encode())
+    x = synth.uniform01(5, r.inputs * r.batch)
+    outs = r.predict(x)
+    data = {"input": x}
+    data.update({f"layer{i}": o for i, o in enumerate(outs)})
+    for name, (w, h, thresh, relative, nms) in YOLOV1_CASES.items():
+        rows = r.get_boxes(w, h, thresh, relative, nms)
+        data[name] = rows if nms == 0 else lexsorted(rows[rows[:, 4] > 0])
+        data[name + "_spec"] = np.array([w, h, thresh, relative, nms], np.float64)
+    table_rows = [{k: L[k] for k in KEYS + ["truths", "max_boxes"] if k in L} for L in r.layers]
+    p = write_cfg(open(path).read().replace("softmax=0", "softmax=1"))
+    r2 = ref.RefNet(p)
+    os.unlink(p)
+    fill_params(r2.set_conv, r2.layers, seed=77, bn="random")
+    data["softmax_out"] = r2.predict(x)[-1]
+    np.savez_compressed(os.path.join(HERE, "yolov1_case.npz"), **data)
+    return table_rows
+
+
 def lexsorted(rows):
     """Rows in a canonical order (the reference leaves its array sorted by the last class after NMS)."""
     if len(rows) == 0:
@@ -268,6 +303,12 @@ def main():
         region_fixture()
         print("region_case.npz written")
         return
+    if sys.argv[1:] == ["yolov1"]:
+        tables = json.load(open(os.path.join(HERE, "layer_tables.json")))
+        tables["yolov1_net"] = yolov1_fixture()
+        json.dump(tables, open(os.path.join(HERE, "layer_tables.json"), "w"), indent=0)
+        print("yolov1 fixtures written")
+        return
     if sys.argv[1:] == ["images"]:
         images_fixture()
         print("image_cases.npz written")
@@ -287,6 +328,7 @@ def main():
                        ("resnext50-224", cfgs.resnext50(1, 224)), ("small_net", SMALL_NET)]:
         _, tables[name] = table(text)
     tables["small_net2"] = small_net2_fixture()
+    tables["yolov1_net"] = yolov1_fixture()
     json.dump(tables, open(os.path.join(HERE, "layer_tables.json"), "w"), indent=0)
 
     # ---- yolov3-tiny forward checksums

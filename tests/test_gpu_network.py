@@ -23,8 +23,12 @@ EXACT_GIVEN_INPUT = ("maxpool", "route", "upsample", "shortcut")
 def build_pair(text, seed=1000, bn="random"):
     net = api.Network(cfg_text=text)
     orc = OracleNet(text)
-    fill_params(net.set_conv, net.layers, seed=seed, bn=bn)
-    fill_params(orc.set_conv, orc.layers, seed=seed, bn=bn)
+    def both(i, *arrays):            # one pass of the generator feeds both networks
+        net.set_conv(i, *arrays)
+        orc.set_conv(i, *arrays)
+
+    assert [(L["type"], L["outputs"]) for L in net.layers] == [(L["type"], L["outputs"]) for L in orc.layers]
+    fill_params(both, orc.layers, seed=seed, bn=bn)
     return net, orc
 
 

@@ -50,7 +50,9 @@ def same_table(want, got, where):
                                        ("yolov3-416", cfgs.yolov3(1, 416)),
                                        ("resnext50-224", cfgs.resnext50(1, 224)),
                                        ("small_net", open(os.path.join(GOLD, "small_net.cfg")).read()),
-                                       ("small_net2", open(os.path.join(GOLD, "small_net2.cfg")).read())])
+                                       ("small_net2", open(os.path.join(GOLD, "small_net2.cfg")).read()),
+                                       ("yolov1_net", open(os.path.join(GOLD, "yolov1_net.cfg")).read())],
+                         ids=["yolov3-tiny-416", "yolov3-416", "resnext50-224", "small_net", "small_net2", "yolov1_net"])
 def test_library_parser_matches_golden_layer_tables(parse_only, name, text):
     gold = json.load(open(os.path.join(GOLD, "layer_tables.json")))[name]
     net = api.Network(cfg_text=text)
@@ -88,7 +90,7 @@ def test_library_parses_every_in_scope_reference_cfg(parse_only):
         same_table(want, net.layers, os.path.basename(path))
         net.free()
         done += 1
-    assert done >= 37
+    assert done >= 40
 
 
 def test_weights_file_round_trip_on_the_host(parse_only, tmp_path):
@@ -104,6 +106,11 @@ def test_weights_file_round_trip_on_the_host(parse_only, tmp_path):
     net = api.Network(cfg_path=os.path.join(GOLD, "small_net2.cfg"), weights=src2)
     net.save_weights(out)
     assert open(out, "rb").read() == open(src2, "rb").read()
+    net.free()
+    src3 = os.path.join(GOLD, "yolov1_net.weights")     # a local layer's block: biases per output, weights per location
+    net = api.Network(cfg_path=os.path.join(GOLD, "yolov1_net.cfg"), weights=src3)
+    net.save_weights(out)
+    assert open(out, "rb").read() == open(src3, "rb").read()
     net.free()
 
 

@@ -39,6 +39,7 @@ def test_host_code_under_address_and_ub_sanitizers(tmp_path):
     again = str(tmp_path / "again.weights")
     cases = [os.path.join(GOLD, "small_net2.cfg") + "@" + os.path.join(GOLD, "small_net2.weights"),
              os.path.join(GOLD, "region_net.cfg"),
+             os.path.join(GOLD, "yolov1_net.cfg") + "@" + os.path.join(GOLD, "yolov1_net.weights"),
              os.path.join(GOLD, "small_net.cfg") + "@" + os.path.join(GOLD, "small_net.weights")]
     if have_reference_tree():
         for path in sorted(glob.glob("/root/reference/cfg/*.cfg")):

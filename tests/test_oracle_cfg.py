@@ -28,6 +28,8 @@ PER_TYPE = {
     "upsample": ["stride", "scale"],
     "yolo": ["classes", "total", "mask", "n"],
     "softmax": ["groups", "temperature"],
+    "local": ["n", "size", "stride", "pad", "activation"],
+    "detection": ["n", "classes", "truths", "max_boxes"],
 }
 
 
@@ -42,7 +44,9 @@ def same_table(a, b, where=""):
                                        ("yolov3-416", cfgs.yolov3(1, 416)),
                                        ("resnext50-224", cfgs.resnext50(1, 224)),
                                        ("small_net", open(os.path.join(GOLD, "small_net.cfg")).read()),
-                                       ("small_net2", open(os.path.join(GOLD, "small_net2.cfg")).read())])
+                                       ("small_net2", open(os.path.join(GOLD, "small_net2.cfg")).read()),
+                                       ("yolov1_net", open(os.path.join(GOLD, "yolov1_net.cfg")).read())],
+                         ids=["yolov3-tiny-416", "yolov3-416", "resnext50-224", "small_net", "small_net2", "yolov1_net"])
 def test_parser_matches_golden_layer_tables(name, text):
     gold = json.load(open(os.path.join(GOLD, "layer_tables.json")))[name]
     same_table(gold, ocfg.parse(text)["layers"], name)
@@ -81,7 +85,8 @@ def test_generated_cfgs_equal_the_reference_files():
         return re.sub(r"(?m)^height\s*=.*$", f"height={size}", t)
 
     for name, gen, size in [("yolov3-tiny", cfgs.yolov3_tiny, 416), ("yolov3", cfgs.yolov3, 608),
-                            ("resnext50", cfgs.resnext50, 256)]:
+                            ("resnext50", cfgs.resnext50, 256), ("yolov1-tiny", cfgs.yolov1_tiny, 448),
+                            ("yolov1", cfgs.yolov1, 448)]:
         p1 = write_cfg(edit(open(f"/root/reference/cfg/{name}.cfg").read(), 2, size))
         p2 = write_cfg(gen(2, size))
         a, b = ref.RefNet(p1).layers, ref.RefNet(p2).layers
