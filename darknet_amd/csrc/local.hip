@@ -156,7 +156,13 @@ __global__ __launch_bounds__(LC_THREADS, 4) void local_kernel(local_args a, int 
 
 static float *g_patches = 0; /* patches of the current call, grown on demand and kept */
 static size_t g_patches_floats = 0;
-#define LC_MAX_PATCH_FLOATS (1L << 28) /* 1 GiB: larger batches run in slices of images */
+static long g_patch_budget = 1L << 28; /* floats (1 GiB): larger batches run in slices of images */
+
+extern "C" void local_set_patch_budget(long floats)
+{
+    if (floats < 1) dn_fatal("local_set_patch_budget: the budget must be positive");
+    g_patch_budget = floats;
+}
 
 /* The reference sizes its output with local_out_height / _width (src/local_layer.c:10-24: h - size
  * without padding, h - 1 with it) but fills its column buffer with im2col_cpu, whose own count is
@@ -178,8 +184,8 @@ extern "C" void forward_local_gpu(const float *input, const float *weights, cons
     if ((long)c * size * size >= (1L << 31) || (long)oh * ow > 0x7fffffffL) dn_fatal("forward_local_gpu: too large");
     const long K = (long)c * size * size;
     const long per_image = (long)oh * ow * K;
-    if (per_image > LC_MAX_PATCH_FLOATS) dn_fatal("forward_local_gpu: one image's patches exceed the work buffer");
-    const int slice = (int)(LC_MAX_PATCH_FLOATS / per_image < batch ? LC_MAX_PATCH_FLOATS / per_image : batch);
+    if (per_image > g_patch_budget) dn_fatal("forward_local_gpu: one image's patches exceed the work buffer's budget");
+    const int slice = (int)(g_patch_budget / per_image < batch ? g_patch_budget / per_image : batch);
     const size_t need = (size_t)per_image * slice;
     if (need > g_patches_floats) {
         if (g_patches) hip_free(g_patches);

@@ -255,6 +255,12 @@ void forward_local_gpu(const float *input, const float *weights, const float *bi
                        int batch, int c, int h, int w, int n, int size, int stride, int pad,
                        int activation);
 
+/* forward_local_gpu gathers its patches into a library-owned device buffer of batch * out_h * out_w *
+ * size*size*c floats, grown on demand and kept; beyond this budget (default 2^28 floats = 1 GiB) a
+ * batch runs in slices of images, with the same result.  No counterpart in the reference, which
+ * keeps one image's im2col in net.workspace. */
+void local_set_patch_budget(long floats);
+
 /* forward_avgpool_layer_gpu (src/avgpool_layer_kernels.cu:46-54). */
 void forward_avgpool_gpu(const float *input, float *output, int batch, int c, int h, int w);
 

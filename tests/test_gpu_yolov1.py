@@ -58,6 +58,23 @@ def test_local_layer_against_checker(dn, orc, batch, c, h, w, n, size, stride, p
     assert np.array_equal(out.numpy((want.size + 64,)), got)         # same bits from run to run
 
 
+def test_local_layer_in_image_slices_changes_no_bit(dn):
+    """A patch budget of two images' worth: a batch of five runs as 2 + 2 + 1."""
+    batch, c, h, w, n, size = 5, 6, 5, 4, 7, 3
+    x = synth.uniform(41, batch * c * h * w, -1, 1)
+    wt = synth.conv_weights(42, h * w * n, c, size)
+    bias = synth.uniform(43, h * w * n, -0.5, 0.5)
+    dx, dw, db = D(x), D(wt), D(bias)
+    outs = []
+    for budget in (1 << 28, 2 * h * w * c * size * size):
+        dn.local_set_patch_budget(budget)
+        out = D(n=batch * n * h * w)
+        dn.forward_local_gpu(dx.ptr, dw.ptr, db.ptr, out.ptr, batch, c, h, w, n, size, 1, 1, ACTIVATIONS.index("leaky"))
+        outs.append(out.numpy())
+    dn.local_set_patch_budget(1 << 28)
+    assert np.array_equal(outs[0], outs[1]) and np.abs(outs[0]).max() > 0.1
+
+
 def test_yolov1_network_on_the_reference_weights_file_and_golden_vectors(dn, tmp_path):
     g = np.load(os.path.join(GOLD, "yolov1_case.npz"))
     src = os.path.join(GOLD, "yolov1_net.weights")
