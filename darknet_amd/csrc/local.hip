@@ -55,19 +55,19 @@ __global__ void local_patches_kernel(local_args a, float *patches)
     }
 }
 
-/* Step 2.  A workgroup owns one location, 16 filters and 16 images; four waves, 4 filters each,
- * lanes along k.  Per chunk of 256 values of k the 16 patches are copied into LDS and every
- * weight that arrives from memory is used for all 16 images.  Both sets of loads of a chunk are
+/* Step 2.  A workgroup owns one location, 4*FW filters and NB images; four waves, FW filters each,
+ * lanes along k.  Per chunk of KC values of k the NB patches are copied into LDS and every
+ * weight that arrives from memory is used for all NB images (local layer: 16 images, 4 filters
+ * per wave, chunks of 256).  Both sets of loads of a chunk are
  * issued before the first barrier, so a chunk costs one memory round trip, which the other
  * workgroups of the CU fill with their arithmetic.  Image groups of one (location, filters) pair
  * are neighbours in the grid, so their common weights are fetched from HBM once and served to the
  * other groups by the memory-side cache. */
-#define LC_FW 4
-#define LC_NB 16
-#define LC_KC 256
+template <int LC_NB, int LC_FW, int LC_KC>
 __global__ __launch_bounds__(LC_THREADS, 4) void local_kernel(local_args a, int image_groups)
 {
-    static_assert(LC_NB * LC_FW == 64, "one lane per (filter, image) pair in the final reduction");
+    static_assert(LC_NB * LC_FW <= 64, "one lane per (filter, image) pair in the final reduction");
+    static_assert(LC_KC % LC_THREADS == 0, "every thread copies the same number of patch columns");
     __shared__ float tile[LC_NB][LC_KC];
     const int j = blockIdx.x / image_groups;
     const int b0 = (blockIdx.x - j * image_groups) * LC_NB;
@@ -96,7 +96,7 @@ __global__ __launch_bounds__(LC_THREADS, 4) void local_kernel(local_args a, int 
     for (int step = 0; step < nchunks; ++step) {
         const int chunk = step + rot < nchunks ? step + rot : step + rot - nchunks;
         const int k0 = chunk * LC_KC;
-        /* the chunk's weights (4 per filter and lane); past the end of K the patch is zero in LDS,
+        /* the chunk's weights (KC/64 per filter and lane); past the end of K the patch is zero in LDS,
          * the weight is read from a clamped address and replaced by zero */
         float wv[LC_KC / 64][LC_FW];
 #pragma unroll
@@ -109,7 +109,7 @@ __global__ __launch_bounds__(LC_THREADS, 4) void local_kernel(local_args a, int 
                 wv[t][i] = k < a.K ? v : 0.f;
             }
         }
-        /* the chunk's patches: thread t copies column t of each image's row */
+        /* the chunk's patches: thread t copies columns t, t+256, ... of each image's row */
         float pv[LC_KC / LC_THREADS][LC_NB];
 #pragma unroll
         for (int h = 0; h < LC_KC / LC_THREADS; ++h) {
@@ -148,7 +148,7 @@ __global__ __launch_bounds__(LC_THREADS, 4) void local_kernel(local_args a, int 
         }
     const int f = f0 + lane / LC_NB;
     const int b = b0 + lane % LC_NB;
-    if (f < a.n && b < a.batch) {
+    if (lane < LC_NB * LC_FW && f < a.n && b < a.batch) {
         const long o = ((long)b * a.n + f) * locations + j;
         a.out[o] = dn_activate(a.biases[(long)f * locations + j] + mine, a.act);
     }
@@ -215,12 +215,47 @@ extern "C" void forward_local_gpu(const float *input, const float *weights, cons
         const long pb = (total + 255) / 256;
         hipLaunchKernelGGL(local_patches_kernel, dim3((unsigned)(pb > 65536 ? 65536 : pb)), dim3(256), 0, dn_stream(), a,
                            g_patches);
-        const int fpb = LC_THREADS / 64 * LC_FW;
-        const int groups = (a.batch + LC_NB - 1) / LC_NB;
+        const int fpb = LC_THREADS / 64 * 4;
+        const int groups = (a.batch + 15) / 16;
         if ((long)oh * ow * groups > 0x7fffffffL) dn_fatal("forward_local_gpu: too many locations x images for one launch");
         dim3 grid((unsigned)(oh * ow * groups), (unsigned)((n + fpb - 1) / fpb));
         if (grid.y > 65535u) dn_fatal("forward_local_gpu: too many filters for one launch");
-        hipLaunchKernelGGL(local_kernel, grid, dim3(LC_THREADS), 0, dn_stream(), a, groups);
+        hipLaunchKernelGGL((local_kernel<16, 4, 256>), grid, dim3(LC_THREADS), 0, dn_stream(), a, groups);
     }
     dn_check_launch("forward_local_gpu");
+}
+
+/* A connected layer without batch-norm at a small batch is the same weight stream with a single
+ * location whose "patches" are the layer's input rows themselves: forward_connected_layer
+ * (src/connected_layer.c:140-167: gemm, add_bias, activate) as one pass over the weights.  One
+ * filter per wave keeps outputs/4 workgroups in flight (1024 for a 4096-wide layer); up to 4 images
+ * share a weight in registers, up to 16 through the wider tile. */
+extern "C" void forward_connected_stream_gpu(const float *input, const float *weights, const float *biases,
+                                             float *output, int batch, int inputs, int outputs, int activation)
+{
+    if (batch < 1 || inputs < 1 || outputs < 1) dn_fatal("forward_connected_stream_gpu: bad geometry");
+    if (activation < 0 || activation > DN_SELU) dn_fatal("forward_connected_stream_gpu: unknown activation");
+    local_args a;
+    a.in = input;
+    a.patches = input;
+    a.weights = weights;
+    a.biases = biases;
+    a.out = output;
+    a.batch = batch;
+    a.c = inputs;
+    a.h = a.w = a.size = a.stride = a.oh = a.ow = 1;
+    a.pad = 0;
+    a.n = outputs;
+    a.K = inputs;
+    a.act = activation;
+    const int nb = batch <= 4 ? 4 : 16;
+    const int fpb = LC_THREADS / 64 * (nb == 4 ? 1 : 2);
+    const int groups = (batch + nb - 1) / nb;
+    dim3 grid((unsigned)groups, (unsigned)((outputs + fpb - 1) / fpb));
+    if (grid.y > 65535u) dn_fatal("forward_connected_stream_gpu: too many outputs for one launch");
+    if (nb == 4)
+        hipLaunchKernelGGL((local_kernel<4, 1, 1024>), grid, dim3(LC_THREADS), 0, dn_stream(), a, groups);
+    else
+        hipLaunchKernelGGL((local_kernel<16, 2, 512>), grid, dim3(LC_THREADS), 0, dn_stream(), a, groups);
+    dn_check_launch("forward_connected_stream_gpu");
 }

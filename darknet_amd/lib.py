@@ -75,6 +75,7 @@ SIGNATURES = {
     "forward_region_gpu": (None, [V, V, i, i, i, i, i, i, i, i]),
     "forward_local_gpu": (None, [V, V, V, V, i, i, i, i, i, i, i, i, i]),
     "local_set_patch_budget": (None, [C.c_long]),
+    "forward_connected_stream_gpu": (None, [V, V, V, V, i, i, i, i]),
     "detection_decode_gpu": (None, [V, i, i, i, i, i, i, f, V, i, V]),
     "num_detections": (i, [V, f]), "make_network_boxes": (V, [V, f, I]),
     "fill_network_boxes": (None, [V, i, i, f, f, I, i, V]),

@@ -261,6 +261,13 @@ void forward_local_gpu(const float *input, const float *weights, const float *bi
  * keeps one image's im2col in net.workspace. */
 void local_set_patch_budget(long floats);
 
+/* forward_connected_layer_gpu without batch-norm (src/connected_layer.c:286-303; the CPU form
+ * :140-167 defines the result) as one streaming pass over the weights [outputs][inputs]: the form
+ * for small batches, where the layer is bound by reading its weights once.  Any batch is accepted;
+ * above 16 images the weights are read once per 16. */
+void forward_connected_stream_gpu(const float *input, const float *weights, const float *biases,
+                                  float *output, int batch, int inputs, int outputs, int activation);
+
 /* forward_avgpool_layer_gpu (src/avgpool_layer_kernels.cu:46-54). */
 void forward_avgpool_gpu(const float *input, float *output, int batch, int c, int h, int w);
 

@@ -163,3 +163,44 @@ def test_yolov1_448_with_its_local_layer(dn):
     from test_gpu_network import check_network
     from darknet_amd import cfgs
     assert check_network(cfgs.yolov1(1, 448)) <= REL_TOL
+
+
+STREAM_CASES = [  # batch, inputs, outputs, activation
+    (1, 9216, 1000, "relu"),        # K a multiple of both chunk widths, ragged filter tile
+    (3, 1000, 37, "linear"),        # ragged K: the last chunk is partial
+    (4, 2500, 256, "leaky"),
+    (5, 777, 130, "logistic"),      # the 16-image tile, ragged everything
+    (16, 4096, 64, "leaky"),
+    (17, 1030, 9, "linear"),        # two image groups, the second with one image
+]
+
+
+@pytest.mark.parametrize("batch,inputs,outputs,act", STREAM_CASES, ids=["b%d_%d_%d" % t[:3] for t in STREAM_CASES])
+def test_connected_stream_against_checker(dn, orc, batch, inputs, outputs, act):
+    x = synth.uniform(51, batch * inputs, -1, 1).reshape(batch, inputs)
+    wt = synth.conv_weights(52, outputs, inputs, 1)
+    bias = synth.uniform(53, outputs, -0.5, 0.5)
+    want = orc.connected(x, wt, bias, outputs=outputs, batch_normalize=0, activation=act)
+    guard = np.full(want.size + 64, 7.5, np.float32)
+    dx, dw, db, out = D(x), D(wt), D(bias), D(guard)
+    dn.forward_connected_stream_gpu(dx.ptr, dw.ptr, db.ptr, out.ptr, batch, inputs, outputs, ACTIVATIONS.index(act))
+    got = out.numpy()
+    assert np.array_equal(got[want.size:], guard[want.size:])
+    assert norm_err(got[:want.size], want.reshape(-1)) <= REL_TOL
+
+
+def test_connected_layer_takes_the_streaming_kernel_at_small_batches(dn):
+    """The layer-level call: batch 2 (streaming kernel) and batch 32 (matrix cores) of the same
+    head agree with the checker; with batch-norm the tiled kernel serves every batch."""
+    from test_gpu_network import build_pair
+    for batch in (2, 32):
+        text = (f"[net]\nbatch={batch}\nsubdivisions=1\nwidth=4\nheight=4\nchannels=64\n"
+                "[connected]\noutput=300\nactivation=leaky\n"
+                "[connected]\noutput=50\nbatch_normalize=1\nactivation=linear\n")
+        net, onet = build_pair(text, seed=61)
+        x = synth.uniform(6, net.inputs * net.batch, -1, 1)
+        net.predict(x)
+        want = onet.forward(x)
+        for i in range(net.n):
+            assert norm_err(net.layer_output(i), want[i]) <= REL_TOL, (batch, i)
+        net.free()
