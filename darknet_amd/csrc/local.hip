@@ -215,12 +215,16 @@ extern "C" void forward_local_gpu(const float *input, const float *weights, cons
         const long pb = (total + 255) / 256;
         hipLaunchKernelGGL(local_patches_kernel, dim3((unsigned)(pb > 65536 ? 65536 : pb)), dim3(256), 0, dn_stream(), a,
                            g_patches);
-        const int fpb = LC_THREADS / 64 * 4;
-        const int groups = (a.batch + 15) / 16;
+        const bool few = a.batch <= 4; /* one filter per wave, 4 images, 1024-wide chunks: more bytes in flight */
+        const int fpb = LC_THREADS / 64 * (few ? 1 : 4);
+        const int groups = few ? 1 : (a.batch + 15) / 16;
         if ((long)oh * ow * groups > 0x7fffffffL) dn_fatal("forward_local_gpu: too many locations x images for one launch");
         dim3 grid((unsigned)(oh * ow * groups), (unsigned)((n + fpb - 1) / fpb));
         if (grid.y > 65535u) dn_fatal("forward_local_gpu: too many filters for one launch");
-        hipLaunchKernelGGL((local_kernel<16, 4, 256>), grid, dim3(LC_THREADS), 0, dn_stream(), a, groups);
+        if (few)
+            hipLaunchKernelGGL((local_kernel<4, 1, 1024>), grid, dim3(LC_THREADS), 0, dn_stream(), a, groups);
+        else
+            hipLaunchKernelGGL((local_kernel<16, 4, 256>), grid, dim3(LC_THREADS), 0, dn_stream(), a, groups);
     }
     dn_check_launch("forward_local_gpu");
 }
