@@ -8,9 +8,11 @@
  * output element (src/local_layer.c:98).  With every weight used once per image the layer streams
  * its weights from HBM (462 MB for yolov1's 7x7x256 layer on 3x3x1024 patches), so the kernel is
  * laid out around that stream: the patches of every location are gathered once into a work
- * buffer; a workgroup then owns one location, 16 filters and 16 images, copies the patches
- * into LDS chunk by chunk of k, and uses every weight that arrives for all 16 images.
- * Lanes run along k, so a wave's weight loads are contiguous rows.
+ * buffer; a workgroup then owns one location, 16 filters and 16 images (4 filters and 4 images
+ * for batches up to 4), copies the patches into LDS chunk by chunk of k, and uses every weight
+ * that arrives for all its images.  Lanes run along k, so a wave's weight loads are contiguous
+ * rows.  A connected layer at a small batch is the one-location case of the same stream
+ * (forward_connected_stream_gpu below).
  * Sums are formed in a fixed order (per lane along k, then a butterfly over the lanes), so
  * the result is the same from run to run.
  */
@@ -57,8 +59,8 @@ __global__ void local_patches_kernel(local_args a, float *patches)
 
 /* Step 2.  A workgroup owns one location, 4*FW filters and NB images; four waves, FW filters each,
  * lanes along k.  Per chunk of KC values of k the NB patches are copied into LDS and every
- * weight that arrives from memory is used for all NB images (local layer: 16 images, 4 filters
- * per wave, chunks of 256).  Both sets of loads of a chunk are
+ * weight that arrives from memory is used for all NB images (16 images, 4 filters per wave and
+ * chunks of 256; 4 images, 1 filter per wave and chunks of 1024 for small batches).  Both sets of loads of a chunk are
  * issued before the first barrier, so a chunk costs one memory round trip, which the other
  * workgroups of the CU fill with their arithmetic.  Image groups of one (location, filters) pair
  * are neighbours in the grid, so their common weights are fetched from HBM once and served to the
