@@ -1145,6 +1145,61 @@ static float *g_partial = 0; /* K-slice accumulators of tail tiles, grown on dem
 static size_t g_partial_floats = 0;
 static int g_cus = 0;
 
+/* ---- allocation-free calls ----------------------------------------------------------------
+ * forward_convolutional_noalloc_gpu serves callers that cannot allocate device memory (stream
+ * capture, tight serving loops).  The only device memory a packed-weights fp32 call needs beyond
+ * its operands is the K-slice accumulator buffer above; for these calls it is a fixed array in
+ * the code object.  `scratch` is the host-side handle of that array, not an address: host code
+ * uses the per-device pointer hipGetSymbolAddress returns (every device holds its own copy). */
+#define DN_NOALLOC_SCRATCH_FLOATS ((size_t)16 << 20) /* 64 MiB */
+#define DN_MAX_DEVICES 16
+static __device__ __align__(256) float scratch[DN_NOALLOC_SCRATCH_FLOATS];
+static float *g_scratch_dev[DN_MAX_DEVICES];
+static int g_cus_dev[DN_MAX_DEVICES];
+static int g_noalloc = 0;       /* inside forward_convolutional_noalloc_gpu */
+static int g_noalloc_error = 0; /* set instead of allocating (or launching) by the paths below */
+
+/* Once per device, with that device current: address of its copy of `scratch`, CU count. */
+extern "C" __attribute__((visibility("hidden"))) void conv_device_setup(void)
+{
+    if (hip_parse_only()) return;
+    const int dev = hip_get_device();
+    if (dev < 0 || dev >= DN_MAX_DEVICES) dn_fatal("conv_device_setup: device index out of range");
+    if (!g_scratch_dev[dev]) {
+        float *ptr = 0;
+        hip_check_error(hipGetSymbolAddress((void **)&ptr, HIP_SYMBOL(scratch)));
+        if (!ptr) dn_fatal("conv_device_setup: hipGetSymbolAddress returned a null pointer");
+        g_scratch_dev[dev] = ptr;
+    }
+    if (!g_cus_dev[dev]) {
+        hipDeviceProp_t prop;
+        hip_check_error(hipGetDeviceProperties(&prop, dev));
+        g_cus_dev[dev] = prop.multiProcessorCount;
+    }
+}
+
+/* The K-slice accumulator buffer for `need` floats: the growing allocation, or in an
+ * allocation-free call the current device's fixed array (null when it is too small). */
+static float *partial_buffer(size_t need)
+{
+    if (g_noalloc) {
+        if (need > DN_NOALLOC_SCRATCH_FLOATS) {
+            fprintf(stderr,
+                    "forward_convolutional_noalloc_gpu: this geometry needs %zu bytes of K-split scratch, the fixed "
+                    "buffer holds %zu\n", need * sizeof(float), DN_NOALLOC_SCRATCH_FLOATS * sizeof(float));
+            g_noalloc_error = 1;
+            return 0;
+        }
+        return g_scratch_dev[hip_get_device()];
+    }
+    if (need > g_partial_floats) {
+        if (g_partial) hip_free(g_partial);
+        g_partial = hip_make_array(0, need);
+        g_partial_floats = need;
+    }
+    return g_partial;
+}
+
 /* How to cover `tiles` equal tiles on `cus` compute units.  Whole tiles are dealt out in rounds;
  * a remainder that would leave most CUs idle for a whole tile time (or, at batch 1, a grid far
  * smaller than the chip) is cut along K into `split` slices each, reduced afterwards.
@@ -1188,10 +1243,11 @@ static void launch_tile(const mfma_args &a0, int mode)
     a.tiles_m = (a.M + BM - 1) / BM;
     a.tiles_n = (int)((a.Ntotal + BN - 1) / BN);
     const long total = (long)a.tiles_m * a.tiles_n;
-    if (!g_cus) {
-        hipDeviceProp_t prop;
-        hip_check_error(hipGetDeviceProperties(&prop, hip_get_device()));
-        g_cus = prop.multiProcessorCount;
+    {
+        const int dev = hip_get_device();
+        if (dev < 0 || dev >= DN_MAX_DEVICES) dn_fatal("conv dispatch: device index out of range");
+        if (!g_cus_dev[dev]) conv_device_setup();
+        g_cus = g_cus_dev[dev];
     }
     int split = 1;
     /* a bf16 chunk takes a small fraction of an fp32 chunk's time; the fixed costs do not shrink */
@@ -1204,13 +1260,8 @@ static void launch_tile(const mfma_args &a0, int mode)
     a.per_xcd = (int)((whole + 7) / 8);
     a.partial = 0;
     if (tail > 0) {
-        const size_t need = (size_t)tail * split * BM * BN;
-        if (need > g_partial_floats) {
-            if (g_partial) hip_free(g_partial);
-            g_partial = hip_make_array(0, need);
-            g_partial_floats = need;
-        }
-        a.partial = g_partial;
+        a.partial = partial_buffer((size_t)tail * split * BM * BN);
+        if (!a.partial) return; /* allocation-free call and the fixed buffer is too small: nothing is launched */
     }
     const dim3 grid((unsigned)(a.per_xcd * 8 + tail * split));
     if (BM > 128 && !bf16) dn_fatal("conv dispatch: the 256-row tile is only built for the bf16-operand mode");
@@ -1321,6 +1372,7 @@ static void conv_forward(const float *input, const float *weights, const float *
                 conv_forward(input + b0 * (in_img / 4), weights, packed, biases, scales, rolling_mean, rolling_variance,
                              output + b0 * out_img, nb, c, h, w, n, groups, size, stride, pad, batch_normalize,
                              activation, add ? add + b0 * out_img : 0, sum ? sum + b0 * out_img : 0, s1, s2, sum_act);
+                if (g_noalloc_error) return;
             }
             return;
         }
@@ -1345,11 +1397,20 @@ static void conv_forward(const float *input, const float *weights, const float *
          * sequence of passes (activate_array, src/convolutional_layer.c:478; shortcut) */
         conv_forward(input, weights, packed, biases, scales, rolling_mean, rolling_variance, output, batch, c, h,
                      w, n, groups, size, stride, pad, batch_normalize, DN_LINEAR, 0, 0, 0.f, 0.f, DN_LINEAR);
+        if (g_noalloc_error) return;
         dn_activate_array(output, (long)batch * n * oh * ow, activation);
         if (sum) forward_shortcut_gpu(output, add, sum, batch, ow, oh, n, ow, oh, n, s1, s2, sum_act);
         return;
     }
 
+    if (g_noalloc && (!packed || (g_precision == 1 && mode == 13))) {
+        fprintf(stderr, !packed ? "forward_convolutional_noalloc_gpu: this geometry runs on packed weights; pass the "
+                                  "buffer conv_pack_weights_gpu wrote\n"
+                                : "forward_convolutional_noalloc_gpu: the bf16-operand mode stages 3x3 inputs in a "
+                                  "buffer it allocates; use conv_set_precision(0) or (2)\n");
+        g_noalloc_error = 1;
+        return;
+    }
     if (!packed) {
         const size_t need = conv_packed_floats(n, c, groups, size);
         if (need > g_scratch_floats) {
@@ -1465,4 +1526,23 @@ extern "C" void forward_convolutional_shortcut_gpu(const float *input, const flo
     conv_forward(input, weights, packed, biases, scales, rolling_mean, rolling_variance, output, batch, c, h, w,
                  n, groups, size, stride, pad, batch_normalize, activation, add, sum_output, alpha, beta,
                  shortcut_activation);
+}
+
+extern "C" int forward_convolutional_noalloc_gpu(const float *input, const float *weights, const float *packed,
+                                                 const float *biases, const float *scales,
+                                                 const float *rolling_mean, const float *rolling_variance,
+                                                 float *output, int batch, int c, int h, int w, int n,
+                                                 int groups, int size, int stride, int pad,
+                                                 int batch_normalize, int activation)
+{
+    hip_require_device("forward_convolutional_noalloc_gpu");
+    const int dev = hip_get_device();
+    if (dev < 0 || dev >= DN_MAX_DEVICES) dn_fatal("forward_convolutional_noalloc_gpu: device index out of range");
+    if (!g_scratch_dev[dev] || !g_cus_dev[dev]) conv_device_setup(); /* first call on this device */
+    g_noalloc = 1;
+    g_noalloc_error = 0;
+    conv_forward(input, weights, packed, biases, scales, rolling_mean, rolling_variance, output, batch, c, h, w,
+                 n, groups, size, stride, pad, batch_normalize, activation, 0, 0, 0.f, 0.f, DN_LINEAR);
+    g_noalloc = 0;
+    return g_noalloc_error ? -1 : 0;
 }

@@ -65,11 +65,16 @@ void hip_require_device(const char *what)
     }
 }
 
+/* conv_mfma.hip: per-device set-up of the convolution dispatcher (CU count, address of the fixed
+ * scratch array of the allocation-free entry point) */
+void conv_device_setup(void);
+
 void hip_set_device(int n)
 {
     gpu_index = n;
     if (g_parse_only) return;
     hip_check_error(hipSetDevice(n));
+    conv_device_setup();
 }
 
 int hip_get_device(void)

@@ -47,6 +47,7 @@ SIGNATURES = {
     # ---- darknet_hip.h: fused layer forwards
     "forward_convolutional_gpu": (None, [V] * 8 + [i] * 11),
     "forward_convolutional_shortcut_gpu": (None, [V] * 8 + [i] * 11 + [V, V, f, f, i]),
+    "forward_convolutional_noalloc_gpu": (i, [V] * 8 + [i] * 11),
     "conv_packed_floats": (z, [i, i, i, i]), "conv_pack_weights_gpu": (None, [V, V, i, i, i, i]),
     "conv_set_algo": (None, [i]),
     "xnor_weight_words": (z, [i, i, i]), "xnor_input_words": (z, [i, i, i, i]),

@@ -149,6 +149,29 @@ void forward_convolutional_shortcut_gpu(const float *input, const float *weights
                                         int activation, const float *add, float *sum_output, float alpha,
                                         float beta, int shortcut_activation);
 
+/* forward_convolutional_gpu for callers that cannot allocate device memory (code under stream
+ * capture, tight serving loops, harnesses that forbid hipMalloc).  No counterpart in the
+ * reference.  Same arguments and same result, bit for bit; the call itself makes no hipMalloc /
+ * hipFree or any other allocating call: the K-split accumulators, the one buffer
+ * forward_convolutional_gpu grows on demand, live in a fixed 64 MiB array inside the library's
+ * code object (one copy per device, held until the process ends).
+ *   - `packed` must be the buffer conv_pack_weights_gpu wrote wherever conv_packed_floats() != 0
+ *     (the per-call repack would need a buffer);
+ *   - conv_set_precision(1) is refused for 3x3 layers (that mode stages its input);
+ *   - a geometry whose K-split needs more than 64 MiB is refused (none of the benchmark
+ *     networks comes near: their largest need is 48 MB).
+ * Returns 0, or -1 after a message on stderr when the call was refused; a refused call launches
+ * nothing.  The address of the array is looked up once per device (hip_set_device does it;
+ * otherwise the first call on that device, which should then precede any stream capture).
+ * Every call on a device shares that device's array: calls that overlap on one device - two
+ * streams, two host threads - race.  Calls on one stream are ordered and safe. */
+int forward_convolutional_noalloc_gpu(const float *input, const float *weights, const float *packed,
+                                      const float *biases, const float *scales,
+                                      const float *rolling_mean, const float *rolling_variance,
+                                      float *output, int batch, int c, int h, int w, int n,
+                                      int groups, int size, int stride, int pad, int batch_normalize,
+                                      int activation);
+
 /* Weight repack for the MFMA kernel (the natural hook is push_convolutional_layer,
  * src/convolutional_kernels.cu:286-297).  conv_packed_floats() == 0 means the layer does not
  * use a packed copy (grouped convolutions outside the 32-filter block-diagonal scheme).  The
