@@ -8,8 +8,10 @@ Default workload: yolov3 at 416x416, batch 64, fp32 - the configuration the head
 quoted on.  Prints ONE JSON line on stdout; progress goes to stderr.
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload yolov3-416|yolov3-608|yolov3-tiny-416|
-                    yolov3-tiny-xnor-416|resnext50-224|yolov1-448|yolov1-tiny-448] [--batch B] [--precision fp32|bf16x3|bf16]
-                    [--per-layer FILE] [--no-cpu]
+                    yolov3-tiny-xnor-416|resnext50-224|yolov1-448|yolov1-tiny-448|sweep] [--batch B]
+                    [--precision fp32|bf16x3|bf16] [--per-layer FILE] [--no-cpu]
+Without --batch the default workload is measured at batch 64 (the line's `value`) and then at
+batch 1 in the same process (the line's `batch1` object): the metric is quoted at both.
     python bench.py --post      (letterbox and detection decode + NMS latency instead of the forward pass)
 
 The line carries, besides the driver's fields:
@@ -19,6 +21,8 @@ The line carries, besides the driver's fields:
                 right after the timed ones; the same pass records an event after every layer
                 for the per-layer table (the timed steps themselves carry no events: those
                 cost a few microseconds each, 20% of a batch-1 pass)
+  roofline      also carries, per network, the conv layer furthest below its own ceiling
+                min(MFMA peak, arithmetic intensity x 8 TB/s); XNOR networks are priced against HBM
   cpu_baseline  the reference CPU path (compiled reference when oracle/_ref is present, else
                 this repository's restatement, both -Ofast -fopenmp) timed on the host cores
                 on a bounded sample of the same network
@@ -248,59 +252,25 @@ def post_bench(args):
     print(json.dumps(out), flush=True)
 
 
-def main():
-    ap = argparse.ArgumentParser()
-    ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=10)
-    ap.add_argument("--warmup", type=int, default=3)
-    ap.add_argument("--workload", default="yolov3-416", choices=sorted(WORKLOADS))
-    ap.add_argument("--batch", type=int, default=64)
-    ap.add_argument("--per-layer", default="")
-    ap.add_argument("--precision", default="fp32", choices=["fp32", "bf16", "bf16x3"],
-                    help="bf16: the tap-blocked MFMA kernels round their operands to bf16 (opt-in, not the "
-                         "headline configuration; its error against fp32 is reported by the tests)")
-    ap.add_argument("--no-cpu", action="store_true")
-    ap.add_argument("--post", action="store_true",
-                    help="time letterbox and detection decode + NMS around the forward pass instead")
-    ap.add_argument("--cpu-kind", default="reference", choices=["reference", "port"])
-    args = ap.parse_args()
-    if args.gpus != 1:
-        log("bench.py: this build runs on one GPU only (the forward path has no exchange step: it shards "
-            "by batch, every GPU running the same forward on its share of the images). Use --gpus 1.")
-        sys.exit(2)
-
-    if args.post:
-        post_bench(args)
-        return
-
+def measure(L, api, synth, workload, batch, precision, steps, warmup, per_layer=""):
+    """One workload at one batch size: the timed steps, then the same steps with events for the
+    roofline and the per-layer table, then the PCIe-inclusive figure.  Returns the JSON fields."""
     import numpy as np
-    from darknet_amd import api, cfgs, synth
-
-    cfg_name, size = WORKLOADS[args.workload]
-    text = cfg_generator(cfg_name)(args.batch, size)
-    api.set_gpu(0)
-    L = api._lib.load()
+    cfg_name, size = WORKLOADS[workload]
+    text = cfg_generator(cfg_name)(batch, size)
     dev = L.hip_device_name().decode()
-    log("device:", dev)
-    L.conv_set_precision({"fp32": 0, "bf16": 1, "bf16x3": 2}[args.precision])
+    L.conv_set_precision({"fp32": 0, "bf16": 1, "bf16x3": 2}[precision])
     # bf16x3 issues six bf16 MFMAs per fp32-equivalent multiply-add: its algorithmic FLOPs are priced
     # against a sixth of the bf16 peak
     peak = {"fp32": PEAK_FP32_MFMA_TFLOPS, "bf16": PEAK_BF16_MFMA_TFLOPS,
-            "bf16x3": PEAK_BF16_MFMA_TFLOPS / 6}[args.precision]
+            "bf16x3": PEAK_BF16_MFMA_TFLOPS / 6}[precision]
     net = api.Network(cfg_text=text)
     fill_params(net.set_conv, net.layers)
     x = synth.uniform01(7, net.inputs * net.batch)
     net.push_input(x)
     flops_img = net.conv_flops()
 
-    # One plain copy of known size (256 MiB read + 256 MiB written): the yardstick that turns a
-    # profiler's FETCH_SIZE / WRITE_SIZE readings for the conv kernel into bytes.
-    cal = api.DeviceArray(n=64 << 20), api.DeviceArray(n=64 << 20)
-    L.copy_gpu(64 << 20, cal[0].ptr, 1, cal[1].ptr, 1)
-    net.synchronize()
-    del cal
-
-    for _ in range(args.warmup):
+    for _ in range(warmup):
         net.forward_device()
     net.synchronize()
 
@@ -310,14 +280,14 @@ def main():
     net.synchronize()
     t0 = time.perf_counter()
     L.hip_event_record(ev0)
-    for _ in range(args.steps):
+    for _ in range(steps):
         net.forward_device()
     L.hip_event_record(ev1)
     net.synchronize()
     wall_ms = (time.perf_counter() - t0) * 1e3
     total_ms = L.hip_event_elapsed_ms(ev0, ev1)
-    ms_per_step = max(total_ms, 0.0) / args.steps
-    value = args.batch / (ms_per_step / 1e3)
+    ms_per_step = max(total_ms, 0.0) / steps
+    value = batch / (ms_per_step / 1e3)
 
     # ---- the same K steps again with a HIP event after every layer (same stream): per-kernel
     # launch durations for the roofline.  The extra events cost a few microseconds per layer, so
@@ -325,15 +295,15 @@ def main():
     layer_ms = np.zeros(net.n)
     kernel_ms = np.zeros(net.n)
     L.hip_event_record(ev0)
-    for _ in range(args.steps):
+    for _ in range(steps):
         _, ms, kms = net.forward_profiled_kernels()
         layer_ms += np.asarray(ms)
         kernel_ms += np.asarray(kms)
     L.hip_event_record(ev1)
     net.synchronize()
-    layer_ms /= args.steps
-    kernel_ms /= args.steps          # -1 stays -1: a layer takes the same kernel every step
-    ms_per_step_events = L.hip_event_elapsed_ms(ev0, ev1) / args.steps
+    layer_ms /= steps
+    kernel_ms /= steps          # -1 stays -1: a layer takes the same kernel every step
+    ms_per_step_events = L.hip_event_elapsed_ms(ev0, ev1) / steps
 
     # ---- PCIe-inclusive figure (network_predict: H2D input + D2H yolo/last outputs), untimed extra
     t0 = time.perf_counter()
@@ -360,8 +330,13 @@ def main():
         if Ly["type"] == "convolutional":
             fl = 2.0 * Ly["n"] * Ly["size"] ** 2 * (Ly["c"] // Ly["groups"]) * Ly["out_h"] * Ly["out_w"] * Ly["batch"]
             name = ("xnor_conv_kernel" if Ly["xnor"] else
-                    L.conv_kernel_name(Ly["n"], Ly["c"], Ly["groups"], Ly["size"]).decode())
-            row.update(flops=fl, kernel=name, tflops=fl / ms / 1e9 if ms > 0 else 0.0,
+                    L.conv_kernel_name_columns(Ly["n"], Ly["c"], Ly["groups"], Ly["size"],
+                                               Ly["batch"] * Ly["out_h"] * Ly["out_w"]).decode())
+            # what bounds the layer: the matrix cores, or HBM at its arithmetic intensity
+            ceiling = min(peak, fl / row["bytes"] * PEAK_HBM_GBS / 1e3)
+            tfl = fl / ms / 1e9 if ms > 0 else 0.0
+            row.update(flops=fl, kernel=name, tflops=tfl, ceiling_tflops=ceiling,
+                       frac_of_ceiling=tfl / ceiling if ceiling > 0 else 0.0,
                        shape=f'{Ly["size"]}x{Ly["size"]}/{Ly["stride"]} {Ly["c"]}->{Ly["n"]} @{Ly["w"]}x{Ly["h"]}')
             row["kernel_ms"] = float(kernel_ms[i])   # the main kernel alone; -1 = not stamped
             k = kernels.setdefault(name, {"ms": 0.0, "kernel_ms": 0.0, "stamped": 0, "flops": 0.0,
@@ -387,55 +362,170 @@ def main():
     # the MFMA path) the interval between the events around its layers
     stamped = dom["stamped"] == dom["launches"]
     dom_ms = dom["kernel_ms"] if stamped else dom["ms"]
-    achieved = dom["flops"] / dom_ms / 1e9  # TFLOP/s
     conv_ms = sum(k["ms"] for k in kernels.values())
     conv_tflops = sum(k["flops"] for k in kernels.values()) / conv_ms / 1e9
-    roofline = {"bound": "mfma", "achieved": round(achieved, 3), "peak": peak,
-                "unit": "TFLOP/s", "frac": round(achieved / peak, 4),
-                "traffic": profiled_traffic(args.workload, args.batch, dom_name),
-                "kernel": dom_name, "launches_per_step": dom["launches"],
-                "avg_launch_ms": round(dom_ms / dom["launches"], 4),
-                "timing": "events on the kernel's dispatch" if stamped else "events between layers",
-                "avg_layer_interval_ms": round(dom["ms"] / dom["launches"], 4),
-                "flops_per_launch": dom["flops"] / dom["launches"],
-                "all_conv_tflops": round(conv_tflops, 3),
-                "all_conv_frac": round(conv_tflops / peak, 4)}
+    common = {"kernel": dom_name, "launches_per_step": dom["launches"],
+              "avg_launch_ms": round(dom_ms / dom["launches"], 4),
+              "timing": "events on the kernel's dispatch" if stamped else "events between layers",
+              "avg_layer_interval_ms": round(dom["ms"] / dom["launches"], 4),
+              "traffic": profiled_traffic(workload, batch, dom_name)}
+    if dom_name == "xnor_conv_kernel":
+        # XNOR layers keep fp32 activations in memory: HBM bounds them (bit-ops reported beside it;
+        # one multiply-add of the fp32 formulation is one XNOR + one popcount bit)
+        gbs = dom["bytes"] / dom_ms / 1e6
+        roofline = {"bound": "hbm", "achieved": round(gbs, 1), "peak": PEAK_HBM_GBS, "unit": "GB/s",
+                    "frac": round(gbs / PEAK_HBM_GBS, 4), **common,
+                    "bytes_per_launch": dom["bytes"] / dom["launches"],
+                    "equivalent_fp32_tflops": round(dom["flops"] / dom_ms / 1e9, 3),
+                    "bit_ops_per_s": round(dom["flops"] / dom_ms * 1e3, 1)}
+    else:
+        achieved = dom["flops"] / dom_ms / 1e9  # TFLOP/s
+        roofline = {"bound": "mfma", "achieved": round(achieved, 3), "peak": peak, "unit": "TFLOP/s",
+                    "frac": round(achieved / peak, 4), **common,
+                    "flops_per_launch": dom["flops"] / dom["launches"]}
+    roofline["all_conv_tflops"] = round(conv_tflops, 3)
+    roofline["all_conv_frac"] = round(conv_tflops / peak, 4)
+    conv_rows = [r for r in rows if r["type"] == "convolutional" and r["ms"] > 0]
+    if conv_rows:
+        worst = min(conv_rows, key=lambda r: r["frac_of_ceiling"])
+        roofline["min_conv_frac_of_ceiling"] = round(worst["frac_of_ceiling"], 4)
+        roofline["min_conv_layer"] = f'{worst["layer"]}: {worst["shape"]}'
 
-    if args.per_layer:
-        with open(args.per_layer, "w") as f:
-            json.dump({"device": dev, "workload": args.workload, "batch": args.batch,
+    if per_layer:
+        with open(per_layer, "w") as f:
+            json.dump({"device": dev, "workload": workload, "batch": batch,
                        "ms_per_step": ms_per_step, "layers": rows, "kernels": kernels}, f, indent=1)
-        log("per-layer table written to", args.per_layer)
-    memk = [r for r in rows if r["type"] != "convolutional" and not r["fused"]]
+        log("per-layer table written to", per_layer)
+    memk = [r for r in rows if r["type"] != "convolutional" and not r["fused"] and r["ms"] > 0]
+    mem = None
     if memk:
         mb = sum(r["bytes"] for r in memk)
         mm = sum(r["ms"] for r in memk)
-        log(f"memory-bound layers: {mm:.3f} ms/step, {mb / mm / 1e6:.0f} GB/s "
+        mem = {"ms_per_step": round(mm, 4), "gbs": round(mb / mm / 1e6, 1), "frac_of_hbm_peak": round(mb / mm / 1e6 / PEAK_HBM_GBS, 4)}
+        log(f"[{workload} b{batch}] memory-bound layers: {mm:.3f} ms/step, {mb / mm / 1e6:.0f} GB/s "
             f"({mb / mm / 1e6 / PEAK_HBM_GBS:.1%} of HBM peak; {sum(r['fused'] for r in rows)} shortcuts run "
             f"inside the preceding convolution and are not counted); conv layers {conv_ms:.3f} ms/step, "
             f"{conv_tflops:.1f} TFLOP/s")
+    net.free()
+    return {"value": round(value, 2), "ms_per_step": round(ms_per_step, 4), "batch": batch,
+            "gflop_per_image": round(flops_img / 1e9, 3), "device": dev,
+            "wall_ms_per_step": round(wall_ms / steps, 4),
+            "ms_per_step_with_layer_events": round(ms_per_step_events, 4),
+            "pcie_inclusive_ms_per_step": round(pcie_ms, 3),
+            "pcie_inclusive_images_per_s": round(batch / (pcie_ms / 1e3), 2),
+            "pcie_inclusive_pinned_input_ms_per_step": round(pcie_pinned_ms, 3),
+            "memory_bound_layers": mem, "roofline": roofline}
 
+
+def sweep_bench(args, L):
+    """--workload sweep: the three single-layer shapes of the benchmark configurations (3x3 s1
+    256->512 @26, 1x1 512->256 @52, 3x3 s2 128->256 @104, batch-norm + leaky) at batch 1 and 64,
+    each timed alone through forward_convolutional_gpu.  One JSON line: `value` is the mean
+    TFLOP/s of the three batch-64 layers, `layers` holds all six."""
+    from darknet_amd import cfgs, layerbench
+    rows = []
+    for name, (c, h, w, n, size, stride) in cfgs.SWEEP.items():
+        for batch in (1, 64):
+            r = layerbench.time_layer(batch, c, h, w, n, size, stride, pad=size // 2 if size > 1 else 0,
+                                      iters=max(args.steps, 20), warmup=max(args.warmup, 3))
+            fl = 2.0 * n * size * size * c * batch * ((h + 2 * (size // 2) - size) // stride + 1) ** 2
+            byts = r["algorithmic_gbs"] * r["ms"] * 1e6
+            ceiling = min(PEAK_FP32_MFMA_TFLOPS, fl / byts * PEAK_HBM_GBS / 1e3)
+            r.update(name=name, ceiling_tflops=round(ceiling, 1), frac_of_ceiling=round(r["tflops"] / ceiling, 4))
+            rows.append(r)
+            log(json.dumps(r))
+    b64 = [r for r in rows if r["batch"] == 64]
+    dom = max(b64, key=lambda r: r["ms"])
+    mean = sum(r["tflops"] for r in b64) / len(b64)
+    out = {"metric": "conv TFLOP/s, single-layer sweep (mean of the three batch-64 layers)", "value": round(mean, 2),
+           "unit": "TFLOP/s", "n_gpus": 1, "steps": max(args.steps, 20), "warmup": max(args.warmup, 3),
+           "ms_per_step": round(sum(r["ms"] for r in b64), 4), "higher_is_better": True, "scaling": "weak",
+           "vs_baseline": None, "dtype": "f32", "data": "synthetic",
+           "config": {"workload": "single conv layer sweep, fp32, batch 1 and 64, BN + leaky, activations and weights "
+                                  "uniform(-1,1)", "device": L.hip_device_name().decode()},
+           "roofline": {"bound": "mfma", "achieved": dom["tflops"], "peak": PEAK_FP32_MFMA_TFLOPS, "unit": "TFLOP/s",
+                        "frac": round(dom["tflops"] / PEAK_FP32_MFMA_TFLOPS, 4), "traffic": None,
+                        "kernel": dom["kernel"], "layer": dom["shape"], "avg_launch_ms": dom["ms"],
+                        "timing": "events around the layer's launches"},
+           "layers": rows}
+    print(json.dumps(out), flush=True)
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=10)
+    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--workload", default="yolov3-416", choices=sorted(WORKLOADS) + ["sweep"])
+    ap.add_argument("--batch", type=int, default=0,
+                    help="default: 64, followed (for the default workload) by a batch-1 leg reported as `batch1`")
+    ap.add_argument("--per-layer", default="")
+    ap.add_argument("--precision", default="fp32", choices=["fp32", "bf16", "bf16x3"],
+                    help="bf16: the tap-blocked MFMA kernels round their operands to bf16 (opt-in, not the "
+                         "headline configuration; its error against fp32 is reported by the tests)")
+    ap.add_argument("--no-cpu", action="store_true")
+    ap.add_argument("--post", action="store_true",
+                    help="time letterbox and detection decode + NMS around the forward pass instead")
+    ap.add_argument("--cpu-kind", default="reference", choices=["reference", "port"])
+    args = ap.parse_args()
+    if args.gpus != 1:
+        log("bench.py: this build runs on one GPU only (the forward path has no exchange step: it shards "
+            "by batch, every GPU running the same forward on its share of the images). Use --gpus 1.")
+        sys.exit(2)
+
+    if args.post:
+        post_bench(args)
+        return
+
+    from darknet_amd import api, synth
+
+    api.set_gpu(0)
+    L = api._lib.load()
+    log("device:", L.hip_device_name().decode())
+    if args.workload == "sweep":
+        sweep_bench(args, L)
+        return
+
+    # One plain copy of known size (256 MiB read + 256 MiB written): the yardstick that turns a
+    # profiler's FETCH_SIZE / WRITE_SIZE readings for the conv kernel into bytes.
+    cal = api.DeviceArray(n=64 << 20), api.DeviceArray(n=64 << 20)
+    L.copy_gpu(64 << 20, cal[0].ptr, 1, cal[1].ptr, 1)
+    L.hip_synchronize()
+    del cal
+
+    batch = args.batch or 64
+    m = measure(L, api, synth, args.workload, batch, args.precision, args.steps, args.warmup, args.per_layer)
+    # The metric is quoted at batch 64 and batch 1 (the reference's own `speed` loop runs at batch 1,
+    # examples/darknet.c:116-134): the default run measures both in one process, batch 64 first.
+    m1 = None
+    if not args.batch and args.workload == "yolov3-416":
+        m1 = measure(L, api, synth, args.workload, 1, args.precision, max(args.steps, 50), max(args.warmup, 10))
+
+    cfg_name, size = WORKLOADS[args.workload]
+    config = {"workload": f"{args.workload} forward, batch {batch}, {args.precision}, input uniform[0,1), "
+                          f"weights uniform(-1,1)*sqrt(2/(k*k*c)), BN mean 0 var 1 scale 1"}
+    config.update({k: m[k] for k in ("gflop_per_image", "device", "wall_ms_per_step", "ms_per_step_with_layer_events",
+                                     "pcie_inclusive_ms_per_step", "pcie_inclusive_images_per_s",
+                                     "pcie_inclusive_pinned_input_ms_per_step", "memory_bound_layers")})
     out = {
-        "metric": "images/sec", "value": round(value, 2), "unit": "images/s", "n_gpus": 1,
-        "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(ms_per_step, 4),
+        "metric": "images/sec", "value": m["value"], "unit": "images/s", "n_gpus": 1,
+        "steps": args.steps, "warmup": args.warmup, "ms_per_step": m["ms_per_step"],
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": {"fp32": "f32", "bf16": "bf16 operands, f32 accumulate and storage",
                   "bf16x3": "f32 emulated with three bf16 pieces per operand, f32 accumulate and storage"}[args.precision],
-        "data": "synthetic",
-        "config": {"workload": f"{args.workload} forward, batch {args.batch}, {args.precision}, input uniform[0,1), "
-                               f"weights uniform(-1,1)*sqrt(2/(k*k*c)), BN mean 0 var 1 scale 1",
-                   "gflop_per_image": round(flops_img / 1e9, 3), "device": dev,
-                   "wall_ms_per_step": round(wall_ms / args.steps, 4),
-                   "ms_per_step_with_layer_events": round(ms_per_step_events, 4),
-                   "pcie_inclusive_ms_per_step": round(pcie_ms, 3),
-                   "pcie_inclusive_images_per_s": round(args.batch / (pcie_ms / 1e3), 2),
-                   "pcie_inclusive_pinned_input_ms_per_step": round(pcie_pinned_ms, 3)},
-        "roofline": roofline,
+        "data": "synthetic", "config": config, "roofline": m["roofline"],
     }
-    net.free()
+    if m1:
+        out["batch1"] = {"metric": "images/sec", "value": m1["value"], "unit": "images/s", "ms_per_step": m1["ms_per_step"],
+                         "steps": max(args.steps, 50), "warmup": max(args.warmup, 10),
+                         "workload": f"{args.workload} forward, batch 1, {args.precision}, same process, after the batch-64 leg",
+                         "pcie_inclusive_ms_per_step": m1["pcie_inclusive_ms_per_step"],
+                         "memory_bound_layers": m1["memory_bound_layers"], "roofline": m1["roofline"]}
     if not args.no_cpu:
         try:
-            out["cpu_baseline"] = cpu_baseline(args.cpu_kind, cfg_name, size)
+            cb = cpu_baseline(args.cpu_kind, cfg_name, size)
+            cb["gflops"] = round(cb["value"] * m["gflop_per_image"], 2)
+            out["cpu_baseline"] = cb
         except Exception as e:  # the CPU leg must not take the GPU result down with it
             log("cpu_baseline failed:", repr(e))
             out["cpu_baseline"] = None

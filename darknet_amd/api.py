@@ -280,12 +280,25 @@ class Network:
         p = self.L.layer_indexes_host(self.net, i)
         return np.ctypeslib.as_array(p, shape=(L["batch"], L["outputs"])).copy()
 
+    def set_batch(self, b):
+        """set_batch_network: 1 .. the batch the cfg was parsed with (buffers are sized for that)."""
+        self.L.set_batch_network(self.net, b)
+        self._refresh_batch()
+
+    def _refresh_batch(self):
+        iv = (C.c_int * 8)()
+        self.L.network_info(self.net, iv)
+        self.batch = list(iv)[1]
+        for L in self.layers:          # layer_output / layer_indexes shape their result from these
+            L["batch"] = self.batch
+
     def predict_image(self, arr):
-        """network_predict_image (python/darknet.py:106-108): letterbox on the device, batch 1."""
+        """network_predict_image (python/darknet.py:106-108): letterbox on the device, batch 1
+        (the network stays at batch 1 afterwards, as in the reference; set_batch() brings it back)."""
         _bind_image_calls(self.L)
         im, keep = _image_of(arr)
         out = self.L.network_predict_image(self.net, im)
-        self.batch = 1
+        self._refresh_batch()
         last = [L for L in self.layers if L["type"] != "cost"][-1]
         return np.ctypeslib.as_array(out, shape=(1, last["outputs"])).copy()
 

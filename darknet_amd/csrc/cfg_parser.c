@@ -38,6 +38,7 @@ static LAYER_TYPE section_type(const char *t)
     if (!strcmp(t, "[upsample]")) return UPSAMPLE;
     if (!strcmp(t, "[conn]") || !strcmp(t, "[connected]")) return CONNECTED;
     if (!strcmp(t, "[dropout]")) return DROPOUT;
+    if (!strcmp(t, "[batchnorm]")) return BATCHNORM;
     if (!strcmp(t, "[reorg]")) return REORG;
     if (!strcmp(t, "[crop]")) return CROP;
     if (!strcmp(t, "[cost]")) return COST;
@@ -81,6 +82,7 @@ char *get_layer_string(LAYER_TYPE a)
     case YOLO: return "yolo";
     case CONNECTED: return "connected";
     case DROPOUT: return "dropout";
+    case BATCHNORM: return "batchnorm";
     case REORG: return "reorg";
     case CROP: return "crop";
     case COST: return "cost";
@@ -453,6 +455,7 @@ network *parse_network_cfg(char *filename)
         case REGION: l = parse_region(o, p); break;
         case LOCAL: l = parse_local(o, p); break;
         case DETECTION: l = parse_detection(o, p); break;
+        case BATCHNORM: l = make_batchnorm_layer(p.batch, p.w, p.h, p.c); break; /* src/parser.c:533-537 */
         case DROPOUT:
             if (count == 0) dn_fatal("dropout cannot be the first layer");
             l = parse_dropout(o, p);
@@ -494,13 +497,19 @@ network *parse_network_cfg(char *filename)
         net->truths = out->outputs;
         if (last->truths) net->truths = last->truths;
         if (!out->output) {
-            out->output = hip_host_alloc((size_t)out->outputs * out->batch);
-            /* a dropout layer behind it shares the buffer (src/parser.c:831) */
-            if (i + 1 < net->n && net->layers[i + 1].type == DROPOUT) net->layers[i + 1].output = out->output;
+            /* a dropout layer's buffers are those of the layer before it (src/parser.c:829-836): the
+             * host copy belongs to that owner, which free_layer releases, and every dropout layer
+             * behind the owner shares it */
+            int owner = i, j;
+            while (owner > 0 && net->layers[owner].type == DROPOUT) --owner;
+            net->layers[owner].output = hip_host_alloc((size_t)out->outputs * out->batch);
+            for (j = owner + 1; j < net->n && net->layers[j].type == DROPOUT; ++j)
+                net->layers[j].output = net->layers[owner].output;
         }
         net->output = out->output;
         net->output_gpu = out->output_gpu;
     }
+    net->max_batch = net->batch;
     net->input = (float *)dn_calloc((size_t)net->inputs * net->batch, sizeof(float));
     net->input_gpu = hip_make_array(net->input, (size_t)net->inputs * net->batch);
     return net;

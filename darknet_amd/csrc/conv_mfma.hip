@@ -95,6 +95,13 @@ struct mfma_args {
      * whole_tiles + j / split and leaves raw accumulators in `partial` for the reduce kernel */
     int whole_tiles, split;
     float *partial;
+    /* fused reduction of the K-slices (null = conv_reduce_kernel does it in a second launch):
+     * two counters per tail tile (arrived, departed), a fault word the host can read, and the
+     * bound of the wait for a tile's other slices */
+    int *tickets;
+    int *fault;
+    int spin_limit;
+    int fences;
     /* grouped layers (see conv_grouped_tile): every 32-filter tile reads its own 32 input
      * channels and its own block of packed weights; 0 for ordinary layers */
     int grouped;
@@ -283,6 +290,76 @@ __device__ __forceinline__ void conv_epilogue(const mfma_args &a, f32x16 (&acc)[
             }
         }
         __builtin_amdgcn_wave_barrier();
+    }
+}
+
+/* Sums the K-slices of one tail tile in slice order (deterministic) and applies the epilogue, for
+ * one unit u of the tile: four accumulator registers of one lane (r = 4g .. 4g+3), i.e. four
+ * consecutive pixels of one filter row (see conv_epilogue for the register map), so consecutive
+ * units read consecutive dwords of every slice and the result leaves as one 16-byte store.
+ * Units whose filter or pixels lie outside the layer read nothing.  COHERENT: the slices were
+ * written during this very launch by workgroups that may sit on other XCDs (each with its own
+ * L2), so they are read with agent-scope loads. */
+template <int BM, int BN, int WM, int WN, bool COHERENT>
+__device__ __forceinline__ void conv_reduce_unit(const mfma_args &a, int t, int u)
+{
+    constexpr int TM = WM / 32, TN = WN / 32;
+    constexpr int WAVES_N = BN / WN;
+    const int lin = a.whole_tiles + t;
+    const int m0 = (lin % a.tiles_m) * BM;
+    const long n0 = (long)(lin / a.tiles_m) * BN;
+    /* u = ((wave*TM*TN + i*TN + j)*4 + g)*64 + lane */
+    const int lane = u & 63;
+    const int g = (u >> 6) & 3;
+    int q = u >> 8;
+    const int j = q % TN;
+    q /= TN;
+    const int i = q % TM;
+    const int wave = q / TM;
+    const int m = m0 + (wave / WAVES_N) * WM + i * 32 + (lane & 31);
+    const long n = n0 + (wave % WAVES_N) * WN + j * 32 + 8 * g + 4 * (lane >> 5);
+    if (m >= a.M || n >= a.Ntotal) return;
+    /* element ((wave*TM*TN + i*TN + j)*16 + 4g + rr)*64 + lane of each slice */
+    const float *ws = a.partial + (long)t * a.split * (BM * BN) + ((u >> 8) * 16 + 4 * g) * 64 + lane;
+    float sum[4] = {0.f, 0.f, 0.f, 0.f};
+    for (int sl = 0; sl < a.split; ++sl) {
+        const float *p = ws + (long)sl * (BM * BN);
+#pragma unroll
+        for (int rr = 0; rr < 4; ++rr)
+            sum[rr] += COHERENT ? __hip_atomic_load(p + rr * 64, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) : p[rr * 64];
+    }
+    const int b = (int)((unsigned)n / (unsigned)a.P);
+    const int px = (int)n - b * a.P;
+    const conv_row_t row = conv_row(a, m);
+    const long off = ((long)b * a.M + m) * a.P + px;
+    float y[4];
+#pragma unroll
+    for (int rr = 0; rr < 4; ++rr) y[rr] = conv_tail_one(sum[rr], row, conv_f2{a.slope_hi, a.slope_lo});
+    if (px + 3 < a.P) { /* the four pixels lie in one image (then n + 3 < Ntotal too) */
+        *(float4u *)(a.out + off) = (float4u){y[0], y[1], y[2], y[3]};
+        if (a.sum) {
+            const float4u r4 = *(const float4u *)(a.add + off);
+            float4u s4;
+            s4.x = conv_residual_one(a, y[0], r4.x);
+            s4.y = conv_residual_one(a, y[1], r4.y);
+            s4.z = conv_residual_one(a, y[2], r4.z);
+            s4.w = conv_residual_one(a, y[3], r4.w);
+            *(float4u *)(a.sum + off) = s4;
+        }
+    } else { /* image boundary or end of N inside the four: element by element */
+        int pc = px;
+        long offc = off;
+        const long wrap = (long)(a.M - 1) * a.P; /* what the offset gains when the pixel index wraps */
+        for (int rr = 0; rr < 4 && n + rr < a.Ntotal; ++rr) {
+            while (pc >= a.P) {
+                pc -= a.P;
+                offc += wrap;
+            }
+            a.out[offc] = y[rr];
+            if (a.sum) a.sum[offc] = conv_residual_one(a, y[rr], a.add[offc]);
+            ++pc;
+            ++offc;
+        }
     }
 }
 
@@ -775,7 +852,59 @@ __global__ __launch_bounds__(DN_THREADS, ((BM == 128 && BF16 != 3) ? 3 : 2)) voi
 
     }
 
-    if (slice_id >= 0) {
+    if (slice_id >= 0 && a.tickets) {
+        /* K-slice with the reduction in this launch.  Every slice parks its raw accumulators with
+         * agent-scope (write-through) stores, so the other XCDs can see them without an L2
+         * write-back, announces itself on the tile's counter once its stores have completed, and
+         * waits for the tile's other slices: they are resident at the same time (the host launches
+         * this variant only when all slices of all tail tiles fit on the chip together, and whole
+         * tiles, which never wait, come first in the grid).  Then each slice reduces its share of
+         * the tile's units in slice order and applies the epilogue.  The wait is bounded: on expiry
+         * the workgroup skips its share, raises the fault word and leaves like the others. */
+        __shared__ int wait_ok;
+        float *ws = a.partial + (long)slice_id * (BM * BN);
+#pragma unroll
+        for (int i = 0; i < TM; ++i)
+#pragma unroll
+            for (int j = 0; j < TN; ++j)
+#pragma unroll
+                for (int r = 0; r < 16; ++r)
+                    __hip_atomic_store(&ws[((wave * TM * TN + i * TN + j) * 16 + r) * 64 + lane], acc[i][j][r],
+                                       __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        const int t = slice_id / a.split, sl = slice_id - t * a.split;
+        int *tk = a.tickets + 2 * t;
+        __builtin_amdgcn_s_waitcnt(0); /* this wave's stores have been acknowledged */
+        __syncthreads();
+        if (tid == 0) {
+            if (a.fences) __builtin_amdgcn_fence(__ATOMIC_RELEASE, "agent");
+            __hip_atomic_fetch_add(tk, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            int spins = 0, ok = 1;
+            while (__hip_atomic_load(tk, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) < a.split) {
+                if (++spins > a.spin_limit) {
+                    ok = 0;
+                    break;
+                }
+                __builtin_amdgcn_s_sleep(8);
+            }
+            wait_ok = ok;
+        }
+        __syncthreads();
+        if (a.fences) __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
+        if (wait_ok) {
+            constexpr int UNITS = BM * BN / 4;
+            const int u0 = (int)((long)sl * UNITS / a.split), u1 = (int)((long)(sl + 1) * UNITS / a.split);
+            for (int u = u0 + tid; u < u1; u += DN_THREADS) conv_reduce_unit<BM, BN, WM, WN, true>(a, t, u);
+        }
+        __syncthreads();
+        if (tid == 0) {
+            if (!wait_ok) __hip_atomic_store(a.fault, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+            /* the last slice to leave puts the tile's counters back to zero for the next launch */
+            if (__hip_atomic_fetch_add(tk + 1, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == a.split - 1) {
+                __hip_atomic_store(tk, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                __hip_atomic_store(tk + 1, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            }
+        }
+    } else if (slice_id >= 0) {
         /* K-slice: park the raw accumulators, lane-major so every store is a full 256-byte row */
         float *ws = a.partial + (long)slice_id * (BM * BN);
 #pragma unroll
@@ -799,75 +928,16 @@ __global__ __launch_bounds__(DN_THREADS, ((BM == 128 && BF16 != 3) ? 3 : 2)) voi
     }
 }
 
-/* Sums the K-slices of the tail tiles in slice order (deterministic) and applies the epilogue.
- * A thread owns four accumulator registers of one lane (r = 4g .. 4g+3): four consecutive pixels
- * of one filter row (see conv_epilogue for the register map), so every read instruction of a
- * wave covers 256 contiguous bytes of a slice and the result leaves as one 16-byte store.
- * Threads whose filter or pixels lie outside the layer read nothing.  Many small workgroups,
- * because a handful of tail tiles must still spread over the whole chip. */
+/* The reduction as a launch of its own (used when the slices cannot all be resident at once, and by
+ * conv_set_algo(4)): many small workgroups, because a handful of tail tiles must still spread over
+ * the whole chip. */
 template <int BM, int BN, int WM, int WN>
 __global__ __launch_bounds__(DN_THREADS) void conv_reduce_kernel(mfma_args a)
 {
-    constexpr int TM = WM / 32, TN = WN / 32;
-    constexpr int WAVES_N = BN / WN;
     constexpr int GROUPS_PER_TILE = BM * BN / 4 / DN_THREADS; /* workgroups per tile */
     const int t = blockIdx.x / GROUPS_PER_TILE;
     const int u = (blockIdx.x - t * GROUPS_PER_TILE) * DN_THREADS + threadIdx.x;
-    const int lin = a.whole_tiles + t;
-    const int m0 = (lin % a.tiles_m) * BM;
-    const long n0 = (long)(lin / a.tiles_m) * BN;
-    /* u = ((wave*TM*TN + i*TN + j)*4 + g)*64 + lane */
-    const int lane = u & 63;
-    const int g = (u >> 6) & 3;
-    int q = u >> 8;
-    const int j = q % TN;
-    q /= TN;
-    const int i = q % TM;
-    const int wave = q / TM;
-    const int m = m0 + (wave / WAVES_N) * WM + i * 32 + (lane & 31);
-    const long n = n0 + (wave % WAVES_N) * WN + j * 32 + 8 * g + 4 * (lane >> 5);
-    if (m >= a.M || n >= a.Ntotal) return;
-    /* element ((wave*TM*TN + i*TN + j)*16 + 4g + rr)*64 + lane of each slice */
-    const float *ws = a.partial + (long)t * a.split * (BM * BN) + ((u >> 8) * 16 + 4 * g) * 64 + lane;
-    float sum[4] = {0.f, 0.f, 0.f, 0.f};
-    for (int sl = 0; sl < a.split; ++sl) {
-        const float *p = ws + (long)sl * (BM * BN);
-#pragma unroll
-        for (int rr = 0; rr < 4; ++rr) sum[rr] += p[rr * 64];
-    }
-    const int b = (int)((unsigned)n / (unsigned)a.P);
-    const int px = (int)n - b * a.P;
-    const conv_row_t row = conv_row(a, m);
-    const long off = ((long)b * a.M + m) * a.P + px;
-    float y[4];
-#pragma unroll
-    for (int rr = 0; rr < 4; ++rr) y[rr] = conv_tail_one(sum[rr], row, conv_f2{a.slope_hi, a.slope_lo});
-    if (px + 3 < a.P) { /* the four pixels lie in one image (then n + 3 < Ntotal too) */
-        *(float4u *)(a.out + off) = (float4u){y[0], y[1], y[2], y[3]};
-        if (a.sum) {
-            const float4u r4 = *(const float4u *)(a.add + off);
-            float4u s4;
-            s4.x = conv_residual_one(a, y[0], r4.x);
-            s4.y = conv_residual_one(a, y[1], r4.y);
-            s4.z = conv_residual_one(a, y[2], r4.z);
-            s4.w = conv_residual_one(a, y[3], r4.w);
-            *(float4u *)(a.sum + off) = s4;
-        }
-    } else { /* image boundary or end of N inside the four: element by element */
-        int pc = px;
-        long offc = off;
-        const long wrap = (long)(a.M - 1) * a.P; /* what the offset gains when the pixel index wraps */
-        for (int rr = 0; rr < 4 && n + rr < a.Ntotal; ++rr) {
-            while (pc >= a.P) {
-                pc -= a.P;
-                offc += wrap;
-            }
-            a.out[offc] = y[rr];
-            if (a.sum) a.sum[offc] = conv_residual_one(a, y[rr], a.add[offc]);
-            ++pc;
-            ++offc;
-        }
-    }
+    conv_reduce_unit<BM, BN, WM, WN, false>(a, t, u);
 }
 
 /* ---- weight packing ---------------------------------------------------------------------- */
@@ -1100,6 +1170,11 @@ extern "C" void conv_profile_next(void *start_event, void *stop_event)
 extern "C" int conv_profile_pending(void) { return g_prof_start != 0; }
 
 static int g_algo = 0;
+/* Tuning and test hooks of the K-split (conv_set_ksplit): 0 / default = automatic. */
+static int g_tune_split = 0;   /* > 0: this many slices for every tail tile (1 = none) */
+static int g_tune_bn = 0;      /* 64 or 128: column width of the 128-row fp32 tile */
+static int g_spin_limit = 1 << 22;
+static int g_fences = 0;
 extern "C" void conv_set_algo(int algo) { g_algo = algo; }
 
 /* 0 = fp32 operands (default, the reference's arithmetic); 1 = the tap-blocked MFMA kernels round
@@ -1117,7 +1192,19 @@ extern "C" int conv_get_precision(void) { return g_precision; }
 
 static int conv_mode(int c, int groups, int size, int stride, int pad, long in_bytes);
 
-extern "C" const char *conv_kernel_name(int n, int c, int groups, int size)
+/* Layers with more than 64 filters run 128x128 tiles, or 128x64 tiles when the layer has fewer
+ * 128-wide tiles than the chip has CUs (batch 1): twice the workgroups before any cut along K,
+ * and fewer padded columns (192 instead of 256 for the 169 pixels of a 13x13 image).  Measured on
+ * every such layer of yolov3 at batch 1: 8-25% less time than the wide tile at its best split. */
+static bool conv_narrow_tile(long columns, int n)
+{
+    if (g_tune_bn) return g_tune_bn == 64;
+    const long tiles = ((columns + 127) / 128) * ((n + 127) / 128);
+    return tiles < 256;
+}
+
+
+extern "C" const char *conv_kernel_name_columns(int n, int c, int groups, int size, long columns)
 {
     static char name[96];
     int mode = conv_mode(c, groups, size, 1, size / 2, 0);
@@ -1132,10 +1219,17 @@ extern "C" const char *conv_kernel_name(int n, int c, int groups, int size)
     if (bf16 && bm == 128 && n > 128) bm = 256;
     if (x3 && bm == 128)
         snprintf(name, sizeof name, "conv_mfma_kernel<128,128,128,32,%d,3>", mode);
+    else if (bm == 128 && g_precision == 0 && conv_narrow_tile(columns, n))
+        snprintf(name, sizeof name, "conv_mfma_kernel<128,64,64,32,%d>", mode);
     else
         snprintf(name, sizeof name, "conv_mfma_kernel<%d,%d,%d,64,%d%s>", bm, bm >= 128 ? 128 : 256,
                  bm == 32 ? 32 : bm == 256 ? 128 : 64, mode, x3 ? ",3" : !bf16 ? "" : mode == 13 ? ",2" : ",1");
     return name;
+}
+
+extern "C" const char *conv_kernel_name(int n, int c, int groups, int size)
+{
+    return conv_kernel_name_columns(n, c, groups, size, 1L << 40);
 }
 
 static float *g_scratch = 0;       /* per-call repack buffer for callers without a packed copy */
@@ -1156,6 +1250,8 @@ static int g_cus = 0;
 static __device__ __align__(256) float scratch[DN_NOALLOC_SCRATCH_FLOATS];
 static float *g_scratch_dev[DN_MAX_DEVICES];
 static int g_cus_dev[DN_MAX_DEVICES];
+static int *g_fault_host[DN_MAX_DEVICES]; /* pinned word a fused K-split reduction raises when its wait expires */
+static int *g_fault_dev[DN_MAX_DEVICES];  /* the same word as the device addresses it */
 static int g_noalloc = 0;       /* inside forward_convolutional_noalloc_gpu */
 static int g_noalloc_error = 0; /* set instead of allocating (or launching) by the paths below */
 
@@ -1176,6 +1272,48 @@ extern "C" __attribute__((visibility("hidden"))) void conv_device_setup(void)
         hip_check_error(hipGetDeviceProperties(&prop, dev));
         g_cus_dev[dev] = prop.multiProcessorCount;
     }
+    if (!g_fault_host[dev] && !g_noalloc) { /* an allocation-free call that arrives first does without */
+        void *h = 0, *d = 0;
+        hip_check_error(hipHostMalloc(&h, 64, hipHostMallocMapped));
+        *(volatile int *)h = 0;
+        hip_check_error(hipHostGetDevicePointer(&d, h, 0));
+        g_fault_host[dev] = (int *)h;
+        g_fault_dev[dev] = (int *)d;
+    }
+}
+
+/* 1 if a fused K-split reduction gave up waiting for its tile's other slices since the last call
+ * (that layer's output is then incomplete); clears the word.  Synchronises the stream first. */
+extern "C" int conv_take_fault(void)
+{
+    if (hip_parse_only()) return 0;
+    const int dev = hip_get_device();
+    if (dev < 0 || dev >= DN_MAX_DEVICES || !g_fault_host[dev]) return 0;
+    hip_check_error(hipStreamSynchronize(dn_stream()));
+    volatile int *f = g_fault_host[dev];
+    const int v = *f;
+    *f = 0;
+    return v != 0;
+}
+
+/* Called by the device shim after it has synchronised with the stream. */
+extern "C" __attribute__((visibility("hidden"))) void conv_check_fault(void)
+{
+    const int dev = gpu_index;
+    if (dev < 0 || dev >= DN_MAX_DEVICES || !g_fault_host[dev]) return;
+    if (*(volatile int *)g_fault_host[dev])
+        dn_fatal("a convolution's K-slices gave up waiting for each other (are the compute units shared with another "
+                 "process?): its output is incomplete; conv_set_algo(4) reduces the slices in a second launch instead");
+}
+
+extern "C" void conv_set_ksplit(int split, int tile_n, int spin_limit, int fences)
+{
+    if (split < 0 || (tile_n != 0 && tile_n != 64 && tile_n != 128))
+        dn_fatal("conv_set_ksplit: split >= 0, tile_n 0, 64 or 128");
+    g_tune_split = split;
+    g_tune_bn = tile_n;
+    g_spin_limit = spin_limit > 0 ? spin_limit : spin_limit == 0 ? (1 << 22) : 0;
+    g_fences = fences;
 }
 
 /* The K-slice accumulator buffer for `need` floats: the growing allocation, or in an
@@ -1202,15 +1340,43 @@ static float *partial_buffer(size_t need)
 
 /* How to cover `tiles` equal tiles on `cus` compute units.  Whole tiles are dealt out in rounds;
  * a remainder that would leave most CUs idle for a whole tile time (or, at batch 1, a grid far
- * smaller than the chip) is cut along K into `split` slices each, reduced afterwards.
+ * smaller than the chip) is cut along K into `split` slices each, which are summed afterwards:
+ * by the slices themselves when all of them can be resident at once (`resident` workgroups fit
+ * the chip; they wait for each other), else by a second launch.
  * Returns the number of whole tiles; *split = 1 means no tail. */
-static long plan_split(long tiles, int kch, int cus, int *split, double fixed_scale)
+static long plan_split(long tiles, int kch, int cus, long resident, int *split, double fixed_scale, int bn)
 {
     *split = 1;
     if (g_algo == 3 || cus <= 0) return tiles;
     const long whole = tiles / cus * cus;
     const long tail = tiles - whole;
-    if (tail == 0 || tail * 10 >= (long)cus * 9) return tiles; /* a nearly full round: leave it */
+    if (tail == 0) return tiles;
+    if (g_tune_split > 0) {
+        *split = g_tune_split < kch ? g_tune_split : kch;
+        return *split > 1 ? whole : tiles;
+    }
+    if (tail * 10 >= (long)cus * 9) return tiles; /* a nearly full round: leave it */
+    if (whole == 0 && fixed_scale == 1.0) {
+        /* The layer does not fill the chip even once (batch 1).  Times in microseconds, fitted to a
+         * sweep of the split factor over the layers of yolov3 at batch 1: a workgroup alone on its
+         * CU cannot hide its LDS reads and barriers behind another one's MFMAs and takes `lone`
+         * per 16-wide chunk, r workgroups sharing a CU take r * `shared`; an unsplit tile pays its
+         * epilogue (2.4), a split one the second launch (5) and, per slice, the extra partial
+         * traffic of both launches. */
+        const double lone = bn <= 64 ? 0.55 : 1.1, shared = bn <= 64 ? 0.45 : 0.9, per_slice = bn <= 64 ? 0.4 : 0.8;
+        double best = kch * lone + 2.4;
+        const int max_s = kch / 2 < 32 ? kch / 2 : 32;
+        for (int s = 2; s <= max_s; ++s) {
+            const long r = (tail * s + cus - 1) / cus; /* workgroups per CU */
+            const double chunks = (double)kch / s;
+            const double cost = chunks * (r == 1 ? lone : shared * (double)r) + 5.0 + per_slice * s;
+            if (cost < 0.92 * best) {
+                best = cost / 0.92; /* later candidates must beat this one outright */
+                *split = s;
+            }
+        }
+        return *split > 1 ? whole : tiles;
+    }
     /* Time in units of one 16-wide K chunk.  A workgroup costs its chunks plus a fixed part
      * (first load latency, epilogue or partial store); the reduce pass costs a little more. */
     const double fixed_whole = 5.0 * fixed_scale, fixed_slice = 8.0 * fixed_scale, reduce = 4.0 * fixed_scale;
@@ -1224,17 +1390,84 @@ static long plan_split(long tiles, int kch, int cus, int *split, double fixed_sc
             *split = s;
         }
     }
+    (void)resident;
     return *split > 1 ? whole : tiles;
 }
 
-#define DN_LAUNCH(K)                                                                                        \
-    do {                                                                                                    \
-        if (g_prof_start)                                                                                   \
-            hipExtLaunchKernelGGL(K, grid, dim3(DN_THREADS), 0, dn_stream(), g_prof_start, g_prof_stop, 0, a); \
-        else                                                                                                \
-            hipLaunchKernelGGL(K, grid, dim3(DN_THREADS), 0, dn_stream(), a);                              \
-        g_prof_start = g_prof_stop = 0;                                                                     \
-    } while (0)
+typedef void (*conv_kernel_t)(mfma_args);
+
+/* Workgroups of `kernel` one CU holds at a time (queried once per kernel). */
+static int kernel_occupancy(conv_kernel_t kernel)
+{
+    static struct { conv_kernel_t k; int n; } cache[64];
+    static int used = 0;
+    for (int i = 0; i < used; ++i)
+        if (cache[i].k == kernel) return cache[i].n;
+    int n = 0;
+    hip_check_error(hipOccupancyMaxActiveBlocksPerMultiprocessor(&n, (const void *)kernel, DN_THREADS, 0));
+    if (n < 1) n = 1;
+    if (used < 64) {
+        cache[used].k = kernel;
+        cache[used].n = n;
+        ++used;
+    }
+    return n;
+}
+
+/* The kernel instance for a tile shape, K order and precision; null when it is not built. */
+template <int BM, int BN, int WM, int WN>
+static conv_kernel_t pick_kernel(int mode, int bf16, int x3)
+{
+    constexpr bool X3_ONLY = WM == 128 && WN == 32; /* the 128x32 wave tile is built for the three-piece mode alone ... */
+    constexpr bool NO_X3 = BM == 128 && WN == 64;   /* ... which never runs the 128x128 tile with 64x64 wave tiles */
+    constexpr bool FP32_ONLY = BN == 64;            /* the narrow tile of small layers */
+    if (BM > 128 && !bf16) dn_fatal("conv dispatch: the 256-row tile is only built for the bf16-operand mode");
+    if (NO_X3 && x3) dn_fatal("conv dispatch: the three-piece mode runs 128x128 tiles with 128x32 wave tiles");
+    if (X3_ONLY && !x3) dn_fatal("conv dispatch: the 128x32 wave tile is only built for the three-piece mode");
+    if (FP32_ONLY && (bf16 || x3)) dn_fatal("conv dispatch: the 128x64 tile is only built for fp32 operands");
+    if constexpr (FP32_ONLY) {
+        switch (mode) {
+        case 11: return conv_mfma_kernel<BM, BN, WM, WN, 11>;
+        case 13: return conv_mfma_kernel<BM, BN, WM, WN, 13>;
+        case 1: return conv_mfma_kernel<BM, BN, WM, WN, 1>;
+        case 3: return conv_mfma_kernel<BM, BN, WM, WN, 3>;
+        default: return conv_mfma_kernel<BM, BN, WM, WN, 0>;
+        }
+    } else {
+        switch (mode) {
+        case 11:
+            if constexpr (X3_ONLY) return conv_mfma_kernel<BM, BN, WM, WN, 11, 3>;
+            else if (bf16) return conv_mfma_kernel<BM, BN, WM, WN, 11, 1>;
+            else if constexpr (BM <= 128) {
+                if constexpr (!NO_X3)
+                    if (x3) return conv_mfma_kernel<BM, BN, WM, WN, 11, 3>;
+                return conv_mfma_kernel<BM, BN, WM, WN, 11>;
+            }
+            break;
+        case 13:
+            if constexpr (X3_ONLY) return conv_mfma_kernel<BM, BN, WM, WN, 13, 3>;
+            else if (bf16) return conv_mfma_kernel<BM, BN, WM, WN, 13, 2>;
+            else if constexpr (BM <= 128) {
+                if constexpr (!NO_X3)
+                    if (x3) return conv_mfma_kernel<BM, BN, WM, WN, 13, 3>;
+                return conv_mfma_kernel<BM, BN, WM, WN, 13>;
+            }
+            break;
+        default:
+            if constexpr (BM <= 128 && !X3_ONLY) {
+                if (mode == 1) return conv_mfma_kernel<BM, BN, WM, WN, 1>;
+                if (mode == 3) return conv_mfma_kernel<BM, BN, WM, WN, 3>;
+                return conv_mfma_kernel<BM, BN, WM, WN, 0>;
+            }
+            break;
+        }
+    }
+    return 0;
+}
+
+/* first floats of the K-slice buffer: the tail tiles' counters (two ints per tile, fewer tail
+ * tiles than CUs) */
+#define DN_TICKET_FLOATS 1024
 
 template <int BM, int BN, int WM, int WN>
 static void launch_tile(const mfma_args &a0, int mode)
@@ -1243,75 +1476,44 @@ static void launch_tile(const mfma_args &a0, int mode)
     a.tiles_m = (a.M + BM - 1) / BM;
     a.tiles_n = (int)((a.Ntotal + BN - 1) / BN);
     const long total = (long)a.tiles_m * a.tiles_n;
-    {
-        const int dev = hip_get_device();
-        if (dev < 0 || dev >= DN_MAX_DEVICES) dn_fatal("conv dispatch: device index out of range");
-        if (!g_cus_dev[dev]) conv_device_setup();
-        g_cus = g_cus_dev[dev];
-    }
-    int split = 1;
-    /* a bf16 chunk takes a small fraction of an fp32 chunk's time; the fixed costs do not shrink */
+    const int dev = hip_get_device();
+    if (dev < 0 || dev >= DN_MAX_DEVICES) dn_fatal("conv dispatch: device index out of range");
+    if (!g_cus_dev[dev]) conv_device_setup();
+    g_cus = g_cus_dev[dev];
     const int bf16 = g_precision == 1 && mode >= 10;
     const int x3 = g_precision == 2 && mode >= 10;
-    const long whole = plan_split(total, a.KCH, g_cus, &split, bf16 ? 6.0 : x3 ? 2.0 : 1.0);
+    const conv_kernel_t kernel = pick_kernel<BM, BN, WM, WN>(mode, bf16, x3);
+    if (!kernel) dn_fatal("conv dispatch: no kernel for this tile shape and mode");
+    /* slices that wait for each other must all be resident; the fault word is set up with the device */
+    long resident = (long)kernel_occupancy(kernel) * g_cus;
+    if (2 * 255 > DN_TICKET_FLOATS || !g_fault_dev[dev]) resident = 0;
+    int split = 1;
+    /* a bf16 chunk takes a small fraction of an fp32 chunk's time; the fixed costs do not shrink */
+    const long whole = plan_split(total, a.KCH, g_cus, resident, &split, bf16 ? 6.0 : x3 ? 2.0 : 1.0, BN);
     const long tail = total - whole;
     a.whole_tiles = (int)whole;
     a.split = split;
     a.per_xcd = (int)((whole + 7) / 8);
     a.partial = 0;
+    a.tickets = 0;
+    a.fault = g_fault_dev[dev];
+    a.spin_limit = g_spin_limit;
+    a.fences = g_fences;
     if (tail > 0) {
-        a.partial = partial_buffer((size_t)tail * split * BM * BN);
-        if (!a.partial) return; /* allocation-free call and the fixed buffer is too small: nothing is launched */
+        float *ws = partial_buffer(DN_TICKET_FLOATS + (size_t)tail * split * BM * BN);
+        if (!ws) return; /* allocation-free call and the fixed buffer is too small: nothing is launched */
+        a.partial = ws + DN_TICKET_FLOATS;
+        if (g_algo == 5 && tail * split <= resident) a.tickets = (int *)ws;
     }
     const dim3 grid((unsigned)(a.per_xcd * 8 + tail * split));
-    if (BM > 128 && !bf16) dn_fatal("conv dispatch: the 256-row tile is only built for the bf16-operand mode");
-    constexpr bool X3_ONLY = WN == 32; /* the 128x32 wave tile is built for the three-piece mode alone ... */
-    constexpr bool NO_X3 = BM == 128 && WN == 64; /* ... which never runs the 128x128 tile with 64x64 wave tiles */
-    if (NO_X3 && x3) dn_fatal("conv dispatch: the three-piece mode runs 128x128 tiles with 128x32 wave tiles");
-    if (X3_ONLY && !x3) dn_fatal("conv dispatch: the 128x32 wave tile is only built for the three-piece mode");
-    switch (mode) {
-    case 11:
-        if constexpr (X3_ONLY) {
-            DN_LAUNCH((conv_mfma_kernel<BM, BN, WM, WN, 11, 3>));
-        } else if (bf16) {
-            DN_LAUNCH((conv_mfma_kernel<BM, BN, WM, WN, 11, 1>));
-        } else if constexpr (BM <= 128) {
-            if constexpr (!NO_X3) {
-                if (x3) {
-                    DN_LAUNCH((conv_mfma_kernel<BM, BN, WM, WN, 11, 3>));
-                    break;
-                }
-            }
-            DN_LAUNCH((conv_mfma_kernel<BM, BN, WM, WN, 11>));
-        }
-        break;
-    case 13:
-        if constexpr (X3_ONLY) {
-            DN_LAUNCH((conv_mfma_kernel<BM, BN, WM, WN, 13, 3>));
-        } else if (bf16) {
-            DN_LAUNCH((conv_mfma_kernel<BM, BN, WM, WN, 13, 2>));
-        } else if constexpr (BM <= 128) {
-            if constexpr (!NO_X3) {
-                if (x3) {
-                    DN_LAUNCH((conv_mfma_kernel<BM, BN, WM, WN, 13, 3>));
-                    break;
-                }
-            }
-            DN_LAUNCH((conv_mfma_kernel<BM, BN, WM, WN, 13>));
-        }
-        break;
-    default:
-        if constexpr (BM <= 128 && !X3_ONLY) {
-            if (mode == 1)
-                DN_LAUNCH((conv_mfma_kernel<BM, BN, WM, WN, 1>));
-            else if (mode == 3)
-                DN_LAUNCH((conv_mfma_kernel<BM, BN, WM, WN, 3>));
-            else
-                DN_LAUNCH((conv_mfma_kernel<BM, BN, WM, WN, 0>));
-        }
-        break;
-    }
-    if (tail > 0)
+    void *args[] = {&a};
+    if (g_prof_start)
+        hip_check_error(hipExtLaunchKernel((const void *)kernel, grid, dim3(DN_THREADS), args, 0, dn_stream(), g_prof_start,
+                                           g_prof_stop, 0));
+    else
+        hip_check_error(hipLaunchKernel((const void *)kernel, grid, dim3(DN_THREADS), args, 0, dn_stream()));
+    g_prof_start = g_prof_stop = 0;
+    if (tail > 0 && !a.tickets)
         hipLaunchKernelGGL((conv_reduce_kernel<BM, BN, WM, WN>), dim3((unsigned)(tail * (BM * BN / 4 / DN_THREADS))),
                            dim3(DN_THREADS), 0, dn_stream(), a);
 }
@@ -1494,6 +1696,8 @@ static void conv_forward(const float *input, const float *weights, const float *
     else if (g_precision == 2 && mode >= 10)
         /* four waves side by side, 128 rows x 32 columns each: no two waves split the same activations */
         launch_tile<128, 128, 128, 32>(a, mode);
+    else if (g_precision == 0 && conv_narrow_tile(a.Ntotal, n))
+        launch_tile<128, 64, 64, 32>(a, mode);
     else
         launch_tile<128, 128, 64, 64>(a, mode);
     dn_check_launch("forward_convolutional_gpu");

@@ -28,6 +28,14 @@ layer make_convolutional_layer(int batch, int h, int w, int c, int n, int groups
     memset(&l, 0, sizeof l);
     if (groups < 1) groups = 1;
     if (c % groups || n % groups) dn_fatal("convolutional layer: groups must divide channels and filters");
+    /* The reference hands a 1x1 layer's image to the GEMM as it lies, whatever stride and padding say
+     * (src/convolutional_layer.c:468-469): with stride 2 it multiplies the first out_h*out_w floats
+     * of every channel block instead of the strided pixels, with padding it reads past the image.
+     * No cfg in the tree asks for that, and there is no meaningful result to be identical to, so the
+     * geometry is refused where the network is built rather than at its first forward. */
+    if (size == 1 && (stride != 1 || padding != 0))
+        dn_fatal("convolutional layer: a 1x1 kernel needs stride 1 and no padding (the reference's result for "
+                 "anything else is a misread image, src/convolutional_layer.c:468-469)");
     l.type = CONVOLUTIONAL;
     l.groups = groups;
     l.h = h;
@@ -448,6 +456,60 @@ void pull_connected_layer(layer l) { pull_convolutional_layer(l); }
 /* ---- dropout: src/dropout_layer.c:7-27.  At inference the layer does nothing
  * (forward_dropout_layer :38-41); its output IS the previous layer's output, which the cfg
  * parser wires up as src/parser.c:829-836 does. --------------------------------------------- */
+/* ---- batchnorm as a layer of its own: src/batchnorm_layer.c:6-67, inference forward :189-235 - */
+layer make_batchnorm_layer(int batch, int w, int h, int c)
+{
+    layer l;
+    int i;
+    memset(&l, 0, sizeof l);
+    if (batch <= 0 || w <= 0 || h <= 0 || c <= 0) dn_fatal("batchnorm layer: bad geometry");
+    l.type = BATCHNORM;
+    l.batch = batch;
+    l.h = l.out_h = h;
+    l.w = l.out_w = w;
+    l.c = l.out_c = c;
+    l.inputs = w * h * c;
+    l.outputs = l.inputs;
+    l.scales = (float *)dn_calloc((size_t)c, sizeof(float));
+    l.biases = (float *)dn_calloc((size_t)c, sizeof(float));
+    for (i = 0; i < c; ++i) l.scales[i] = 1;
+    l.rolling_mean = (float *)dn_calloc((size_t)c, sizeof(float));
+    l.rolling_variance = (float *)dn_calloc((size_t)c, sizeof(float));
+    l.forward_gpu = forward_batchnorm_layer_gpu;
+    if (gpu_index < 0) dn_fatal("this library has no CPU path: gpu_index must name a device");
+    l.output_gpu = hip_make_array(0, (size_t)batch * l.outputs);
+    l.biases_gpu = hip_make_array(l.biases, (size_t)c);
+    l.scales_gpu = hip_make_array(l.scales, (size_t)c);
+    l.rolling_mean_gpu = hip_make_array(l.rolling_mean, (size_t)c);
+    l.rolling_variance_gpu = hip_make_array(l.rolling_variance, (size_t)c);
+    if (dn_verbose) fprintf(stderr, "Batch Normalization Layer: %d x %d x %d image\n", w, h, c);
+    return l;
+}
+
+/* The inference branch: copy, normalize with the rolling statistics, scale, bias - one pass. */
+void forward_batchnorm_layer_gpu(layer l, network net)
+{
+    if (net.train) dn_fatal("forward_batchnorm_layer_gpu: training (batch statistics) is not served");
+    forward_batchnorm_gpu(net.input_gpu, l.output_gpu, l.scales_gpu, l.biases_gpu, l.rolling_mean_gpu,
+                          l.rolling_variance_gpu, l.batch, l.out_c, l.out_h * l.out_w);
+}
+
+/* src/batchnorm_layer.c:176-187: the three vectors a weights file holds for this layer (the biases
+ * are not part of it, src/parser.c:979-990,1122-1133) */
+void pull_batchnorm_layer(layer l)
+{
+    hip_pull_array(l.scales_gpu, l.scales, (size_t)l.c);
+    hip_pull_array(l.rolling_mean_gpu, l.rolling_mean, (size_t)l.c);
+    hip_pull_array(l.rolling_variance_gpu, l.rolling_variance, (size_t)l.c);
+}
+
+void push_batchnorm_layer(layer l)
+{
+    hip_push_array(l.scales_gpu, l.scales, (size_t)l.c);
+    hip_push_array(l.rolling_mean_gpu, l.rolling_mean, (size_t)l.c);
+    hip_push_array(l.rolling_variance_gpu, l.rolling_variance, (size_t)l.c);
+}
+
 layer make_dropout_layer(int batch, int inputs, float probability)
 {
     layer l;
@@ -592,6 +654,7 @@ layer make_region_layer(int batch, int w, int h, int n, int classes, int coords)
     layer l;
     int i;
     memset(&l, 0, sizeof l);
+    if (coords != 4) dn_fatal("region layer: coords must be 4 (forward_region_gpu and region_decode_gpu serve nothing else)");
     l.type = REGION;
     l.n = n;
     l.batch = batch;

@@ -56,9 +56,9 @@ void set_batch_network(network *net, int b)
 {
     int i;
     if (b < 1) dn_fatal("set_batch_network: batch must be at least 1");
-    for (i = 0; i < net->n; ++i)
-        if (b > net->layers[i].batch && net->layers[i].batch > 0 && b > net->batch)
-            dn_fatal("set_batch_network: buffers were allocated for a smaller batch (batch is fixed at parse time)");
+    if (net->max_batch < net->batch) net->max_batch = net->batch; /* a network built without the parser */
+    if (b > net->max_batch)
+        dn_fatal("set_batch_network: buffers were allocated for a smaller batch (the cfg's batch is the limit)");
     net->batch = b;
     for (i = 0; i < net->n; ++i) net->layers[i].batch = b;
 }
@@ -249,8 +249,12 @@ float *layer_output_host(network *net, int i)
     layer *l;
     if (i < 0 || i >= net->n) dn_fatal("layer_output_host: layer index out of range");
     l = &net->layers[i];
+    /* a dropout layer's output is the buffer of the layer before it (src/parser.c:829-836) */
+    if (l->type == DROPOUT && i > 0) return layer_output_host(net, i - 1);
     if (!l->output) {
-        l->output = (float *)dn_calloc((size_t)l->outputs * l->batch, sizeof(float));
+        /* sized for the batch the network was built with: set_batch_network may come back up to it */
+        const int cap = net->max_batch > l->batch ? net->max_batch : l->batch;
+        l->output = (float *)dn_calloc((size_t)l->outputs * cap, sizeof(float));
         if (i == net->n - 1) net->output = l->output;
     }
     hip_pull_array(l->output_gpu, l->output, (size_t)l->outputs * l->batch);
@@ -263,7 +267,8 @@ int *layer_indexes_host(network *net, int i)
     if (i < 0 || i >= net->n) dn_fatal("layer_indexes_host: layer index out of range");
     l = &net->layers[i];
     if (l->type != MAXPOOL || !l->indexes_gpu) dn_fatal("layer_indexes_host: layer has no indexes");
-    if (!l->indexes) l->indexes = (int *)dn_calloc((size_t)l->outputs * l->batch, sizeof(int));
+    if (!l->indexes)
+        l->indexes = (int *)dn_calloc((size_t)l->outputs * (net->max_batch > l->batch ? net->max_batch : l->batch), sizeof(int));
     /* the forward pass leaves the argmax out (only the backward pass reads it): compute it now from
      * the layer's input, which is still resident (nothing is recycled between layers) */
     forward_maxpool_gpu(i ? net->layers[i - 1].output_gpu : net->input_gpu, l->output_gpu, l->indexes_gpu,
@@ -283,8 +288,18 @@ void network_set_conv(network *net, int i, const float *weights, const float *bi
         push_local_layer(l);
         return;
     }
+    if (i >= 0 && i < net->n && net->layers[i].type == BATCHNORM) { /* c values each; no weights */
+        l = net->layers[i];
+        if (biases) memcpy(l.biases, biases, sizeof(float) * (size_t)l.c);
+        if (scales) memcpy(l.scales, scales, sizeof(float) * (size_t)l.c);
+        if (rolling_mean) memcpy(l.rolling_mean, rolling_mean, sizeof(float) * (size_t)l.c);
+        if (rolling_variance) memcpy(l.rolling_variance, rolling_variance, sizeof(float) * (size_t)l.c);
+        push_batchnorm_layer(l);
+        hip_push_array(l.biases_gpu, l.biases, (size_t)l.c);
+        return;
+    }
     if (i < 0 || i >= net->n || (net->layers[i].type != CONVOLUTIONAL && net->layers[i].type != CONNECTED))
-        dn_fatal("network_set_conv: not a convolutional, connected or local layer");
+        dn_fatal("network_set_conv: not a convolutional, connected, batchnorm or local layer");
     l = net->layers[i];
     if (weights) memcpy(l.weights, weights, sizeof(float) * (size_t)l.nweights);
     if (biases) memcpy(l.biases, biases, sizeof(float) * (size_t)l.n);

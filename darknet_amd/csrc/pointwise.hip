@@ -173,6 +173,59 @@ extern "C" void add_bias_gpu(float *output, float *biases, int batch, int n, int
     dn_check_launch("add_bias_gpu");
 }
 
+/* The inference branch of a standalone [batchnorm] layer (src/batchnorm_layer.c:191-192,231-234;
+ * CPU form :135-155) in one pass: out = ((in - mean) / (sqrt(var) + 1e-6f)) * scale + bias with a
+ * rounding to float after each step, as the reference's copy / normalize / scale_bias / add_bias
+ * passes round. */
+__global__ void batchnorm_kernel(const float *in, float *out, const float *scales, const float *biases,
+                                 const float *mean, const float *variance, long n, int filters, int spatial)
+{
+    for (long i = blockIdx.x * (long)blockDim.x + threadIdx.x; i < n; i += (long)gridDim.x * blockDim.x) {
+        const int f = (int)((i / spatial) % filters);
+        const dn_bn_row r = dn_bn_make(1, biases[f], scales[f], mean[f], variance[f]);
+        out[i] = dn_bn_apply(in[i], r, 1);
+    }
+}
+
+extern "C" void forward_batchnorm_gpu(const float *input, float *output, const float *scales, const float *biases,
+                                      const float *rolling_mean, const float *rolling_variance, int batch,
+                                      int c, int spatial)
+{
+    const long n = (long)batch * c * spatial;
+    if (n <= 0) return;
+    if (!input || !output || !scales || !biases || !rolling_mean || !rolling_variance)
+        dn_fatal("forward_batchnorm_gpu: null pointer");
+    hipLaunchKernelGGL(batchnorm_kernel, dim3(dn_blocks(n)), dim3(DN_BLOCK), 0, dn_stream(), input, output,
+                       scales, biases, rolling_mean, rolling_variance, n, c, spatial);
+    dn_check_launch("forward_batchnorm_gpu");
+}
+
+/* cuda_random (src/cuda.c:106-118): n uniform floats in (0, 1], as curandGenerateUniform fills them.
+ * The reference seeds its generator with time(0), so the values were never reproducible there; the
+ * stream here is a counter-based hash of (call number, index).  Only training-time dropout and
+ * crop read it; inference never does. */
+__global__ void random_kernel(float *x, long n, unsigned long long call)
+{
+    for (long i = blockIdx.x * (long)blockDim.x + threadIdx.x; i < n; i += (long)gridDim.x * blockDim.x) {
+        unsigned long long z = call * 0xD1342543DE82EF95ull + (unsigned long long)(i + 1) * 0x9E3779B97F4A7C15ull;
+        z = (z ^ (z >> 30)) * 0xBF58476D1CE4E5B9ull;
+        z = (z ^ (z >> 27)) * 0x94D049BB133111EBull;
+        z ^= z >> 31;
+        x[i] = (float)((z >> 40) + 1) * (1.0f / 16777216.0f); /* 24 bits: (0, 1] */
+    }
+}
+
+extern "C" void hip_random(float *x_gpu, size_t n)
+{
+    static unsigned long long calls = 0;
+    if (!n) return;
+    hip_require_device("cuda_random");
+    hipLaunchKernelGGL(random_kernel, dim3(dn_blocks((long)n)), dim3(DN_BLOCK), 0, dn_stream(), x_gpu, (long)n, ++calls);
+    dn_check_launch("cuda_random");
+}
+
+extern "C" void cuda_random(float *x_gpu, size_t n) { hip_random(x_gpu, n); }
+
 /* ---- shortcut --------------------------------------------------------------------------- */
 /* Same-geometry residual add (every shortcut of the darknet53 family): 16-byte accesses. */
 __global__ void shortcut_same4_kernel(const float4 *in, const float4 *add, float4 *out, long n4,
@@ -531,8 +584,12 @@ __global__ void region_softmax_kernel(const float *in, float *out, long rows, in
 extern "C" void forward_region_gpu(const float *input, float *output, int batch, int w, int h, int n_anchors,
                                    int classes, int coords, int background, int softmax)
 {
-    if (batch <= 0 || w <= 0 || h <= 0 || n_anchors <= 0 || classes < 0 || coords < 4)
+    if (batch <= 0 || w <= 0 || h <= 0 || n_anchors <= 0 || classes < 0)
         dn_fatal("forward_region_gpu: bad geometry");
+    /* with more than four coordinates the reference's two forwards disagree (its GPU form applies
+     * the logistic to entries 4 .. coords-1, src/region_layer.c:450-453, its CPU form does not,
+     * :164-173), and no cfg in the tree uses them */
+    if (coords != 4) dn_fatal("forward_region_gpu: coords must be 4");
     if (input == output) dn_fatal("forward_region_gpu: in-place operation is not supported");
     const int entries = coords + classes + 1;
     const int plane = w * h;

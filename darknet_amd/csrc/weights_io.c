@@ -45,17 +45,21 @@ static void transpose_matrix(float *a, int rows, int cols)
 
 static void load_convolutional_weights(layer l, FILE *fp)
 {
-    int num;
-    if (l.numload) l.n = l.numload;
-    num = l.c / l.groups * l.n * l.size * l.size;
-    read_floats(l.biases, (size_t)l.n, fp, "convolutional biases");
+    /* numload: the file holds only the first `numload` filters (src/parser.c:1166).  The reference
+     * shrinks its by-value copy's n for the whole function; here only the reads and the transpose
+     * see the smaller count, the push runs on the layer as built, whose packed copy is laid out for
+     * all n filters. */
+    const int n = l.numload ? l.numload : l.n;
+    const int num = l.c / l.groups * n * l.size * l.size;
+    if (n < 0 || n > l.n) dn_fatal("convolutional layer: numload exceeds the number of filters");
+    read_floats(l.biases, (size_t)n, fp, "convolutional biases");
     if (l.batch_normalize && !l.dontloadscales) {
-        read_floats(l.scales, (size_t)l.n, fp, "convolutional scales");
-        read_floats(l.rolling_mean, (size_t)l.n, fp, "convolutional rolling_mean");
-        read_floats(l.rolling_variance, (size_t)l.n, fp, "convolutional rolling_variance");
+        read_floats(l.scales, (size_t)n, fp, "convolutional scales");
+        read_floats(l.rolling_mean, (size_t)n, fp, "convolutional rolling_mean");
+        read_floats(l.rolling_variance, (size_t)n, fp, "convolutional rolling_variance");
     }
     read_floats(l.weights, (size_t)num, fp, "convolutional weights");
-    if (l.flipped) transpose_matrix(l.weights, l.c * l.size * l.size, l.n);
+    if (l.flipped) transpose_matrix(l.weights, l.c * l.size * l.size, n);
     push_convolutional_layer(l);
 }
 
@@ -98,6 +102,12 @@ void load_weights_upto(network *net, char *filename, int start, int cutoff)
         if (l.dontload) continue;
         if (l.type == CONVOLUTIONAL) load_convolutional_weights(l, fp);
         if (l.type == CONNECTED) load_connected_weights(l, fp, transpose);
+        if (l.type == BATCHNORM) { /* src/parser.c:1122-1133 */
+            read_floats(l.scales, (size_t)l.c, fp, "batchnorm scales");
+            read_floats(l.rolling_mean, (size_t)l.c, fp, "batchnorm rolling_mean");
+            read_floats(l.rolling_variance, (size_t)l.c, fp, "batchnorm rolling_variance");
+            push_batchnorm_layer(l);
+        }
         if (l.type == LOCAL) { /* src/parser.c:1292-1302 */
             read_floats(l.biases, (size_t)l.outputs, fp, "local biases");
             read_floats(l.weights, (size_t)l.nweights, fp, "local weights");
@@ -136,6 +146,13 @@ void save_weights_upto(network *net, char *filename, int cutoff)
                 fwrite(l.rolling_mean, sizeof(float), (size_t)l.outputs, fp);
                 fwrite(l.rolling_variance, sizeof(float), (size_t)l.outputs, fp);
             }
+            continue;
+        }
+        if (l.type == BATCHNORM) { /* src/parser.c:979-990 */
+            pull_batchnorm_layer(l);
+            fwrite(l.scales, sizeof(float), (size_t)l.c, fp);
+            fwrite(l.rolling_mean, sizeof(float), (size_t)l.c, fp);
+            fwrite(l.rolling_variance, sizeof(float), (size_t)l.c, fp);
             continue;
         }
         if (l.type == LOCAL) { /* src/parser.c:1066-1077 */

@@ -25,6 +25,8 @@ SIGNATURES = {
     "hip_make_array": (V, [F, z]), "hip_make_int_array": (V, [I, z]), "hip_free": (None, [V]),
     "hip_push_array": (None, [V, F, z]), "hip_pull_array": (None, [V, F, z]),
     "hip_mag_array": (f, [V, z]), "hip_compare": (f, [V, F, z, C.c_char_p]),
+    "hip_random": (None, [V, z]), "cuda_random": (None, [V, z]),
+    "forward_batchnorm_gpu": (None, [V] * 6 + [i, i, i]),
     "hip_pull_int_array": (None, [V, I, z]), "hip_push_int_array": (None, [V, I, z]),
     "hip_synchronize": (None, []),
     "hip_get_stream": (V, []), "hip_set_stream": (None, [V]), "hip_device_name": (C.c_char_p, []),
@@ -49,7 +51,7 @@ SIGNATURES = {
     "forward_convolutional_shortcut_gpu": (None, [V] * 8 + [i] * 11 + [V, V, f, f, i]),
     "forward_convolutional_noalloc_gpu": (i, [V] * 8 + [i] * 11),
     "conv_packed_floats": (z, [i, i, i, i]), "conv_pack_weights_gpu": (None, [V, V, i, i, i, i]),
-    "conv_set_algo": (None, [i]),
+    "conv_set_algo": (None, [i]), "conv_set_ksplit": (None, [i, i, i, i]), "conv_take_fault": (i, []),
     "xnor_weight_words": (z, [i, i, i]), "xnor_input_words": (z, [i, i, i, i]),
     "xnor_pack_weights_gpu": (None, [V, V, V, i, i, i]),
     "xnor_pack_input_gpu": (None, [V, V, i, i, i, i]),
@@ -95,7 +97,8 @@ SIGNATURES = {
     "hip_host_alloc": (F, [z]), "hip_host_free": (None, [F]),
     "conv_set_precision": (None, [i]), "conv_get_precision": (i, []),
     "conv_profile_next": (None, [V, V]), "conv_profile_pending": (i, []),
-    "conv_kernel_name": (C.c_char_p, [i, i, i, i]), "layer_output_host": (F, [V, i]),
+    "conv_kernel_name": (C.c_char_p, [i, i, i, i]),
+    "conv_kernel_name_columns": (C.c_char_p, [i, i, i, i, C.c_long]), "layer_output_host": (F, [V, i]),
     "layer_indexes_host": (I, [V, i]), "network_set_verbose": (None, [i]),
     "network_set_conv": (None, [V, i, F, F, F, F, F]),
     "network_layer_info": (None, [V, i, I, F]), "network_route_inputs": (i, [V, i, I, I, i]),
@@ -117,6 +120,7 @@ STRUCT_BY_VALUE = [
     "make_region_layer", "forward_region_layer_gpu",
     "make_local_layer", "forward_local_layer_gpu", "push_local_layer", "pull_local_layer",
     "make_detection_layer", "forward_detection_layer_gpu",
+    "make_batchnorm_layer", "forward_batchnorm_layer_gpu", "push_batchnorm_layer", "pull_batchnorm_layer",
     "make_image", "make_empty_image", "free_image", "resize_image", "letterbox_image", "network_predict_image",
     "network_letterbox_input",
 ]

@@ -11,6 +11,15 @@
  * pointer) is always NULL and forward_network() ends the process if gpu_index < 0 - this library
  * has no CPU path to fall back to.
  *
+ * LAYOUT: `layer` and `network` here hold the members inference uses, under the reference's names
+ * and types, but NOT at the reference's offsets and not all of them (the reference's structs carry
+ * some three hundred training, recurrent and cuDNN members, and their size depends on its GPU /
+ * CUDNN macros, include/darknet.h:334-421).  Both structs travel by value through this API, so an
+ * object file compiled against the reference's include/darknet.h cannot exchange layer / network
+ * objects with this library: a program either compiles against THIS header (same source text:
+ * same names, same calls), or keeps the reference's own host files and structs and binds the
+ * plain-pointer device layer of darknet_hip.h, whose signatures carry no struct at all.
+ *
  * Training-only members (delta, updates, x, x_norm, adam state, cost) are not allocated:
  * inference never reads them and at batch 64 they would triple the footprint.
  *
@@ -159,10 +168,12 @@ typedef struct network {
     float *delta_gpu;
     float *output_gpu;
 
-    /* additions of this library: device row buffer of the detection decode */
+    /* additions of this library: device row buffer of the detection decode; the batch the buffers
+     * were allocated for (set_batch_network may go down and come back up to it) */
     float *det_rows_gpu;
     int *det_count_gpu;
     int det_max_rows;
+    int max_batch;
 } network;
 
 /* include/darknet.h:515-526 */
@@ -207,6 +218,7 @@ layer make_avgpool_layer(int batch, int w, int h, int c); /* src/avgpool_layer.c
 layer make_connected_layer(int batch, int inputs, int outputs, ACTIVATION activation,
                            int batch_normalize, int adam); /* src/connected_layer.c:14 */
 layer make_dropout_layer(int batch, int inputs, float probability); /* src/dropout_layer.c:7 */
+layer make_batchnorm_layer(int batch, int w, int h, int c);          /* src/batchnorm_layer.c:6 */
 layer make_reorg_layer(int batch, int w, int h, int c, int stride, int reverse, int flatten,
                        int extra);                        /* src/reorg_layer.c:8 */
 layer make_crop_layer(int batch, int h, int w, int c, int crop_height, int crop_width, int flip,
@@ -231,6 +243,9 @@ void forward_avgpool_layer_gpu(layer l, network net);       /* src/avgpool_layer
 void forward_softmax_layer_gpu(layer l, network net);       /* src/softmax_layer.c:71 */
 void forward_connected_layer_gpu(layer l, network net);     /* src/connected_layer.c:286 */
 void forward_dropout_layer_gpu(layer l, network net);       /* src/dropout_layer_kernels.cu:17 (inference: nothing) */
+void forward_batchnorm_layer_gpu(layer l, network net);     /* src/batchnorm_layer.c:189 (src/batchnorm_layer.h:13; inference branch) */
+void push_batchnorm_layer(layer l);                         /* src/batchnorm_layer.c:182 (src/batchnorm_layer.h:16) */
+void pull_batchnorm_layer(layer l);                         /* src/batchnorm_layer.c:176 (src/batchnorm_layer.h:15) */
 void forward_reorg_layer_gpu(layer l, network net);         /* src/reorg_layer.c:149 */
 void forward_crop_layer_gpu(layer l, network net);          /* src/crop_layer_kernels.cu:183 */
 void forward_cost_layer_gpu(layer l, network net);          /* src/cost_layer.c:120 (no truth: nothing) */
@@ -250,7 +265,7 @@ void free_network(network *net);                            /* src/network.c:699
 void forward_network(network *net);                         /* src/network.c:188 */
 void forward_network_gpu(network *net);                     /* src/network.c:762 */
 float *network_predict(network *net, float *input);         /* src/network.c:497 */
-void set_batch_network(network *net, int b);                /* src/network.c:339 (shrink only) */
+void set_batch_network(network *net, int b);                /* src/network.c:339 (1 .. the batch the cfg was parsed with) */
 layer get_network_output_layer(network *net);               /* src/network.c:689 */
 float *network_output(network *net);                        /* src/network.c:755 */
 void pull_network_output(network *net);                     /* src/network.c:1123 */
@@ -314,7 +329,8 @@ int *layer_indexes_host(network *net, int i);
 void network_set_verbose(int on);
 /* Overwrites layer i's parameters (host and device copies); NULL leaves a vector as it is.
  * Convolutional: weights[nweights], biases/scales/mean/variance[n]; connected: the same with
- * n = outputs; local: weights[nweights], biases[outputs] (the other three are ignored). */
+ * n = outputs; local: weights[nweights], biases[outputs] (the other three are ignored); batchnorm:
+ * biases/scales/mean/variance[c] (weights ignored). */
 void network_set_conv(network *net, int i, const float *weights, const float *biases,
                       const float *scales, const float *rolling_mean,
                       const float *rolling_variance);

@@ -45,6 +45,10 @@ void   hip_push_array(float *x_gpu, float *x, size_t n);/* cuda_push_array      
 void   hip_pull_array(float *x_gpu, float *x, size_t n);/* cuda_pull_array      src/cuda.c:160 */
 float  hip_mag_array(float *x_gpu, size_t n);           /* cuda_mag_array       src/cuda.c:167 */
 float  hip_compare(float *x_gpu, float *x, size_t n, char *s); /* cuda_compare  src/cuda.c:120 */
+void   hip_random(float *x_gpu, size_t n);              /* cuda_random          src/cuda.c:106: n uniform floats in
+                                                         * (0, 1]; the reference seeds with time(0), the stream here
+                                                         * is a counter-based hash (dropout / crop at training time
+                                                         * are its only readers; inference never calls it) */
 void   hip_pull_int_array(int *x_gpu, int *x, size_t n);/* (maxpool indexes; no reference twin) */
 void   hip_push_int_array(int *x_gpu, int *x, size_t n);/* (counters; no reference twin)        */
 void   hip_synchronize(void);                           /* hipStreamSynchronize on the stream  */
@@ -74,6 +78,7 @@ void   cuda_push_array(float *x_gpu, float *x, size_t n);
 void   cuda_pull_array(float *x_gpu, float *x, size_t n);
 float  cuda_mag_array(float *x_gpu, size_t n);
 float  cuda_compare(float *x_gpu, float *x, size_t n, char *s);
+void   cuda_random(float *x_gpu, size_t n);
 
 /* Event timing on the library's stream (used by the benchmark; no reference twin). */
 void  *hip_event_create(void);
@@ -183,6 +188,9 @@ void conv_pack_weights_gpu(const float *weights, float *packed, int n, int c, in
 /* Name of the kernel forward_convolutional_gpu launches for this geometry, as it appears in a
  * profiler trace (e.g. "conv_mfma_kernel<128,128,64,64,3>"); for reports only. */
 const char *conv_kernel_name(int n, int c, int groups, int size);
+/* The same for a layer of `columns` = batch*out_h*out_w output columns: small layers (batch 1) of
+ * more than 64 filters run a narrower tile, which the name shows. */
+const char *conv_kernel_name_columns(int n, int c, int groups, int size, long columns);
 
 /* Kernel timing for reports: the next forward_convolutional[_shortcut]_gpu call that runs on the
  * MFMA kernel attaches these two events (hip_event_create) to its main kernel's dispatch, so
@@ -193,9 +201,25 @@ void conv_profile_next(void *start_event, void *stop_event);
 int conv_profile_pending(void);
 
 /* Selects the convolution kernel: 0 = automatic (default), 1 = always the plain direct
- * kernel, 3 = MFMA kernel without the K-split of the last partial round of tiles.  The direct
+ * kernel, 3 = MFMA kernel without the K-split of the last partial round of tiles, 4 = K-split
+ * with the slices summed by a second launch instead of by the slices themselves.  The direct
  * kernel is the in-library cross-check of the MFMA kernel. */
 void conv_set_algo(int algo);
+
+/* Tuning and test hooks of the K-split (no counterpart in the reference).  When a layer's last
+ * round of tiles would leave most of the chip idle, those tiles are cut along K into slices;
+ * the slices park their accumulators, wait for each other (they are all resident at once) and
+ * each reduces a share of the tile in slice order, so the result does not depend on timing.
+ *   split       0 = the cost model decides, n > 0 = n slices for every such tile (1 = none)
+ *   tile_n      0 = automatic, 64 or 128 = column width of the tile of layers with > 64 filters
+ *   spin_limit  polls a slice waits for the others: 0 = default (seconds), < 0 = none at all
+ *               (a slice that finds the others not finished gives up at once: for tests)
+ *   fences      0 = default
+ * conv_take_fault(): synchronises, then returns 1 if a slice gave up waiting since the last call
+ * (the output of that layer is then incomplete) and clears the condition; left unasked, the next
+ * hip_synchronize / hip_pull_array ends the process with a message, the library's convention. */
+void conv_set_ksplit(int split, int tile_n, int spin_limit, int fences);
+int conv_take_fault(void);
 
 /* Operand precision of the tap-blocked MFMA convolution kernels (channels a multiple of 16, 1x1 or
  * 3x3 pad 1; grouped 32-filter tiles):
@@ -290,6 +314,14 @@ void local_set_patch_budget(long floats);
  * above 16 images the weights are read once per 16. */
 void forward_connected_stream_gpu(const float *input, const float *weights, const float *biases,
                                   float *output, int batch, int inputs, int outputs, int activation);
+
+/* forward_batchnorm_layer_gpu at inference (src/batchnorm_layer.c:189-235 with net.train == 0; CPU form
+ * :135-155): output = ((input - rolling_mean) / (sqrt(rolling_variance) + 1e-6f)) * scales + biases per
+ * channel, each step rounded to float as the reference's copy / normalize / scale_bias / add_bias passes
+ * round it, in one pass.  input and output are [batch][c][spatial]; they may be the same buffer. */
+void forward_batchnorm_gpu(const float *input, float *output, const float *scales, const float *biases,
+                           const float *rolling_mean, const float *rolling_variance, int batch, int c,
+                           int spatial);
 
 /* forward_avgpool_layer_gpu (src/avgpool_layer_kernels.cu:46-54). */
 void forward_avgpool_gpu(const float *input, float *output, int batch, int c, int h, int w);

@@ -25,7 +25,7 @@ SECTION_ALIASES = {
     "[route]": "route", "[shortcut]": "shortcut", "[upsample]": "upsample", "[yolo]": "yolo",
     "[conn]": "connected", "[connected]": "connected", "[dropout]": "dropout", "[reorg]": "reorg",
     "[crop]": "crop", "[cost]": "cost", "[region]": "region",
-    "[local]": "local", "[detection]": "detection",
+    "[local]": "local", "[detection]": "detection", "[batchnorm]": "batchnorm",
     "[net]": "net", "[network]": "net",
 }
 
@@ -117,6 +117,9 @@ def parse(text: str) -> dict:
                      activation=o.get("activation", "logistic"),
                      batch_normalize=gi(o, "batch_normalize", 0), binary=0, xnor=0,
                      out_h=1, out_w=1, out_c=outputs, outputs=outputs, nweights=inputs * outputs)
+        elif kind == "batchnorm":
+            # parse_batchnorm src/parser.c:533-537, make_batchnorm_layer src/batchnorm_layer.c:6-19
+            L.update(out_h=h, out_w=w, out_c=c, outputs=h * w * c, inputs=h * w * c)
         elif kind == "dropout":
             # parse_dropout src/parser.c:513-521: geometry passes through, output = input
             L.update(probability=gf(o, "probability", 0.5), out_h=h, out_w=w, out_c=c, outputs=inputs,

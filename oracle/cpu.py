@@ -93,6 +93,19 @@ class Oracle:
         self.lib.orc_normalize(_fp(y), _fp(mean), _fp(var), b, f, y.size // (b * f))
         return y
 
+    def batchnorm_layer(self, x, scales, biases, mean, var):
+        """forward_batchnorm_layer at inference (src/batchnorm_layer.c:135-155 with net.train == 0):
+        copy, normalize_cpu with the rolling statistics, scale_bias, add_bias, each a pass of its own
+        over [batch, c, spatial]."""
+        y = np.ascontiguousarray(x, np.float32).copy()
+        b, f = y.shape[0], y.shape[1]
+        sp = y.size // (b * f)
+        self.lib.orc_normalize(_fp(y), _fp(np.ascontiguousarray(mean, np.float32)),
+                               _fp(np.ascontiguousarray(var, np.float32)), b, f, sp)
+        self.lib.orc_scale_bias(_fp(y), _fp(np.ascontiguousarray(scales, np.float32)), b, f, sp)
+        self.lib.orc_add_bias(_fp(y), _fp(np.ascontiguousarray(biases, np.float32)), b, f, sp)
+        return y
+
     def binarize_weights(self, w, n):
         out = np.empty_like(w)
         self.lib.orc_binarize_weights(_fp(w), n, w.size // n, _fp(out))

@@ -65,6 +65,9 @@ class OracleNet:
             w, bi, sc, mu, var = self.params[i]
             return o.connected(x.reshape(b, -1), w, bi, sc, mu, var, outputs=L["outputs"],
                                batch_normalize=L["batch_normalize"], activation=L["activation"])
+        if t == "batchnorm":
+            _, bi, sc, mu, var = self.params[i]
+            return o.batchnorm_layer(x.reshape(b, L["c"], L["h"] * L["w"]), sc, bi, mu, var)
         if t == "dropout":
             return x                                   # forward_dropout_layer returns at once when not training
         if t == "cost":

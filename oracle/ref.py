@@ -83,6 +83,7 @@ class RefNet:
         H.refh_set_conv.argtypes = [C.c_void_p, C.c_int] + [_F] * 5
         H.refh_set_connected.argtypes = [C.c_void_p, C.c_int] + [_F] * 5
         H.refh_set_local.argtypes = [C.c_void_p, C.c_int] + [_F] * 2
+        H.refh_set_batchnorm.argtypes = [C.c_void_p, C.c_int] + [_F] * 4
         H.refh_predict.restype = _F
         H.refh_predict.argtypes = [C.c_void_p, _F]
         for f in ("refh_layer_output", "refh_layer_weights", "refh_layer_binary_weights",
@@ -128,6 +129,9 @@ class RefNet:
         p = lambda a: None if a is None else np.ascontiguousarray(a, np.float32).ctypes.data_as(_F)
         if self.layers[i]["type"] == "local":
             self.h.refh_set_local(self.net, i, p(weights), p(biases))
+            return
+        if self.layers[i]["type"] == "batchnorm":
+            self.h.refh_set_batchnorm(self.net, i, p(biases), p(scales), p(mean), p(var))
             return
         f = self.h.refh_set_connected if self.layers[i]["type"] == "connected" else self.h.refh_set_conv
         f(self.net, i, p(weights), p(biases), p(scales), p(mean), p(var))

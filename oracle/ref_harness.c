@@ -107,6 +107,17 @@ void refh_set_conv(network *net, int i, const float *weights, const float *biase
     }
 }
 
+/* The same for a [batchnorm] layer: c values per vector, no weights (src/batchnorm_layer.c:20-33). */
+void refh_set_batchnorm(network *net, int i, const float *biases, const float *scales, const float *mean,
+                        const float *variance)
+{
+    layer l = net->layers[i];
+    if (biases) memcpy(l.biases, biases, sizeof(float) * (size_t)l.c);
+    if (scales) memcpy(l.scales, scales, sizeof(float) * (size_t)l.c);
+    if (mean) memcpy(l.rolling_mean, mean, sizeof(float) * (size_t)l.c);
+    if (variance) memcpy(l.rolling_variance, variance, sizeof(float) * (size_t)l.c);
+}
+
 /* The same for a connected layer (its parameter vectors are sized by outputs / inputs). */
 void refh_set_connected(network *net, int i, const float *weights, const float *biases,
                         const float *scales, const float *mean, const float *variance)

@@ -25,7 +25,7 @@ seeded synthetic inputs; nothing from the reference's sources is stored.  Fixtur
   detections_case.npz    the two yolo tensors of a yolov3-tiny forward at 96x96 and what
                          get_network_boxes / do_nms_sort make of them (rows x,y,w,h,obj,prob[80])
 
-`python tests/golden/make_golden.py detections|small_net2|images|region|yolov1` rewrites only that fixture.
+`python tests/golden/make_golden.py detections|small_net2|images|region|yolov1|bn_net` rewrites only that fixture.
 """
 import json
 import os
@@ -201,6 +201,51 @@ def small_net2_fixture():
     return [{k: L[k] for k in KEYS if k in L} for L in r.layers]
 
 
+BN_NET = """[net]
+batch=2
+height=12
+width=10
+channels=3
+
+[convolutional]
+filters=8
+size=3
+stride=1
+pad=1
+activation=linear
+
+[batchnorm]
+
+[maxpool]
+size=2
+stride=2
+
+[convolutional]
+batch_normalize=1
+filters=6
+size=1
+stride=1
+activation=leaky
+
+[batchnorm]
+"""
+
+
+def bn_net_fixture():
+    """[batchnorm] as a layer of its own, after a plain and after a batch-normalised convolution:
+    the layer table and the weights file the reference saves.  No outputs: the reference's CPU
+    forward_batchnorm_layer copies into l.x (src/batchnorm_layer.c:138), which make_batchnorm_layer
+    allocates only in a GPU build (:16-33 against :58-59), so a CPU build cannot run this layer."""
+    open(os.path.join(HERE, "bn_net.cfg"), "w").write(BN_NET)
+    r = ref.RefNet(os.path.join(HERE, "bn_net.cfg"))
+    fill_params(r.set_conv, r.layers, seed=710, bn="random")
+    import ctypes as C
+    lib = ref.raw()
+    lib.save_weights.argtypes = [C.c_void_p, C.c_char_p]
+    lib.save_weights(r.net, os.path.join(HERE, "bn_net.weights").encode())
+    return [{k: L[k] for k in KEYS if k in L} for L in r.layers]
+
+
 IMAGE_CASES = {"wide": (3, 37, 53, 32, 32), "tall": (3, 41, 19, 24, 40), "up": (1, 9, 12, 30, 26),
                "same": (2, 16, 16, 16, 16)}
 
@@ -313,6 +358,12 @@ def main():
         images_fixture()
         print("image_cases.npz written")
         return
+    if sys.argv[1:] == ["bn_net"]:
+        tables = json.load(open(os.path.join(HERE, "layer_tables.json")))
+        tables["bn_net"] = bn_net_fixture()
+        json.dump(tables, open(os.path.join(HERE, "layer_tables.json"), "w"), indent=0)
+        print("bn_net fixtures written")
+        return
     if sys.argv[1:] == ["small_net2"]:
         tables = json.load(open(os.path.join(HERE, "layer_tables.json")))
         tables["small_net2"] = small_net2_fixture()
@@ -329,6 +380,7 @@ def main():
         _, tables[name] = table(text)
     tables["small_net2"] = small_net2_fixture()
     tables["yolov1_net"] = yolov1_fixture()
+    tables["bn_net"] = bn_net_fixture()
     json.dump(tables, open(os.path.join(HERE, "layer_tables.json"), "w"), indent=0)
 
     # ---- yolov3-tiny forward checksums

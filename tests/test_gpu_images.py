@@ -53,6 +53,8 @@ def test_letterbox_into_the_network_input_and_predict_image(dn, orc):
     dev = net.layer_output(net.n - 1)
     assert np.array_equal(dev, net.predict(boxed))
     # network_predict_image: batch 1, letterbox on the device, same result as predicting the boxed frame
+    # (the K-split of a small layer depends on the batch size, so the summation order does too:
+    # equal to rounding, not bit for bit)
     one = net.predict_image(frames[1])
-    assert np.array_equal(one[0], dev[1])
+    assert np.abs(one[0] - dev[1]).max() <= 1e-5 * max(np.abs(dev[1]).max(), 1.0)
     net.free()

@@ -251,3 +251,28 @@ def test_pinned_host_buffers_copy_directly_and_predict_the_same(dn):
     assert np.array_equal(got, want)
     api.free_pinned_array(p)
     net.free()
+
+
+def test_forward_batchnorm_gpu_bit_exact(dn, orc):
+    """The standalone batch-norm forward: one pass, the bits of the reference's four."""
+    x = synth.uniform(5, 5 * 13 * 33).reshape(5, 13, 33)
+    bias, scale, mean, var = synth.bn_random(6, 13)
+    want = orc.batchnorm_layer(x, scale, bias, mean, var)
+    d = [api.DeviceArray(a) for a in (x, scale, bias, mean, var)]
+    out = api.DeviceArray(n=x.size)
+    dn.forward_batchnorm_gpu(d[0].ptr, out.ptr, d[1].ptr, d[2].ptr, d[3].ptr, d[4].ptr, 5, 13, 33)
+    assert np.array_equal(out.numpy(x.shape), want)
+    dn.forward_batchnorm_gpu(d[0].ptr, d[0].ptr, d[1].ptr, d[2].ptr, d[3].ptr, d[4].ptr, 5, 13, 33)   # in place
+    assert np.array_equal(d[0].numpy(x.shape), want)
+
+
+def test_cuda_random_fills_the_unit_interval(dn):
+    """cuda_random (src/cuda.c:106): uniform floats in (0, 1], a new stream on every call."""
+    n = 1 << 20
+    a, b = api.DeviceArray(n=n), api.DeviceArray(n=n)
+    dn.cuda_random(a.ptr, n)
+    dn.cuda_random(b.ptr, n)
+    x, y = a.numpy(), b.numpy()
+    for v in (x, y):
+        assert v.min() > 0 and v.max() <= 1 and abs(v.mean() - 0.5) < 2e-3 and abs(v.var() - 1 / 12) < 1e-3
+    assert (x != y).mean() > 0.99

@@ -165,15 +165,20 @@ def test_yolov3_batch_64_runs_and_is_consistent(dn):
     net1.free()
 
 
-def test_set_batch_network_shrinks(dn):
+def test_set_batch_network_shrinks_and_grows_back(dn):
     net = api.Network(cfg_text=cfgs.yolov3_tiny(4, 160))
     fill_params(net.set_conv, net.layers)
     x = synth.uniform01(9, net.inputs * 4).reshape(4, -1)
     full = net.predict(x)
-    net.L.set_batch_network(net.net, 1)
-    net.batch = 1
+    net.set_batch(1)
     one = net.predict(x[0])
-    assert np.array_equal(one[0], full[0])
+    assert np.abs(one[0] - full[0]).max() <= 1e-5 * max(np.abs(full[0]).max(), 1.0)   # another K-split, same values
+    assert net.layer_output(3).shape[0] == 1          # shaped from the current batch, not the parse-time one
+    # and back up to the batch the buffers were allocated for
+    net.set_batch(4)
+    again = net.predict(x)
+    assert np.array_equal(again, full)
+    assert net.layer_output(3).shape[0] == 4
     net.free()
 
 
@@ -249,6 +254,39 @@ def test_small_net2_crop_reorg_dropout_connected_cost(dn, tmp_path):
     out = str(tmp_path / "roundtrip.weights")
     net.save_weights(out)
     assert open(out, "rb").read() == open(os.path.join(GOLD, "small_net2.weights"), "rb").read()
+    net.free()
+
+
+def test_batchnorm_layer_network_and_weights_file(dn, tmp_path):
+    """[batchnorm] as a layer of its own (after a plain and after a batch-normalised convolution):
+    layer table, the weights file the reference saved for it (scales, mean, variance of those
+    layers; byte-identical round trip), and every layer against the checker."""
+    text = open(os.path.join(GOLD, "bn_net.cfg")).read()
+    gold = json.load(open(os.path.join(GOLD, "layer_tables.json")))["bn_net"]
+    net = api.Network(cfg_text=text, weights=os.path.join(GOLD, "bn_net.weights"))
+    assert [L["type"] for L in net.layers] == [L["type"] for L in gold] and net.layers[1]["type"] == "batchnorm"
+    orc = OracleNet(text)
+    fill_params(orc.set_conv, orc.layers, seed=710, bn="random")   # what the fixture's weights file holds
+    x = synth.uniform01(17, net.inputs * net.batch)
+    final = net.predict(x)
+    want = orc.forward(x)
+    for i, L in enumerate(net.layers):
+        assert norm_err(net.layer_output(i), want[i]) <= REL_TOL, (i, L["type"])
+    assert np.array_equal(final, net.layer_output(net.n - 1))
+    out = str(tmp_path / "roundtrip.weights")
+    net.save_weights(out)
+    assert open(out, "rb").read() == open(os.path.join(GOLD, "bn_net.weights"), "rb").read()
+    # with non-zero biases too (a weights file never carries them for this layer)
+    fill_params(net.set_conv, net.layers, seed=33, bn="random")
+    fill_params(orc.set_conv, orc.layers, seed=33, bn="random")
+    b4 = synth.uniform(91, net.layers[4]["c"], -0.5, 0.5)
+    p = orc.params[4]
+    orc.set_conv(4, None, b4, p[2], p[3], p[4])
+    net.set_conv(4, None, b4, p[2], p[3], p[4])
+    net.predict(x)
+    want = orc.forward(x)
+    for i, L in enumerate(net.layers):
+        assert norm_err(net.layer_output(i), want[i]) <= REL_TOL, (i, L["type"])
     net.free()
 
 

@@ -45,8 +45,10 @@ def same_table(a, b, where=""):
                                        ("resnext50-224", cfgs.resnext50(1, 224)),
                                        ("small_net", open(os.path.join(GOLD, "small_net.cfg")).read()),
                                        ("small_net2", open(os.path.join(GOLD, "small_net2.cfg")).read()),
-                                       ("yolov1_net", open(os.path.join(GOLD, "yolov1_net.cfg")).read())],
-                         ids=["yolov3-tiny-416", "yolov3-416", "resnext50-224", "small_net", "small_net2", "yolov1_net"])
+                                       ("yolov1_net", open(os.path.join(GOLD, "yolov1_net.cfg")).read()),
+                                       ("bn_net", open(os.path.join(GOLD, "bn_net.cfg")).read())],
+                         ids=["yolov3-tiny-416", "yolov3-416", "resnext50-224", "small_net", "small_net2", "yolov1_net",
+                              "bn_net"])
 def test_parser_matches_golden_layer_tables(name, text):
     gold = json.load(open(os.path.join(GOLD, "layer_tables.json")))[name]
     same_table(gold, ocfg.parse(text)["layers"], name)

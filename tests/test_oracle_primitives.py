@@ -176,6 +176,30 @@ def test_bn_identity_and_closed_form(orc):
     assert np.array_equal(y, want.astype(np.float32))
 
 
+def test_batchnorm_layer_is_normalize_scale_bias_in_sequence(orc):
+    """The [batchnorm] layer at inference (src/batchnorm_layer.c:135-155): copy, normalize_cpu,
+    scale_bias, add_bias.  Pinned by arithmetic done here in numpy, one rounding to float per
+    pass as the reference's separate loops round, and by the fp64 closed form; a dropped pass, a
+    swapped scale/bias or variance used without its square root each miss by far more than the
+    bound.  (The compiled reference cannot serve as the pin: its CPU forward copies into l.x,
+    which a CPU build never allocates for this layer, src/batchnorm_layer.c:16-33,138.)"""
+    x = synth.uniform(5, 3 * 4 * 7).reshape(3, 4, 7)
+    bias, scale, mean, var = synth.bn_random(6, 4)
+    got = orc.batchnorm_layer(x, scale, bias, mean, var)
+    r = lambda v: v.reshape(1, 4, 1)
+    step = ((x - r(mean)).astype(np.float64) / (np.sqrt(r(var).astype(np.float64)) + float(np.float32(1e-6)))).astype(np.float32)
+    step = (step * r(scale)).astype(np.float32)
+    step = (step + r(bias)).astype(np.float32)
+    assert np.array_equal(got, step)
+    closed = (x.astype(np.float64) - r(mean)) / (np.sqrt(r(var).astype(np.float64)) + 1e-6) * r(scale) + r(bias)
+    assert np.abs(got - closed).max() <= 1e-6 * np.abs(closed).max()
+    # identity statistics leave only the 1.000001 divisor
+    ident = orc.batchnorm_layer(x, np.ones(4, np.float32), np.zeros(4, np.float32), np.zeros(4, np.float32),
+                                np.ones(4, np.float32))
+    assert np.array_equal(ident, (x.astype(np.float64) / (1.0 + float(np.float32(1e-6)))).astype(np.float32))
+    assert np.array_equal(x, synth.uniform(5, 3 * 4 * 7).reshape(3, 4, 7))      # the input is not modified
+
+
 # ---------------------------------------------------------------------------- activations
 def test_activation_closed_forms(orc):
     x = np.array([-3.5, -1.0, -0.0, 0.0, 0.25, 1.0, 7.0], np.float32)

@@ -22,6 +22,10 @@ def fill_params(setter, layers, seed=1000, bn="random"):
         elif L["type"] == "connected":      # weights [outputs][inputs]: a 1x1 convolution of a 1x1 image
             n = L["outputs"]
             w = synth.conv_weights(seed + i, n, L["inputs"], 1)
+        elif L["type"] == "batchnorm":      # c values per vector; the weights file carries no biases for it
+            _, s, m, v = synth.bn_random(seed * 2 + i, L["c"]) if bn == "random" else synth.bn_identity(L["c"])
+            setter(i, None, np.zeros(L["c"], np.float32), s, m, v)
+            continue
         elif L["type"] == "local":          # one [n][c*size*size] matrix per location, one bias per output
             w = synth.conv_weights(seed + i, L["out_h"] * L["out_w"] * L["n"], L["c"], L["size"])
             b = (synth.uniform(seed * 3 + i, L["outputs"], -0.5, 0.5) if bn == "random"
