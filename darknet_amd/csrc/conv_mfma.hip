@@ -95,13 +95,6 @@ struct mfma_args {
      * whole_tiles + j / split and leaves raw accumulators in `partial` for the reduce kernel */
     int whole_tiles, split;
     float *partial;
-    /* fused reduction of the K-slices (null = conv_reduce_kernel does it in a second launch):
-     * two counters per tail tile (arrived, departed), a fault word the host can read, and the
-     * bound of the wait for a tile's other slices */
-    int *tickets;
-    int *fault;
-    int spin_limit;
-    int fences;
     /* grouped layers (see conv_grouped_tile): every 32-filter tile reads its own 32 input
      * channels and its own block of packed weights; 0 for ordinary layers */
     int grouped;
@@ -297,10 +290,8 @@ __device__ __forceinline__ void conv_epilogue(const mfma_args &a, f32x16 (&acc)[
  * one unit u of the tile: four accumulator registers of one lane (r = 4g .. 4g+3), i.e. four
  * consecutive pixels of one filter row (see conv_epilogue for the register map), so consecutive
  * units read consecutive dwords of every slice and the result leaves as one 16-byte store.
- * Units whose filter or pixels lie outside the layer read nothing.  COHERENT: the slices were
- * written during this very launch by workgroups that may sit on other XCDs (each with its own
- * L2), so they are read with agent-scope loads. */
-template <int BM, int BN, int WM, int WN, bool COHERENT>
+ * Units whose filter or pixels lie outside the layer read nothing. */
+template <int BM, int BN, int WM, int WN>
 __device__ __forceinline__ void conv_reduce_unit(const mfma_args &a, int t, int u)
 {
     constexpr int TM = WM / 32, TN = WN / 32;
@@ -322,11 +313,26 @@ __device__ __forceinline__ void conv_reduce_unit(const mfma_args &a, int t, int 
     /* element ((wave*TM*TN + i*TN + j)*16 + 4g + rr)*64 + lane of each slice */
     const float *ws = a.partial + (long)t * a.split * (BM * BN) + ((u >> 8) * 16 + 4 * g) * 64 + lane;
     float sum[4] = {0.f, 0.f, 0.f, 0.f};
-    for (int sl = 0; sl < a.split; ++sl) {
+    int sl = 0;
+    /* four slices' loads in flight at a time; the additions keep slice order */
+    for (; sl + 4 <= a.split; sl += 4) {
+        float v[4][4];
+#pragma unroll
+        for (int q2 = 0; q2 < 4; ++q2) {
+            const float *p = ws + (long)(sl + q2) * (BM * BN);
+#pragma unroll
+            for (int rr = 0; rr < 4; ++rr)
+                v[q2][rr] = p[rr * 64];
+        }
+#pragma unroll
+        for (int q2 = 0; q2 < 4; ++q2)
+#pragma unroll
+            for (int rr = 0; rr < 4; ++rr) sum[rr] += v[q2][rr];
+    }
+    for (; sl < a.split; ++sl) {
         const float *p = ws + (long)sl * (BM * BN);
 #pragma unroll
-        for (int rr = 0; rr < 4; ++rr)
-            sum[rr] += COHERENT ? __hip_atomic_load(p + rr * 64, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) : p[rr * 64];
+        for (int rr = 0; rr < 4; ++rr) sum[rr] += p[rr * 64];
     }
     const int b = (int)((unsigned)n / (unsigned)a.P);
     const int px = (int)n - b * a.P;
@@ -787,14 +793,16 @@ __global__ __launch_bounds__(DN_THREADS, ((BM == 128 && BF16 != 3) ? 3 : 2)) voi
     };
 
     /* One pipeline step, in program order (pinned by scheduling barriers):
-     *   1. direct-to-LDS loads of chunk kc+1 into the other buffer (nobody reads it: every wave
-     *      passed the previous barrier only after its MFMAs had consumed that buffer)
-     *   2. LDS operand reads of chunk kc, 32 MFMAs
-     *   3. wait for this wave's loads (vmcnt), barrier: chunk kc+1 is now visible to all waves */
+     *   1. LDS operand reads of chunk kc are issued
+     *   2. while they are under way, direct-to-LDS loads of chunk kc+1 into the other buffer
+     *      (nobody reads it: every wave passed the previous barrier only after its MFMAs had
+     *      consumed that buffer)
+     *   3. the MFMAs of chunk kc
+     *   4. wait for this wave's loads (vmcnt), barrier: chunk kc+1 is now visible to all waves */
     auto step = [&](int kc_next, int buf) {
-        load_chunk(kc_next, buf ^ 1);
-        __builtin_amdgcn_sched_barrier(0);
         read_operands(buf, 0);
+        __builtin_amdgcn_sched_barrier(0);
+        load_chunk(kc_next, buf ^ 1);
         __builtin_amdgcn_sched_barrier(0);
         mfma_chunk(0);
         __builtin_amdgcn_sched_barrier(0);
@@ -852,59 +860,7 @@ __global__ __launch_bounds__(DN_THREADS, ((BM == 128 && BF16 != 3) ? 3 : 2)) voi
 
     }
 
-    if (slice_id >= 0 && a.tickets) {
-        /* K-slice with the reduction in this launch.  Every slice parks its raw accumulators with
-         * agent-scope (write-through) stores, so the other XCDs can see them without an L2
-         * write-back, announces itself on the tile's counter once its stores have completed, and
-         * waits for the tile's other slices: they are resident at the same time (the host launches
-         * this variant only when all slices of all tail tiles fit on the chip together, and whole
-         * tiles, which never wait, come first in the grid).  Then each slice reduces its share of
-         * the tile's units in slice order and applies the epilogue.  The wait is bounded: on expiry
-         * the workgroup skips its share, raises the fault word and leaves like the others. */
-        __shared__ int wait_ok;
-        float *ws = a.partial + (long)slice_id * (BM * BN);
-#pragma unroll
-        for (int i = 0; i < TM; ++i)
-#pragma unroll
-            for (int j = 0; j < TN; ++j)
-#pragma unroll
-                for (int r = 0; r < 16; ++r)
-                    __hip_atomic_store(&ws[((wave * TM * TN + i * TN + j) * 16 + r) * 64 + lane], acc[i][j][r],
-                                       __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        const int t = slice_id / a.split, sl = slice_id - t * a.split;
-        int *tk = a.tickets + 2 * t;
-        __builtin_amdgcn_s_waitcnt(0); /* this wave's stores have been acknowledged */
-        __syncthreads();
-        if (tid == 0) {
-            if (a.fences) __builtin_amdgcn_fence(__ATOMIC_RELEASE, "agent");
-            __hip_atomic_fetch_add(tk, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-            int spins = 0, ok = 1;
-            while (__hip_atomic_load(tk, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) < a.split) {
-                if (++spins > a.spin_limit) {
-                    ok = 0;
-                    break;
-                }
-                __builtin_amdgcn_s_sleep(8);
-            }
-            wait_ok = ok;
-        }
-        __syncthreads();
-        if (a.fences) __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
-        if (wait_ok) {
-            constexpr int UNITS = BM * BN / 4;
-            const int u0 = (int)((long)sl * UNITS / a.split), u1 = (int)((long)(sl + 1) * UNITS / a.split);
-            for (int u = u0 + tid; u < u1; u += DN_THREADS) conv_reduce_unit<BM, BN, WM, WN, true>(a, t, u);
-        }
-        __syncthreads();
-        if (tid == 0) {
-            if (!wait_ok) __hip_atomic_store(a.fault, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
-            /* the last slice to leave puts the tile's counters back to zero for the next launch */
-            if (__hip_atomic_fetch_add(tk + 1, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == a.split - 1) {
-                __hip_atomic_store(tk, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-                __hip_atomic_store(tk + 1, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-            }
-        }
-    } else if (slice_id >= 0) {
+    if (slice_id >= 0) {
         /* K-slice: park the raw accumulators, lane-major so every store is a full 256-byte row */
         float *ws = a.partial + (long)slice_id * (BM * BN);
 #pragma unroll
@@ -928,16 +884,19 @@ __global__ __launch_bounds__(DN_THREADS, ((BM == 128 && BF16 != 3) ? 3 : 2)) voi
     }
 }
 
-/* The reduction as a launch of its own (used when the slices cannot all be resident at once, and by
- * conv_set_algo(4)): many small workgroups, because a handful of tail tiles must still spread over
- * the whole chip. */
+/* The reduction is a launch of its own, of many small workgroups: a handful of tail tiles must
+ * still spread over the whole chip.  (Letting the slices of a tile wait for each other and sum
+ * themselves inside the main launch was built and measured, with the slices placed on one XCD
+ * and talking through its L2: correct, and no faster - every hand-over between workgroups costs
+ * a round trip of 0.5-1 microsecond even inside an XCD, and storing, announcing, polling, loading
+ * and leaving add up to what the second launch costs.) */
 template <int BM, int BN, int WM, int WN>
 __global__ __launch_bounds__(DN_THREADS) void conv_reduce_kernel(mfma_args a)
 {
     constexpr int GROUPS_PER_TILE = BM * BN / 4 / DN_THREADS; /* workgroups per tile */
     const int t = blockIdx.x / GROUPS_PER_TILE;
     const int u = (blockIdx.x - t * GROUPS_PER_TILE) * DN_THREADS + threadIdx.x;
-    conv_reduce_unit<BM, BN, WM, WN, false>(a, t, u);
+    conv_reduce_unit<BM, BN, WM, WN>(a, t, u);
 }
 
 /* ---- weight packing ---------------------------------------------------------------------- */
@@ -1173,8 +1132,6 @@ static int g_algo = 0;
 /* Tuning and test hooks of the K-split (conv_set_ksplit): 0 / default = automatic. */
 static int g_tune_split = 0;   /* > 0: this many slices for every tail tile (1 = none) */
 static int g_tune_bn = 0;      /* 64 or 128: column width of the 128-row fp32 tile */
-static int g_spin_limit = 1 << 22;
-static int g_fences = 0;
 extern "C" void conv_set_algo(int algo) { g_algo = algo; }
 
 /* 0 = fp32 operands (default, the reference's arithmetic); 1 = the tap-blocked MFMA kernels round
@@ -1250,8 +1207,6 @@ static int g_cus = 0;
 static __device__ __align__(256) float scratch[DN_NOALLOC_SCRATCH_FLOATS];
 static float *g_scratch_dev[DN_MAX_DEVICES];
 static int g_cus_dev[DN_MAX_DEVICES];
-static int *g_fault_host[DN_MAX_DEVICES]; /* pinned word a fused K-split reduction raises when its wait expires */
-static int *g_fault_dev[DN_MAX_DEVICES];  /* the same word as the device addresses it */
 static int g_noalloc = 0;       /* inside forward_convolutional_noalloc_gpu */
 static int g_noalloc_error = 0; /* set instead of allocating (or launching) by the paths below */
 
@@ -1272,48 +1227,14 @@ extern "C" __attribute__((visibility("hidden"))) void conv_device_setup(void)
         hip_check_error(hipGetDeviceProperties(&prop, dev));
         g_cus_dev[dev] = prop.multiProcessorCount;
     }
-    if (!g_fault_host[dev] && !g_noalloc) { /* an allocation-free call that arrives first does without */
-        void *h = 0, *d = 0;
-        hip_check_error(hipHostMalloc(&h, 64, hipHostMallocMapped));
-        *(volatile int *)h = 0;
-        hip_check_error(hipHostGetDevicePointer(&d, h, 0));
-        g_fault_host[dev] = (int *)h;
-        g_fault_dev[dev] = (int *)d;
-    }
 }
 
-/* 1 if a fused K-split reduction gave up waiting for its tile's other slices since the last call
- * (that layer's output is then incomplete); clears the word.  Synchronises the stream first. */
-extern "C" int conv_take_fault(void)
-{
-    if (hip_parse_only()) return 0;
-    const int dev = hip_get_device();
-    if (dev < 0 || dev >= DN_MAX_DEVICES || !g_fault_host[dev]) return 0;
-    hip_check_error(hipStreamSynchronize(dn_stream()));
-    volatile int *f = g_fault_host[dev];
-    const int v = *f;
-    *f = 0;
-    return v != 0;
-}
-
-/* Called by the device shim after it has synchronised with the stream. */
-extern "C" __attribute__((visibility("hidden"))) void conv_check_fault(void)
-{
-    const int dev = gpu_index;
-    if (dev < 0 || dev >= DN_MAX_DEVICES || !g_fault_host[dev]) return;
-    if (*(volatile int *)g_fault_host[dev])
-        dn_fatal("a convolution's K-slices gave up waiting for each other (are the compute units shared with another "
-                 "process?): its output is incomplete; conv_set_algo(4) reduces the slices in a second launch instead");
-}
-
-extern "C" void conv_set_ksplit(int split, int tile_n, int spin_limit, int fences)
+extern "C" void conv_set_ksplit(int split, int tile_n)
 {
     if (split < 0 || (tile_n != 0 && tile_n != 64 && tile_n != 128))
         dn_fatal("conv_set_ksplit: split >= 0, tile_n 0, 64 or 128");
     g_tune_split = split;
     g_tune_bn = tile_n;
-    g_spin_limit = spin_limit > 0 ? spin_limit : spin_limit == 0 ? (1 << 22) : 0;
-    g_fences = fences;
 }
 
 /* The K-slice accumulator buffer for `need` floats: the growing allocation, or in an
@@ -1340,11 +1261,9 @@ static float *partial_buffer(size_t need)
 
 /* How to cover `tiles` equal tiles on `cus` compute units.  Whole tiles are dealt out in rounds;
  * a remainder that would leave most CUs idle for a whole tile time (or, at batch 1, a grid far
- * smaller than the chip) is cut along K into `split` slices each, which are summed afterwards:
- * by the slices themselves when all of them can be resident at once (`resident` workgroups fit
- * the chip; they wait for each other), else by a second launch.
+ * smaller than the chip) is cut along K into `split` slices each, which conv_reduce_kernel sums.
  * Returns the number of whole tiles; *split = 1 means no tail. */
-static long plan_split(long tiles, int kch, int cus, long resident, int *split, double fixed_scale, int bn)
+static long plan_split(long tiles, int kch, int cus, int *split, double fixed_scale, int bn)
 {
     *split = 1;
     if (g_algo == 3 || cus <= 0) return tiles;
@@ -1390,29 +1309,10 @@ static long plan_split(long tiles, int kch, int cus, long resident, int *split, 
             *split = s;
         }
     }
-    (void)resident;
     return *split > 1 ? whole : tiles;
 }
 
 typedef void (*conv_kernel_t)(mfma_args);
-
-/* Workgroups of `kernel` one CU holds at a time (queried once per kernel). */
-static int kernel_occupancy(conv_kernel_t kernel)
-{
-    static struct { conv_kernel_t k; int n; } cache[64];
-    static int used = 0;
-    for (int i = 0; i < used; ++i)
-        if (cache[i].k == kernel) return cache[i].n;
-    int n = 0;
-    hip_check_error(hipOccupancyMaxActiveBlocksPerMultiprocessor(&n, (const void *)kernel, DN_THREADS, 0));
-    if (n < 1) n = 1;
-    if (used < 64) {
-        cache[used].k = kernel;
-        cache[used].n = n;
-        ++used;
-    }
-    return n;
-}
 
 /* The kernel instance for a tile shape, K order and precision; null when it is not built. */
 template <int BM, int BN, int WM, int WN>
@@ -1465,10 +1365,6 @@ static conv_kernel_t pick_kernel(int mode, int bf16, int x3)
     return 0;
 }
 
-/* first floats of the K-slice buffer: the tail tiles' counters (two ints per tile, fewer tail
- * tiles than CUs) */
-#define DN_TICKET_FLOATS 1024
-
 template <int BM, int BN, int WM, int WN>
 static void launch_tile(const mfma_args &a0, int mode)
 {
@@ -1484,26 +1380,17 @@ static void launch_tile(const mfma_args &a0, int mode)
     const int x3 = g_precision == 2 && mode >= 10;
     const conv_kernel_t kernel = pick_kernel<BM, BN, WM, WN>(mode, bf16, x3);
     if (!kernel) dn_fatal("conv dispatch: no kernel for this tile shape and mode");
-    /* slices that wait for each other must all be resident; the fault word is set up with the device */
-    long resident = (long)kernel_occupancy(kernel) * g_cus;
-    if (2 * 255 > DN_TICKET_FLOATS || !g_fault_dev[dev]) resident = 0;
     int split = 1;
     /* a bf16 chunk takes a small fraction of an fp32 chunk's time; the fixed costs do not shrink */
-    const long whole = plan_split(total, a.KCH, g_cus, resident, &split, bf16 ? 6.0 : x3 ? 2.0 : 1.0, BN);
+    const long whole = plan_split(total, a.KCH, g_cus, &split, bf16 ? 6.0 : x3 ? 2.0 : 1.0, BN);
     const long tail = total - whole;
     a.whole_tiles = (int)whole;
     a.split = split;
     a.per_xcd = (int)((whole + 7) / 8);
     a.partial = 0;
-    a.tickets = 0;
-    a.fault = g_fault_dev[dev];
-    a.spin_limit = g_spin_limit;
-    a.fences = g_fences;
     if (tail > 0) {
-        float *ws = partial_buffer(DN_TICKET_FLOATS + (size_t)tail * split * BM * BN);
-        if (!ws) return; /* allocation-free call and the fixed buffer is too small: nothing is launched */
-        a.partial = ws + DN_TICKET_FLOATS;
-        if (g_algo == 5 && tail * split <= resident) a.tickets = (int *)ws;
+        a.partial = partial_buffer((size_t)tail * split * BM * BN);
+        if (!a.partial) return; /* allocation-free call and the fixed buffer is too small: nothing is launched */
     }
     const dim3 grid((unsigned)(a.per_xcd * 8 + tail * split));
     void *args[] = {&a};
@@ -1513,7 +1400,7 @@ static void launch_tile(const mfma_args &a0, int mode)
     else
         hip_check_error(hipLaunchKernel((const void *)kernel, grid, dim3(DN_THREADS), args, 0, dn_stream()));
     g_prof_start = g_prof_stop = 0;
-    if (tail > 0 && !a.tickets)
+    if (tail > 0)
         hipLaunchKernelGGL((conv_reduce_kernel<BM, BN, WM, WN>), dim3((unsigned)(tail * (BM * BN / 4 / DN_THREADS))),
                            dim3(DN_THREADS), 0, dn_stream(), a);
 }

@@ -68,8 +68,6 @@ void hip_require_device(const char *what)
 /* conv_mfma.hip: per-device set-up of the convolution dispatcher (CU count, address of the fixed
  * scratch array of the allocation-free entry point) */
 void conv_device_setup(void);
-/* conv_mfma.hip: ends the process if a convolution's K-slices gave up waiting for each other */
-void conv_check_fault(void);
 
 void hip_set_device(int n)
 {
@@ -100,7 +98,6 @@ void hip_set_stream(void *stream) { g_stream = (hipStream_t)stream; }
 void hip_synchronize(void)
 {
     hip_check_error(hipStreamSynchronize(g_stream));
-    conv_check_fault();
 }
 
 float *hip_make_array(float *x, size_t n)
@@ -267,12 +264,10 @@ void hip_pull_array(float *x_gpu, float *x, size_t n)
     if (g_parse_only) return;
     if (sizeof(float) * n >= DN_STAGE_MIN && !host_is_pinned(x, sizeof(float) * n)) {
         staged_copy((char *)x_gpu, (char *)x, sizeof(float) * n, 0);
-        conv_check_fault();
         return;
     }
     if (g_stream) hip_check_error(hipStreamSynchronize(g_stream));
     hip_check_error(hipMemcpy(x, x_gpu, sizeof(float) * n, hipMemcpyDeviceToHost));
-    conv_check_fault();
 }
 
 void hip_push_int_array(int *x_gpu, int *x, size_t n)

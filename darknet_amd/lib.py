@@ -51,7 +51,7 @@ SIGNATURES = {
     "forward_convolutional_shortcut_gpu": (None, [V] * 8 + [i] * 11 + [V, V, f, f, i]),
     "forward_convolutional_noalloc_gpu": (i, [V] * 8 + [i] * 11),
     "conv_packed_floats": (z, [i, i, i, i]), "conv_pack_weights_gpu": (None, [V, V, i, i, i, i]),
-    "conv_set_algo": (None, [i]), "conv_set_ksplit": (None, [i, i, i, i]), "conv_take_fault": (i, []),
+    "conv_set_algo": (None, [i]), "conv_set_ksplit": (None, [i, i]),
     "xnor_weight_words": (z, [i, i, i]), "xnor_input_words": (z, [i, i, i, i]),
     "xnor_pack_weights_gpu": (None, [V, V, V, i, i, i]),
     "xnor_pack_input_gpu": (None, [V, V, i, i, i, i]),

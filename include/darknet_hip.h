@@ -201,25 +201,16 @@ void conv_profile_next(void *start_event, void *stop_event);
 int conv_profile_pending(void);
 
 /* Selects the convolution kernel: 0 = automatic (default), 1 = always the plain direct
- * kernel, 3 = MFMA kernel without the K-split of the last partial round of tiles, 4 = K-split
- * with the slices summed by a second launch instead of by the slices themselves.  The direct
+ * kernel, 3 = MFMA kernel without the K-split of the last partial round of tiles.  The direct
  * kernel is the in-library cross-check of the MFMA kernel. */
 void conv_set_algo(int algo);
 
-/* Tuning and test hooks of the K-split (no counterpart in the reference).  When a layer's last
- * round of tiles would leave most of the chip idle, those tiles are cut along K into slices;
- * the slices park their accumulators, wait for each other (they are all resident at once) and
- * each reduces a share of the tile in slice order, so the result does not depend on timing.
- *   split       0 = the cost model decides, n > 0 = n slices for every such tile (1 = none)
- *   tile_n      0 = automatic, 64 or 128 = column width of the tile of layers with > 64 filters
- *   spin_limit  polls a slice waits for the others: 0 = default (seconds), < 0 = none at all
- *               (a slice that finds the others not finished gives up at once: for tests)
- *   fences      0 = default
- * conv_take_fault(): synchronises, then returns 1 if a slice gave up waiting since the last call
- * (the output of that layer is then incomplete) and clears the condition; left unasked, the next
- * hip_synchronize / hip_pull_array ends the process with a message, the library's convention. */
-void conv_set_ksplit(int split, int tile_n, int spin_limit, int fences);
-int conv_take_fault(void);
+/* Tuning hooks of the K-split (no counterpart in the reference).  When a layer's last round of
+ * tiles would leave most of the chip idle, those tiles are cut along K into slices that a second
+ * launch sums in slice order.
+ *   split   0 = the cost model decides, n > 0 = n slices for every such tile (1 = none)
+ *   tile_n  0 = automatic, 64 or 128 = column width of the tile of layers with more than 64 filters */
+void conv_set_ksplit(int split, int tile_n);
 
 /* Operand precision of the tap-blocked MFMA convolution kernels (channels a multiple of 16, 1x1 or
  * 3x3 pad 1; grouped 32-filter tiles):
