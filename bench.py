@@ -355,6 +355,10 @@ def measure(L, api, synth, workload, batch, precision, steps, warmup, per_layer=
                             and not prev["xnor"] and 0 <= Ly["index"] < i - 1
                             and (Ly["w"], Ly["h"], Ly["c"]) == (Ly["out_w"], Ly["out_h"], Ly["out_c"])
                             and (Ly["out_w"], Ly["out_h"], Ly["out_c"]) == (prev["out_w"], prev["out_h"], prev["out_c"]))
+        # likewise a yolo head right after the convolution that feeds it
+        row["fused"] = row["fused"] or bool(Ly["type"] == "yolo" and prev and prev["type"] == "convolutional"
+                                            and not prev["xnor"] and prev["n"] == Ly["n"] * (5 + Ly["classes"])
+                                            and (prev["out_w"], prev["out_h"]) == (Ly["w"], Ly["h"]))
         row["gbs"] = row["bytes"] / ms / 1e6 if ms > 0 and not row["fused"] else 0.0
         rows.append(row)
     dom_name, dom = max(kernels.items(), key=lambda kv: kv[1]["ms"])
@@ -403,8 +407,8 @@ def measure(L, api, synth, workload, batch, precision, steps, warmup, per_layer=
         mm = sum(r["ms"] for r in memk)
         mem = {"ms_per_step": round(mm, 4), "gbs": round(mb / mm / 1e6, 1), "frac_of_hbm_peak": round(mb / mm / 1e6 / PEAK_HBM_GBS, 4)}
         log(f"[{workload} b{batch}] memory-bound layers: {mm:.3f} ms/step, {mb / mm / 1e6:.0f} GB/s "
-            f"({mb / mm / 1e6 / PEAK_HBM_GBS:.1%} of HBM peak; {sum(r['fused'] for r in rows)} shortcuts run "
-            f"inside the preceding convolution and are not counted); conv layers {conv_ms:.3f} ms/step, "
+            f"({mb / mm / 1e6 / PEAK_HBM_GBS:.1%} of HBM peak; {sum(r['fused'] for r in rows)} shortcuts "
+            f"and yolo heads run inside the preceding convolution and are not counted); conv layers {conv_ms:.3f} ms/step, "
             f"{conv_tflops:.1f} TFLOP/s")
     net.free()
     return {"value": round(value, 2), "ms_per_step": round(ms_per_step, 4), "batch": batch,

@@ -103,6 +103,10 @@ struct mfma_args {
     const float *add;
     float *sum;
     float s1, s2;
+    /* fused yolo head instead (add == null, sum = the yolo layer's output): sum[i] = out[i] on the
+     * w and h entries of every anchor, logistic(out[i]) elsewhere (src/yolo_layer.c:132-148);
+     * > 0 = entries per anchor (5 + classes) */
+    int yolo_entries;
 };
 
 /* k -> (channel, ky, kx) for a size x size kernel in the reference's im2col row order. */
@@ -201,6 +205,14 @@ __device__ __forceinline__ float conv_residual_one(const mfma_args &a, float y, 
     return conv_slope(__fadd_rn(__fmul_rn(a.s1, y), __fmul_rn(a.s2, r)), conv_f2{a.sum_slope_hi, a.sum_slope_lo});
 }
 
+/* the yolo head's value for filter m */
+__device__ __forceinline__ bool conv_yolo_keeps(const mfma_args &a, int m)
+{
+    const int e = m % a.yolo_entries;
+    return e == 2 || e == 3;
+}
+__device__ __forceinline__ float conv_yolo_one(float y, bool keep) { return keep ? y : dn_logistic_fast(y); }
+
 /* Batch-norm / bias / activation and the store.  The MFMAs are issued with the pixel tile as
  * the row operand and the filter tile as the column operand, so accumulator register r of lane l
  * holds filter (l % 32) and pixel 8*(r/4) + 4*(l/32) + r%4 of its 32x32 block: a lane owns one
@@ -257,7 +269,15 @@ __device__ __forceinline__ void conv_epilogue(const mfma_args &a, f32x16 (&acc)[
             const long o_off = off + (long)m * P;
             if (quad_ok) {
                 *(float4u *)(a.out + o_off) = (float4u){o.x, o.y, o.z, o.w};
-                if (a.sum) {
+                if (a.yolo_entries) {
+                    const bool keep = conv_yolo_keeps(a, m);
+                    float4u s;
+                    s.x = conv_yolo_one(o.x, keep);
+                    s.y = conv_yolo_one(o.y, keep);
+                    s.z = conv_yolo_one(o.z, keep);
+                    s.w = conv_yolo_one(o.w, keep);
+                    *(float4u *)(a.sum + o_off) = s;
+                } else if (a.sum) {
                     const float4u r = *(const float4u *)(a.add + o_off);
                     float4u s;
                     s.x = conv_residual_one(a, o.x, r.x);
@@ -276,7 +296,10 @@ __device__ __forceinline__ void conv_epilogue(const mfma_args &a, f32x16 (&acc)[
                         offc += wrap;
                     }
                     a.out[offc] = v[c];
-                    if (a.sum) a.sum[offc] = conv_residual_one(a, v[c], a.add[offc]);
+                    if (a.yolo_entries)
+                        a.sum[offc] = conv_yolo_one(v[c], conv_yolo_keeps(a, m));
+                    else if (a.sum)
+                        a.sum[offc] = conv_residual_one(a, v[c], a.add[offc]);
                     ++pc;
                     ++offc;
                 }
@@ -343,7 +366,11 @@ __device__ __forceinline__ void conv_reduce_unit(const mfma_args &a, int t, int 
     for (int rr = 0; rr < 4; ++rr) y[rr] = conv_tail_one(sum[rr], row, conv_f2{a.slope_hi, a.slope_lo});
     if (px + 3 < a.P) { /* the four pixels lie in one image (then n + 3 < Ntotal too) */
         *(float4u *)(a.out + off) = (float4u){y[0], y[1], y[2], y[3]};
-        if (a.sum) {
+        if (a.yolo_entries) {
+            const bool keep = conv_yolo_keeps(a, m);
+            *(float4u *)(a.sum + off) = (float4u){conv_yolo_one(y[0], keep), conv_yolo_one(y[1], keep),
+                                                  conv_yolo_one(y[2], keep), conv_yolo_one(y[3], keep)};
+        } else if (a.sum) {
             const float4u r4 = *(const float4u *)(a.add + off);
             float4u s4;
             s4.x = conv_residual_one(a, y[0], r4.x);
@@ -362,7 +389,10 @@ __device__ __forceinline__ void conv_reduce_unit(const mfma_args &a, int t, int 
                 offc += wrap;
             }
             a.out[offc] = y[rr];
-            if (a.sum) a.sum[offc] = conv_residual_one(a, y[rr], a.add[offc]);
+            if (a.yolo_entries)
+                a.sum[offc] = conv_yolo_one(y[rr], conv_yolo_keeps(a, m));
+            else if (a.sum)
+                a.sum[offc] = conv_residual_one(a, y[rr], a.add[offc]);
             ++pc;
             ++offc;
         }
@@ -796,13 +826,21 @@ __global__ __launch_bounds__(DN_THREADS, ((BM == 128 && BF16 != 3) ? 3 : 2)) voi
      *   1. LDS operand reads of chunk kc are issued
      *   2. while they are under way, direct-to-LDS loads of chunk kc+1 into the other buffer
      *      (nobody reads it: every wave passed the previous barrier only after its MFMAs had
-     *      consumed that buffer)
+     *      consumed that buffer); the two swap places for the tiles with 256 columns
      *   3. the MFMAs of chunk kc
      *   4. wait for this wave's loads (vmcnt), barrier: chunk kc+1 is now visible to all waves */
     auto step = [&](int kc_next, int buf) {
-        read_operands(buf, 0);
-        __builtin_amdgcn_sched_barrier(0);
-        load_chunk(kc_next, buf ^ 1);
+        /* the 128-row tiles gain 1-5% from having their reads under way while the loads are issued;
+         * the 256-column tiles, with twice the loads per wave, lose 7% and keep loads first */
+        if constexpr (BM >= 128) {
+            read_operands(buf, 0);
+            __builtin_amdgcn_sched_barrier(0);
+            load_chunk(kc_next, buf ^ 1);
+        } else {
+            load_chunk(kc_next, buf ^ 1);
+            __builtin_amdgcn_sched_barrier(0);
+            read_operands(buf, 0);
+        }
         __builtin_amdgcn_sched_barrier(0);
         mfma_chunk(0);
         __builtin_amdgcn_sched_barrier(0);
@@ -1425,13 +1463,14 @@ static int conv_mode(int c, int groups, int size, int stride, int pad, long in_b
 
 extern "C" void forward_shortcut_gpu(const float *, const float *, float *, int, int, int, int, int, int, int,
                                      float, float, int);
+extern "C" void forward_yolo_gpu(const float *, float *, int, int, int, int, int);
 extern "C" void dn_activate_array(float *x, long n, int activation);
 
 static void conv_forward(const float *input, const float *weights, const float *packed, const float *biases,
                          const float *scales, const float *rolling_mean, const float *rolling_variance,
                          float *output, int batch, int c, int h, int w, int n, int groups, int size, int stride,
                          int pad, int batch_normalize, int activation, const float *add, float *sum, float s1,
-                         float s2, int sum_act)
+                         float s2, int sum_act, int yolo_entries)
 {
     if (batch <= 0 || c <= 0 || h <= 0 || w <= 0 || n <= 0 || groups <= 0 || size <= 0 || stride <= 0 || pad < 0)
         dn_fatal("forward_convolutional_gpu: bad geometry");
@@ -1460,7 +1499,8 @@ static void conv_forward(const float *input, const float *weights, const float *
                 const int nb = (int)(batch - b0 < per ? batch - b0 : per);
                 conv_forward(input + b0 * (in_img / 4), weights, packed, biases, scales, rolling_mean, rolling_variance,
                              output + b0 * out_img, nb, c, h, w, n, groups, size, stride, pad, batch_normalize,
-                             activation, add ? add + b0 * out_img : 0, sum ? sum + b0 * out_img : 0, s1, s2, sum_act);
+                             activation, add ? add + b0 * out_img : 0, sum ? sum + b0 * out_img : 0, s1, s2, sum_act,
+                             yolo_entries);
                 if (g_noalloc_error) return;
             }
             return;
@@ -1477,18 +1517,25 @@ static void conv_forward(const float *input, const float *weights, const float *
     if (mode < 0) {
         conv_direct_forward(input, weights, biases, scales, rolling_mean, rolling_variance, output, batch, c,
                             h, w, n, groups, size, stride, pad, batch_normalize, activation);
-        if (sum) forward_shortcut_gpu(output, add, sum, batch, ow, oh, n, ow, oh, n, s1, s2, sum_act);
+        if (sum && yolo_entries)
+            forward_yolo_gpu(output, sum, batch, ow, oh, n / yolo_entries, yolo_entries - 5);
+        else if (sum)
+            forward_shortcut_gpu(output, add, sum, batch, ow, oh, n, ow, oh, n, s1, s2, sum_act);
         return;
     }
     double slope = 1., sum_slope = 1.;
-    if (!conv_inline_activation(activation, &slope) || (sum && !conv_inline_activation(sum_act, &sum_slope))) {
+    if (!conv_inline_activation(activation, &slope) ||
+        (sum && !yolo_entries && !conv_inline_activation(sum_act, &sum_slope))) {
         /* an activation the epilogue does not carry: linear convolution, then the reference's own
          * sequence of passes (activate_array, src/convolutional_layer.c:478; shortcut) */
         conv_forward(input, weights, packed, biases, scales, rolling_mean, rolling_variance, output, batch, c, h,
-                     w, n, groups, size, stride, pad, batch_normalize, DN_LINEAR, 0, 0, 0.f, 0.f, DN_LINEAR);
+                     w, n, groups, size, stride, pad, batch_normalize, DN_LINEAR, 0, 0, 0.f, 0.f, DN_LINEAR, 0);
         if (g_noalloc_error) return;
         dn_activate_array(output, (long)batch * n * oh * ow, activation);
-        if (sum) forward_shortcut_gpu(output, add, sum, batch, ow, oh, n, ow, oh, n, s1, s2, sum_act);
+        if (sum && yolo_entries)
+            forward_yolo_gpu(output, sum, batch, ow, oh, n / yolo_entries, yolo_entries - 5);
+        else if (sum)
+            forward_shortcut_gpu(output, add, sum, batch, ow, oh, n, ow, oh, n, s1, s2, sum_act);
         return;
     }
 
@@ -1548,6 +1595,7 @@ static void conv_forward(const float *input, const float *weights, const float *
     a.partial = 0;
     a.add = add;
     a.sum = sum;
+    a.yolo_entries = sum ? yolo_entries : 0;
     a.s1 = s1;
     a.s2 = s2;
     a.sum_slope_hi = conv_split(sum_slope).hi;
@@ -1598,7 +1646,7 @@ extern "C" void forward_convolutional_gpu(const float *input, const float *weigh
                                           int batch_normalize, int activation)
 {
     conv_forward(input, weights, packed, biases, scales, rolling_mean, rolling_variance, output, batch, c, h, w,
-                 n, groups, size, stride, pad, batch_normalize, activation, 0, 0, 0.f, 0.f, DN_LINEAR);
+                 n, groups, size, stride, pad, batch_normalize, activation, 0, 0, 0.f, 0.f, DN_LINEAR, 0);
 }
 
 extern "C" void forward_convolutional_shortcut_gpu(const float *input, const float *weights, const float *packed,
@@ -1616,7 +1664,23 @@ extern "C" void forward_convolutional_shortcut_gpu(const float *input, const flo
         dn_fatal("forward_convolutional_shortcut_gpu: unknown activation");
     conv_forward(input, weights, packed, biases, scales, rolling_mean, rolling_variance, output, batch, c, h, w,
                  n, groups, size, stride, pad, batch_normalize, activation, add, sum_output, alpha, beta,
-                 shortcut_activation);
+                 shortcut_activation, 0);
+}
+
+extern "C" void forward_convolutional_yolo_gpu(const float *input, const float *weights, const float *packed,
+                                               const float *biases, const float *scales,
+                                               const float *rolling_mean, const float *rolling_variance,
+                                               float *output, int batch, int c, int h, int w, int n, int groups,
+                                               int size, int stride, int pad, int batch_normalize, int activation,
+                                               float *yolo_output, int n_anchors, int classes)
+{
+    if (!yolo_output) dn_fatal("forward_convolutional_yolo_gpu: null pointer");
+    if (yolo_output == output) dn_fatal("forward_convolutional_yolo_gpu: yolo_output must not alias output");
+    if (n_anchors <= 0 || classes < 0 || n != n_anchors * (5 + classes))
+        dn_fatal("forward_convolutional_yolo_gpu: the filters must be n_anchors * (5 + classes)");
+    conv_forward(input, weights, packed, biases, scales, rolling_mean, rolling_variance, output, batch, c, h, w,
+                 n, groups, size, stride, pad, batch_normalize, activation, 0, yolo_output, 0.f, 0.f, DN_LINEAR,
+                 5 + classes);
 }
 
 extern "C" int forward_convolutional_noalloc_gpu(const float *input, const float *weights, const float *packed,
@@ -1633,7 +1697,7 @@ extern "C" int forward_convolutional_noalloc_gpu(const float *input, const float
     g_noalloc = 1;
     g_noalloc_error = 0;
     conv_forward(input, weights, packed, biases, scales, rolling_mean, rolling_variance, output, batch, c, h, w,
-                 n, groups, size, stride, pad, batch_normalize, activation, 0, 0, 0.f, 0.f, DN_LINEAR);
+                 n, groups, size, stride, pad, batch_normalize, activation, 0, 0, 0.f, 0.f, DN_LINEAR, 0);
     g_noalloc = 0;
     return g_noalloc_error ? -1 : 0;
 }

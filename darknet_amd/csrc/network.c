@@ -89,6 +89,24 @@ static int forward_conv_shortcut_pair(network net, int i)
     return 1;
 }
 
+/* Runs layers i and i+1 together when they are a convolution and the yolo head it feeds
+ * (src/yolo_layer.c:347-361): the head's copy + logistic rides in the convolution's epilogue.
+ * Returns 1 if it did. */
+static int forward_conv_yolo_pair(network net, int i)
+{
+    layer l, y;
+    if (!g_fuse_shortcut || i + 1 >= net.n) return 0;
+    l = net.layers[i];
+    y = net.layers[i + 1];
+    if (l.type != CONVOLUTIONAL || l.xnor || y.type != YOLO) return 0;
+    if (y.w != l.out_w || y.h != l.out_h || y.batch != l.batch || y.n * (5 + y.classes) != l.n) return 0;
+    forward_convolutional_yolo_gpu(net.input_gpu, l.weights_gpu, l.weights_packed_gpu, l.biases_gpu, l.scales_gpu,
+                                   l.rolling_mean_gpu, l.rolling_variance_gpu, l.output_gpu, l.batch, l.c, l.h,
+                                   l.w, l.n, l.groups, l.size, l.stride, l.pad, l.batch_normalize,
+                                   (int)l.activation, y.output_gpu, y.n, y.classes);
+    return 1;
+}
+
 /* The layer loop of src/network.c:773-785 without the copies around it. */
 void forward_network_device(network *netp)
 {
@@ -100,7 +118,7 @@ void forward_network_device(network *netp)
         layer l = net.layers[i];
         net.index = i;
         if (!l.forward_gpu) dn_fatal("layer without a GPU forward");
-        if (forward_conv_shortcut_pair(net, i)) {
+        if (forward_conv_shortcut_pair(net, i) || forward_conv_yolo_pair(net, i)) {
             ++i;
             l = net.layers[i];
         } else {
@@ -146,7 +164,7 @@ float forward_network_profiled_kernels(network *netp, float *layer_ms, float *ke
             conv_profile_next(ks[i], ke[i]);
             timed = 1;
         }
-        if (forward_conv_shortcut_pair(net, i)) {
+        if (forward_conv_shortcut_pair(net, i) || forward_conv_yolo_pair(net, i)) {
             hip_event_record(ev[i + 1]);
             ++i;
             if (kernel_ms) kernel_ms[i] = -1.f;

@@ -326,6 +326,20 @@ __global__ void upsample2_kernel(const float2 *in, float4 *out, long npairs, int
     }
 }
 
+/* stride 2, any width: a thread turns one input into two 8-byte stores (rows 2y and 2y + 1; the
+ * output rows have an even length, so the pairs are aligned whenever the tensor is). */
+__global__ void upsample2e_kernel(const float *in, float2 *out, long n, int w, float scale)
+{
+    for (long i = blockIdx.x * (long)blockDim.x + threadIdx.x; i < n; i += (long)gridDim.x * blockDim.x) {
+        const int x = (int)(i % w);
+        const long row = i / w; /* plane*h + y */
+        const float a = __fmul_rn(scale, in[i]);
+        const float2 o = make_float2(a, a);
+        out[(row * 2) * w + x] = o;
+        out[(row * 2 + 1) * w + x] = o;
+    }
+}
+
 extern "C" void upsample_gpu(float *in, int w, int h, int c, int batch, int stride, int forward,
                              float scale, float *out)
 {
@@ -336,6 +350,10 @@ extern "C" void upsample_gpu(float *in, int w, int h, int c, int batch, int stri
         const long npairs = (long)batch * c * h * (w / 2);
         hipLaunchKernelGGL(upsample2_kernel, dim3(dn_blocks(npairs)), dim3(DN_BLOCK), 0, dn_stream(),
                            (const float2 *)in, (float4 *)out, npairs, w / 2, h, scale);
+    } else if (stride == 2 && ((uintptr_t)out & 7) == 0) {
+        const long nin = (long)batch * c * h * w;
+        hipLaunchKernelGGL(upsample2e_kernel, dim3(dn_blocks(nin)), dim3(DN_BLOCK), 0, dn_stream(),
+                           (const float *)in, (float2 *)out, nin, w, scale);
     } else {
         hipLaunchKernelGGL(upsample_kernel, dim3(dn_blocks(n)), dim3(DN_BLOCK), 0, dn_stream(),
                            (const float *)in, out, n, w, h, stride, scale);
@@ -406,7 +424,23 @@ __global__ void yolo_kernel(const float *in, float *out, long n, int plane, int 
     for (long i = blockIdx.x * (long)blockDim.x + threadIdx.x; i < n; i += (long)gridDim.x * blockDim.x) {
         const int e = (int)((i / plane) % entries);
         const float v = in[i];
-        out[i] = (e == 2 || e == 3) ? v : dn_activate(v, DN_LOGISTIC);
+        out[i] = (e == 2 || e == 3) ? v : dn_logistic_fast(v);
+    }
+}
+
+/* plane a multiple of 4: a 16-byte quad never straddles two entries */
+__global__ void yolo4_kernel(const float4 *in, float4 *out, long n4, int plane4, int entries)
+{
+    for (long i = blockIdx.x * (long)blockDim.x + threadIdx.x; i < n4; i += (long)gridDim.x * blockDim.x) {
+        const int e = (int)((i / plane4) % entries);
+        float4 v = in[i];
+        if (e != 2 && e != 3) {
+            v.x = dn_logistic_fast(v.x);
+            v.y = dn_logistic_fast(v.y);
+            v.z = dn_logistic_fast(v.z);
+            v.w = dn_logistic_fast(v.w);
+        }
+        out[i] = v;
     }
 }
 
@@ -416,8 +450,12 @@ extern "C" void forward_yolo_gpu(const float *input, float *output, int batch, i
     if (batch <= 0 || w <= 0 || h <= 0 || n_anchors <= 0 || classes < 0) dn_fatal("forward_yolo_gpu: bad geometry");
     const int entries = 4 + classes + 1;
     const long n = (long)batch * n_anchors * entries * w * h;
-    hipLaunchKernelGGL(yolo_kernel, dim3(dn_blocks(n)), dim3(DN_BLOCK), 0, dn_stream(), input, output,
-                       n, w * h, entries);
+    if (((w * h) & 3) == 0 && aligned16(input) && aligned16(output))
+        hipLaunchKernelGGL(yolo4_kernel, dim3(dn_blocks(n / 4)), dim3(DN_BLOCK), 0, dn_stream(),
+                           (const float4 *)input, (float4 *)output, n / 4, w * h / 4, entries);
+    else
+        hipLaunchKernelGGL(yolo_kernel, dim3(dn_blocks(n)), dim3(DN_BLOCK), 0, dn_stream(), input, output,
+                           n, w * h, entries);
     dn_check_launch("forward_yolo_gpu");
 }
 

@@ -320,9 +320,9 @@ float forward_network_profiled(network *net, float *layer_ms);
  * kernel alone, from events attached to its dispatch (-1 where there is none) */
 float forward_network_profiled_kernels(network *net, float *layer_ms, float *kernel_ms);
 /* 1 (default): forward_network_device runs a convolution and the same-geometry shortcut right
- * after it as one pass (forward_convolutional_shortcut_gpu); 0: layer by layer as
- * src/network.c:773-785 does.  Every layer's output buffer is written in both modes and holds
- * the same bits. */
+ * after it as one pass (forward_convolutional_shortcut_gpu), likewise a convolution and the yolo
+ * head it feeds (forward_convolutional_yolo_gpu); 0: layer by layer as src/network.c:773-785
+ * does.  Every layer's output buffer is written in both modes and holds the same bits. */
 void network_set_fusion(int on);
 float *layer_output_host(network *net, int i);
 int *layer_indexes_host(network *net, int i);

@@ -154,6 +154,19 @@ void forward_convolutional_shortcut_gpu(const float *input, const float *weights
                                         int activation, const float *add, float *sum_output, float alpha,
                                         float beta, int shortcut_activation);
 
+/* Convolution layer followed by the yolo layer it feeds, in one pass: `output` receives what
+ * forward_convolutional_gpu writes and `yolo_output` what forward_yolo_gpu would make of it
+ * (src/yolo_layer.c:132-148: the copy, with the logistic on x, y, objectness and classes of every
+ * anchor; n must be n_anchors * (5 + classes)).  Replaces the pair forward_convolutional_layer_gpu
+ * + forward_yolo_layer_gpu of a detection head; both buffers hold the bits the two separate
+ * calls write, and the head's own pass over memory disappears.  yolo_output must not alias output. */
+void forward_convolutional_yolo_gpu(const float *input, const float *weights, const float *packed,
+                                    const float *biases, const float *scales,
+                                    const float *rolling_mean, const float *rolling_variance,
+                                    float *output, int batch, int c, int h, int w, int n, int groups,
+                                    int size, int stride, int pad, int batch_normalize, int activation,
+                                    float *yolo_output, int n_anchors, int classes);
+
 /* forward_convolutional_gpu for callers that cannot allocate device memory (code under stream
  * capture, tight serving loops, harnesses that forbid hipMalloc).  No counterpart in the
  * reference.  Same arguments and same result, bit for bit; the call itself makes no hipMalloc /
@@ -272,7 +285,9 @@ void forward_shortcut_gpu(const float *in, const float *add, float *out, int bat
                           int activation);
 
 /* forward_yolo_layer_gpu, inference part (src/yolo_layer.c:347-361 on the GPU; the CPU form
- * src/yolo_layer.c:132-148 defines the result): copy + logistic on x,y,objectness,classes. */
+ * src/yolo_layer.c:132-148 defines the result): copy + logistic on x,y,objectness,classes.  The
+ * logistic is evaluated in single precision (correctly rounded expf, hardware reciprocal): within
+ * 3e-7 absolute of the reference's double evaluation, which made this kernel compute-bound. */
 void forward_yolo_gpu(const float *input, float *output, int batch, int w, int h, int n_anchors,
                       int classes);
 
