@@ -937,6 +937,162 @@ __global__ __launch_bounds__(DN_THREADS) void conv_reduce_kernel(mfma_args a)
     conv_reduce_unit<BM, BN, WM, WN>(a, t, u);
 }
 
+/* ---- first layers: 3 input channels, 3x3, stride 1, pad 1 --------------------------------- */
+/* With K = 27 the general kernel spends its time on the gather (one 4-byte load per column and k,
+ * each with its own index split) and on per-tile index arithmetic, not on its two chunks of MFMAs.
+ * Here a workgroup owns 256 consecutive output pixels of one image and every filter: it copies
+ * the input rows those pixels touch into LDS once (16 bytes per lane, zero columns left and right
+ * and zero rows above and below the image, so no tap needs a border test), keeps the weights in
+ * registers (a lane holds its filter's 14 k of the MFMA's k pairs), and feeds the MFMAs from LDS
+ * with one 4-byte read per pixel and k: address = pixel base + a per-k offset.  K order is the
+ * reference's (channel, ky, kx), padded from 27 to 28.  Accumulators are laid out as in
+ * conv_mfma_kernel (pixel rows, filter columns), so the epilogue is shared.  The layer is bound by
+ * writing its output (32 filters x 416 x 416: 22 MB per image for 0.6 MB read). */
+#define DN_PATCH_FLOATS 8192     /* at most 32 KB for the input rows of a tile */
+#define DN_PATCH_MIN_FLOATS 4096 /* 16 KB: the buffer also turns 16 filters x 256 pixels for the store */
+extern __shared__ __attribute__((aligned(16))) float conv_patch_lds[];
+template <int TM, int C>
+__global__ __launch_bounds__(DN_THREADS, 4) void conv_patch_kernel(mfma_args a)
+{
+    constexpr int K = 9 * C, NS = (K + 1) / 2; /* MFMA k pairs */
+    typedef __attribute__((address_space(3))) void *lds_ptr;
+    float *buf = conv_patch_lds; /* sized by the launch: the tile's input rows (what the geometry needs, so
+                                  * that as many tiles as possible are in flight on a CU: their trips to
+                                  * memory, not their arithmetic, are what takes the time) */
+    __shared__ __attribute__((aligned(16))) float wsm[TM * 32 * K]; /* the weights, as they lie in memory */
+    __shared__ conv_row_t rows_s[TM * 32];
+    const int tid = threadIdx.x, lane = tid & 63, li = lane & 31, kh = lane >> 5;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int W = a.W, H = a.H, P = a.P;
+    const int tiles_per_image = P / 256; /* the host checks P % 256 == 0 */
+    const int b = blockIdx.x / tiles_per_image;
+    const int p0 = (blockIdx.x - b * tiles_per_image) * 256;
+    const int y0 = p0 / W, y1 = (p0 + 255) / W;
+    const int nrows = y1 - y0 + 3, RS = W + 8; /* a row: four zeros, the W pixels, four zeros */
+
+    /* Input rows y0-1 .. y1+1 of every channel, copied by loads that write straight to LDS, 16
+     * bytes per lane: the patch is one flat array of C * nrows * RS / 4 quads cut into wave-loads
+     * of 64 consecutive quads, dealt round-robin to the four waves; lane i of a wave-load owns quad
+     * 64 * segment + i = (channel-row cr, quad qx of the row), walked without divisions.  W is a
+     * multiple of 4, so a quad is either four pixels of one row or padding; quads of padding, of
+     * rows outside the image and past the end of the patch carry an offset beyond the buffer's
+     * range and arrive as zeros. */
+    const __amdgpu_buffer_rsrc_t in_rsrc = __builtin_amdgcn_make_buffer_rsrc(
+        (void *)(a.in + (long)b * C * H * W), 0, C * H * W * 4, 0x00020000);
+    const int RQ = RS >> 2, total = C * nrows * RQ; /* quads per row, quads in all */
+    {
+        int e = wave * 64 + lane;
+        int cr = e / RQ, qx = e - cr * RQ;       /* one division per lane */
+        int ci = cr / nrows, r = cr - ci * nrows;
+        for (int seg = wave; seg * 64 < total; seg += 4) {
+            const int iy = y0 - 1 + r;
+            const bool ok = e < total && (unsigned)iy < (unsigned)H && qx >= 1 && qx < RQ - 1;
+            const unsigned voff = ok ? (unsigned)(((ci * H + iy) * W + 4 * (qx - 1)) * 4) : 0xFFFFFFF0u;
+            __builtin_amdgcn_raw_ptr_buffer_load_lds(in_rsrc, (lds_ptr)&buf[seg * 256], 16, voff, 0, 0, 0);
+            e += 256;
+            qx += 256;
+            while (qx >= RQ) {
+                qx -= RQ;
+                if (++r == nrows) {
+                    r = 0;
+                    ++ci;
+                }
+            }
+        }
+    }
+    /* the weights of all filters, coalesced, then each lane picks its own: filter 32i + li,
+     * k = 2s + kh in (channel, ky, kx) order (rows are 27 floats apart: no bank conflicts) */
+    for (int i = tid; i < TM * 32 * K; i += DN_THREADS) wsm[i] = i < a.M * K ? a.wp[i] : 0.f;
+    if (tid < TM * 32) rows_s[tid] = conv_row(a, tid < a.M ? tid : a.M - 1);
+    __builtin_amdgcn_s_waitcnt(0);
+    __syncthreads();
+
+    float aw[TM][NS];
+    int koff[NS]; /* LDS offset of k relative to the pixel's base (row y - y0, column x) */
+#pragma unroll
+    for (int s = 0; s < NS; ++s) {
+        const int k = 2 * s + kh;
+        const int ci = k / 9, r9 = k - 9 * ci, ky = r9 / 3, kx = r9 - 3 * ky;
+        koff[s] = k < K ? (ci * nrows + ky) * RS + kx + 3 : 0; /* pixel x sits in column x + 4 */
+#pragma unroll
+        for (int i = 0; i < TM; ++i) aw[i][s] = k < K ? wsm[(i * 32 + li) * K + k] : 0.f;
+    }
+
+    f32x16 acc[TM][2];
+#pragma unroll
+    for (int i = 0; i < TM; ++i)
+#pragma unroll
+        for (int j = 0; j < 2; ++j)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
+    int base[2];
+#pragma unroll
+    for (int j = 0; j < 2; ++j) {
+        const int p = p0 + wave * 64 + j * 32 + li;
+        const int y = (int)((unsigned)p / (unsigned)W);
+        base[j] = (y - y0) * RS + (p - y * W);
+    }
+#pragma unroll
+    for (int s = 0; s < NS; ++s) {
+#pragma unroll
+        for (int j = 0; j < 2; ++j) {
+            const float bv = buf[base[j] + koff[s]];
+#pragma unroll
+            for (int i = 0; i < TM; ++i) acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(bv, aw[i][s], acc[i][j], 0, 0, 0);
+        }
+    }
+    /* Tail and store.  The output is what bounds this layer, and memory takes whole kilobytes
+     * better than the 256-byte pieces a wave's own 64 pixels make per filter: the four waves pool
+     * their finished values in LDS, 16 filters x 256 pixels at a time (16-byte quads XOR-swizzled
+     * by the filter), and each wave then stores four filter rows, one contiguous kilobyte per
+     * instruction. */
+    const long out_base = ((long)b * a.M) * P + p0;
+#pragma unroll
+    for (int i = 0; i < TM; ++i) {
+        const conv_row_t row = rows_s[i * 32 + li];
+#pragma unroll
+        for (int hf = 0; hf < 2; ++hf) {
+            __syncthreads(); /* the buffer is free: pixels read (first pass), rows stored (later ones) */
+            if ((li >> 4) == hf) {
+                const int f16 = li & 15;
+#pragma unroll
+                for (int j = 0; j < 2; ++j)
+#pragma unroll
+                    for (int rg = 0; rg < 4; ++rg) {
+                        float4 o;
+                        o.x = conv_tail_one(acc[i][j][rg * 4 + 0], row, conv_f2{a.slope_hi, a.slope_lo});
+                        o.y = conv_tail_one(acc[i][j][rg * 4 + 1], row, conv_f2{a.slope_hi, a.slope_lo});
+                        o.z = conv_tail_one(acc[i][j][rg * 4 + 2], row, conv_f2{a.slope_hi, a.slope_lo});
+                        o.w = conv_tail_one(acc[i][j][rg * 4 + 3], row, conv_f2{a.slope_hi, a.slope_lo});
+                        const int q = wave * 16 + j * 8 + 2 * rg + kh; /* quad of four pixels within the tile */
+                        *(float4 *)&buf[f16 * 256 + ((q ^ f16) << 2)] = o;
+                    }
+            }
+            __syncthreads();
+#pragma unroll
+            for (int t = 0; t < 4; ++t) {
+                const int f16 = wave * 4 + t, m = i * 32 + hf * 16 + f16;
+                const float4 o = *(const float4 *)&buf[f16 * 256 + ((lane ^ f16) << 2)];
+                if (m < a.M) *(float4u *)(a.out + out_base + (long)m * P + 4 * lane) = (float4u){o.x, o.y, o.z, o.w};
+            }
+        }
+    }
+}
+
+/* Floats of LDS a tile's input rows take (0: conv_patch_kernel does not serve the layer). */
+static long conv_patch_floats(int c, int h, int w, int n, int groups, int size, int stride, int pad)
+{
+    if (groups != 1 || c != 3 || size != 3 || stride != 1 || pad != 1 || n > 64) return 0;
+    const long P = (long)h * w;
+    if (P % 256 || w % 4) return 0; /* whole tiles per image; rows are copied 16 bytes at a time */
+    if ((long)3 * h * w * 4 >= (1L << 31)) return 0;
+    const long rows = 255 / w + 2 + 2; /* output rows a tile can touch, plus one above and below */
+    const long floats = 3 * rows * (w + 8);
+    if (floats > DN_PATCH_FLOATS) return 0;
+    /* the copy moves whole wave-loads of 256 floats */
+    return floats < DN_PATCH_MIN_FLOATS ? DN_PATCH_MIN_FLOATS : (floats + 255) / 256 * 256;
+}
+
 /* ---- weight packing ---------------------------------------------------------------------- */
 /* taps > 0 selects the tap-blocked order (taps = size*size, c % 16 == 0): packed row k' holds
  * channel (k'/16/taps)*16 + k'%16 of tap (k'/16) % taps; taps == 0 keeps the reference order. */
@@ -1209,12 +1365,14 @@ extern "C" const char *conv_kernel_name_columns(int n, int c, int groups, int si
         bm = 32;
     }
     if (mode < 0) return "conv_direct_kernel";
+    if (g_algo == 0 && mode == 3 && c == 3 && n <= 64 && columns > 0 && columns % 256 == 0)
+        return n <= 32 ? "conv_patch_kernel<1,3>" : "conv_patch_kernel<2,3>"; /* for the stride-1 pad-1 layers it serves */
     const int bf16 = g_precision == 1 && mode >= 10;
     const int x3 = g_precision == 2 && mode >= 10;
     if (bf16 && bm == 128 && n > 128) bm = 256;
     if (x3 && bm == 128)
         snprintf(name, sizeof name, "conv_mfma_kernel<128,128,128,32,%d,3>", mode);
-    else if (bm == 128 && g_precision == 0 && conv_narrow_tile(columns, n))
+    else if (bm == 128 && g_precision == 0 && columns > 0 && conv_narrow_tile(columns, n))
         snprintf(name, sizeof name, "conv_mfma_kernel<128,64,64,32,%d>", mode);
     else
         snprintf(name, sizeof name, "conv_mfma_kernel<%d,%d,%d,64,%d%s>", bm, bm >= 128 ? 128 : 256,
@@ -1224,7 +1382,7 @@ extern "C" const char *conv_kernel_name_columns(int n, int c, int groups, int si
 
 extern "C" const char *conv_kernel_name(int n, int c, int groups, int size)
 {
-    return conv_kernel_name_columns(n, c, groups, size, 1L << 40);
+    return conv_kernel_name_columns(n, c, groups, size, -1); /* size of the layer unknown: the large-layer kernel */
 }
 
 static float *g_scratch = 0;       /* per-call repack buffer for callers without a packed copy */
@@ -1539,7 +1697,8 @@ static void conv_forward(const float *input, const float *weights, const float *
         return;
     }
 
-    if (g_noalloc && (!packed || (g_precision == 1 && mode == 13))) {
+    const long patch = (g_algo == 0 && mode == 3 && !sum) ? conv_patch_floats(c, h, w, n, groups, size, stride, pad) : 0;
+    if (g_noalloc && !patch && (!packed || (g_precision == 1 && mode == 13))) {
         fprintf(stderr, !packed ? "forward_convolutional_noalloc_gpu: this geometry runs on packed weights; pass the "
                                   "buffer conv_pack_weights_gpu wrote\n"
                                 : "forward_convolutional_noalloc_gpu: the bf16-operand mode stages 3x3 inputs in a "
@@ -1547,7 +1706,7 @@ static void conv_forward(const float *input, const float *weights, const float *
         g_noalloc_error = 1;
         return;
     }
-    if (!packed) {
+    if (!packed && !patch) {
         const size_t need = conv_packed_floats(n, c, groups, size);
         if (need > g_scratch_floats) {
             if (g_scratch) hip_free(g_scratch);
@@ -1622,7 +1781,19 @@ static void conv_forward(const float *input, const float *weights, const float *
         a.in16 = g_stage;
         a.in16_records = (unsigned)(rows * 16 + (long)(w + 1) * 16);
     }
-    if (n <= 32 || a.grouped)
+    if (patch) {
+        /* first layers (3 channels, 3x3): input rows through LDS, weights in registers */
+        a.wp = weights;
+        void *args[] = {&a};
+        const void *kernel = n <= 32 ? (const void *)conv_patch_kernel<1, 3> : (const void *)conv_patch_kernel<2, 3>;
+        const dim3 grid((unsigned)((long)batch * a.P / 256));
+        if (g_prof_start)
+            hip_check_error(hipExtLaunchKernel(kernel, grid, dim3(DN_THREADS), args, (size_t)patch * 4, dn_stream(),
+                                               g_prof_start, g_prof_stop, 0));
+        else
+            hip_check_error(hipLaunchKernel(kernel, grid, dim3(DN_THREADS), args, (size_t)patch * 4, dn_stream()));
+        g_prof_start = g_prof_stop = 0;
+    } else if (n <= 32 || a.grouped)
         launch_tile<32, 256, 32, 64>(a, mode);
     else if (n > 128 && g_precision == 1 && mode >= 10)
         launch_tile<256, 128, 128, 64>(a, mode);

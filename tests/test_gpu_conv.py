@@ -60,6 +60,11 @@ SHAPES = [  # b, c, h, w, n, size, stride, pad, groups, act
     (2, 64, 12, 12, 64, 3, 1, 1, 64, "relu"),       # depthwise: 1 per group
     (2, 48, 9, 9, 96, 3, 1, 1, 3, "leaky"),         # 16 channels -> 32 filters per group: direct kernel
     (2, 96, 9, 9, 96, 3, 1, 1, 2, "leaky"),         # 48 per group: direct kernel
+    (2, 3, 16, 16, 32, 3, 1, 1, 1, "leaky"),        # first-layer kernel (3 channels, pixels a multiple of 256)
+    (1, 3, 32, 24, 16, 3, 1, 1, 1, "leaky"),        # the same with 16 filters (half a filter block)
+    (3, 3, 16, 48, 64, 3, 1, 1, 1, "linear"),       # two filter blocks, tiles of 5.3 rows
+    (1, 3, 64, 20, 20, 3, 1, 1, 1, "relu"),         # ragged filter count, narrow image (13 rows per tile)
+    (2, 3, 8, 512, 8, 3, 1, 1, 1, "leaky"),         # rows longer than a tile
 ]
 
 
