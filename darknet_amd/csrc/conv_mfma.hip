@@ -915,9 +915,11 @@ __global__ __launch_bounds__(DN_THREADS, ((BM == 128 && BF16 != 3) ? 3 : 2)) voi
         if (tid < BM) rows_s[tid] = conv_row(a, m0 + tid < a.M ? m0 + tid : a.M - 1);
         __syncthreads(); /* every wave has read its last operands: the LDS buffers are free */
         float *E = V3 ? S_BUF(wave)
-                   : BM >= 128 ? (BFP ? (wave == 0 ? Bs2 : wave == 1 ? Bs3 : wave == 2 ? Bs0 : Bs1)
-                                       : (wave == 0 ? As0 : wave == 1 ? As1 : wave == 2 ? Bs0 : Bs1))
-                               : (wave < 2 ? Bs0 : Bs1) + (wave & 1) * 2048;
+                   : (BM >= 128 || BN == 64) ? (BFP ? (wave == 0 ? Bs2 : wave == 1 ? Bs3 : wave == 2 ? Bs0 : Bs1)
+                                                    : (wave == 0 ? As0 : wave == 1 ? As1 : wave == 2 ? Bs0 : Bs1))
+                                             : (wave < 2 ? Bs0 : Bs1) + (wave & 1) * 2048;
+        static_assert(BN != 64 || (A_FLOATS >= 32 * 32 * TN && B_FLOATS >= 32 * 32 * TN),
+                      "each operand buffer holds one wave's turn of 32 filters x 32*TN pixels");
         conv_epilogue<TM, TN>(a, acc, E, rows_s, m0, n0, wm0, wn0, lane);
     }
 }
@@ -1347,6 +1349,18 @@ static int conv_mode(int c, int groups, int size, int stride, int pad, long in_b
  * 128-wide tiles than the chip has CUs (batch 1): twice the workgroups before any cut along K,
  * and fewer padded columns (192 instead of 256 for the 169 pixels of a 13x13 image).  Measured on
  * every such layer of yolov3 at batch 1: 8-25% less time than the wide tile at its best split. */
+/* 64x64 tiles (four waves of 32x32) for the smallest layers: those of 33..64 filters whose 64x256
+ * tiles number fewer than the CUs (the early layers at batch 1: 23 instead of 34-37 microseconds for
+ * the 3x3 32->64 layers at 208x208, 7 instead of 15 for 1x1 128->64 at 104x104), and 1x1 layers of
+ * more filters that do not fill the chip with 128x64 tiles either (K up to 1024: 9-10 instead of
+ * 11-12 microseconds each; for the 3x3 layers, with nine times the K, the two tiles tie). */
+static bool conv_small_tile(long columns, int n, int kch)
+{
+    if (g_tune_bn) return g_tune_bn == 1 || (g_tune_bn == 64 && n <= 64);
+    if (n <= 64) return (columns + 255) / 256 < 256;
+    return kch <= 64 && ((columns + 63) / 64) * ((n + 127) / 128) < 256;
+}
+
 static bool conv_narrow_tile(long columns, int n)
 {
     if (g_tune_bn) return g_tune_bn == 64;
@@ -1372,8 +1386,12 @@ extern "C" const char *conv_kernel_name_columns(int n, int c, int groups, int si
     if (bf16 && bm == 128 && n > 128) bm = 256;
     if (x3 && bm == 128)
         snprintf(name, sizeof name, "conv_mfma_kernel<128,128,128,32,%d,3>", mode);
+    else if (bm == 128 && g_precision == 0 && columns > 0 && conv_small_tile(columns, n, (c * size * size + 15) / 16))
+        snprintf(name, sizeof name, "conv_mfma_kernel<64,64,32,32,%d>", mode);
     else if (bm == 128 && g_precision == 0 && columns > 0 && conv_narrow_tile(columns, n))
         snprintf(name, sizeof name, "conv_mfma_kernel<128,64,64,32,%d>", mode);
+    else if (bm == 64 && g_precision == 0 && columns > 0 && conv_small_tile(columns, n, (c * size * size + 15) / 16))
+        snprintf(name, sizeof name, "conv_mfma_kernel<64,64,32,32,%d>", mode);
     else
         snprintf(name, sizeof name, "conv_mfma_kernel<%d,%d,%d,64,%d%s>", bm, bm >= 128 ? 128 : 256,
                  bm == 32 ? 32 : bm == 256 ? 128 : 64, mode, x3 ? ",3" : !bf16 ? "" : mode == 13 ? ",2" : ",1");
@@ -1427,8 +1445,8 @@ extern "C" __attribute__((visibility("hidden"))) void conv_device_setup(void)
 
 extern "C" void conv_set_ksplit(int split, int tile_n)
 {
-    if (split < 0 || (tile_n != 0 && tile_n != 64 && tile_n != 128))
-        dn_fatal("conv_set_ksplit: split >= 0, tile_n 0, 64 or 128");
+    if (split < 0 || (tile_n != 0 && tile_n != 1 && tile_n != 64 && tile_n != 128))
+        dn_fatal("conv_set_ksplit: split >= 0, tile_n 0, 1, 64 or 128");
     g_tune_split = split;
     g_tune_bn = tile_n;
 }
@@ -1459,7 +1477,7 @@ static float *partial_buffer(size_t need)
  * a remainder that would leave most CUs idle for a whole tile time (or, at batch 1, a grid far
  * smaller than the chip) is cut along K into `split` slices each, which conv_reduce_kernel sums.
  * Returns the number of whole tiles; *split = 1 means no tail. */
-static long plan_split(long tiles, int kch, int cus, int *split, double fixed_scale, int bn)
+static long plan_split(long tiles, int kch, int cus, int *split, double fixed_scale, int bm, int bn)
 {
     *split = 1;
     if (g_algo == 3 || cus <= 0) return tiles;
@@ -1478,7 +1496,9 @@ static long plan_split(long tiles, int kch, int cus, int *split, double fixed_sc
          * per 16-wide chunk, r workgroups sharing a CU take r * `shared`; an unsplit tile pays its
          * epilogue (2.4), a split one the second launch (5) and, per slice, the extra partial
          * traffic of both launches. */
-        const double lone = bn <= 64 ? 0.55 : 1.1, shared = bn <= 64 ? 0.45 : 0.9, per_slice = bn <= 64 ? 0.4 : 0.8;
+        const double work = (double)bm * bn / (128.0 * 128.0); /* MFMAs per chunk against the 128x128 tile */
+        const double lone = work <= 0.25 ? 0.28 : work <= 0.5 ? 0.55 : 1.1, shared = work <= 0.25 ? 0.23 : work <= 0.5 ? 0.45 : 0.9,
+                     per_slice = work <= 0.25 ? 0.22 : work <= 0.5 ? 0.4 : 0.8;
         double best = kch * lone + 2.4;
         const int max_s = kch / 2 < 32 ? kch / 2 : 32;
         for (int s = 2; s <= max_s; ++s) {
@@ -1520,7 +1540,7 @@ static conv_kernel_t pick_kernel(int mode, int bf16, int x3)
     if (BM > 128 && !bf16) dn_fatal("conv dispatch: the 256-row tile is only built for the bf16-operand mode");
     if (NO_X3 && x3) dn_fatal("conv dispatch: the three-piece mode runs 128x128 tiles with 128x32 wave tiles");
     if (X3_ONLY && !x3) dn_fatal("conv dispatch: the 128x32 wave tile is only built for the three-piece mode");
-    if (FP32_ONLY && (bf16 || x3)) dn_fatal("conv dispatch: the 128x64 tile is only built for fp32 operands");
+    if (FP32_ONLY && (bf16 || x3)) dn_fatal("conv dispatch: the 64-column tiles are only built for fp32 operands");
     if constexpr (FP32_ONLY) {
         switch (mode) {
         case 11: return conv_mfma_kernel<BM, BN, WM, WN, 11>;
@@ -1578,7 +1598,7 @@ static void launch_tile(const mfma_args &a0, int mode)
     if (!kernel) dn_fatal("conv dispatch: no kernel for this tile shape and mode");
     int split = 1;
     /* a bf16 chunk takes a small fraction of an fp32 chunk's time; the fixed costs do not shrink */
-    const long whole = plan_split(total, a.KCH, g_cus, &split, bf16 ? 6.0 : x3 ? 2.0 : 1.0, BN);
+    const long whole = plan_split(total, a.KCH, g_cus, &split, bf16 ? 6.0 : x3 ? 2.0 : 1.0, BM, BN);
     const long tail = total - whole;
     a.whole_tiles = (int)whole;
     a.split = split;
@@ -1797,6 +1817,8 @@ static void conv_forward(const float *input, const float *weights, const float *
         launch_tile<32, 256, 32, 64>(a, mode);
     else if (n > 128 && g_precision == 1 && mode >= 10)
         launch_tile<256, 128, 128, 64>(a, mode);
+    else if (g_precision == 0 && conv_small_tile(a.Ntotal, n, a.KCH))
+        launch_tile<64, 64, 32, 32>(a, mode);
     else if (n <= 64)
         launch_tile<64, 256, 64, 64>(a, mode);
     else if (g_precision == 2 && mode >= 10)

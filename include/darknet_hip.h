@@ -222,7 +222,8 @@ void conv_set_algo(int algo);
  * tiles would leave most of the chip idle, those tiles are cut along K into slices that a second
  * launch sums in slice order.
  *   split   0 = the cost model decides, n > 0 = n slices for every such tile (1 = none)
- *   tile_n  0 = automatic, 64 or 128 = column width of the tile of layers with more than 64 filters */
+ *   tile_n  0 = automatic, 64 or 128 = column width of the tile of layers with more than 64 filters
+ *           (64 also gives layers of 33..64 filters the 64x64 tile), 1 = 64x64 tiles for every layer */
 void conv_set_ksplit(int split, int tile_n);
 
 /* Operand precision of the tap-blocked MFMA convolution kernels (channels a multiple of 16, 1x1 or
