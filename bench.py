@@ -360,6 +360,11 @@ def measure(L, api, synth, workload, batch, precision, steps, warmup, per_layer=
                                             and not prev["xnor"] and prev["n"] == Ly["n"] * (5 + Ly["classes"])
                                             and (prev["out_w"], prev["out_h"]) == (Ly["w"], Ly["h"]))
         row["gbs"] = row["bytes"] / ms / 1e6 if ms > 0 and not row["fused"] else 0.0
+        if row["fused"]:
+            # the conv kernel reads the shortcut's second operand and writes the fused layer's output
+            # beside its own (both layer outputs stay observable, as in the reference)
+            extra = 4 * Ly["batch"] * Ly["outputs"] * (2 if Ly["type"] == "shortcut" else 1)
+            kernels[rows[i - 1]["kernel"]]["fused_bytes"] = kernels[rows[i - 1]["kernel"]].get("fused_bytes", 0.0) + extra
         rows.append(row)
     dom_name, dom = max(kernels.items(), key=lambda kv: kv[1]["ms"])
     # the kernel's own duration when every one of its launches was stamped; else (a kernel outside
@@ -372,7 +377,8 @@ def measure(L, api, synth, workload, batch, precision, steps, warmup, per_layer=
               "avg_launch_ms": round(dom_ms / dom["launches"], 4),
               "timing": "events on the kernel's dispatch" if stamped else "events between layers",
               "avg_layer_interval_ms": round(dom["ms"] / dom["launches"], 4),
-              "traffic": profiled_traffic(workload, batch, dom_name)}
+              "traffic": profiled_traffic(workload, batch, dom_name),
+              "algorithmic_bytes_per_launch": round((dom["bytes"] + dom.get("fused_bytes", 0.0)) / dom["launches"])}
     if dom_name == "xnor_conv_kernel":
         # XNOR layers keep fp32 activations in memory: HBM bounds them (bit-ops reported beside it;
         # one multiply-add of the fp32 formulation is one XNOR + one popcount bit)

@@ -52,7 +52,7 @@ SIGNATURES = {
     "forward_convolutional_noalloc_gpu": (i, [V] * 8 + [i] * 11),
     "forward_convolutional_yolo_gpu": (None, [V] * 8 + [i] * 11 + [V, i, i]),
     "conv_packed_floats": (z, [i, i, i, i]), "conv_pack_weights_gpu": (None, [V, V, i, i, i, i]),
-    "conv_set_algo": (None, [i]), "conv_set_ksplit": (None, [i, i]),
+    "conv_set_algo": (None, [i]), "conv_set_ksplit": (None, [i, i]), "conv_set_bands": (None, [i]),
     "xnor_weight_words": (z, [i, i, i]), "xnor_input_words": (z, [i, i, i, i]),
     "xnor_pack_weights_gpu": (None, [V, V, V, i, i, i]),
     "xnor_pack_input_gpu": (None, [V, V, i, i, i, i]),

@@ -226,6 +226,12 @@ void conv_set_algo(int algo);
  *           (64 also gives layers of 33..64 filters the 64x64 tile), 1 = 64x64 tiles for every layer */
 void conv_set_ksplit(int split, int tile_n);
 
+/* Tuning hook of the tile order (no counterpart in the reference).  The filter tiles of a layer are
+ * cut into `bands` groups (1, 2, 4 or 8; halved until it divides the number of filter tiles); an
+ * XCD's consecutive share of the tiles then reads 1/bands of the weights and bands/8 of the input
+ * through its private L2.  0 = automatic: the count that minimises weights*8/bands + input*bands. */
+void conv_set_bands(int bands);
+
 /* Operand precision of the tap-blocked MFMA convolution kernels (channels a multiple of 16, 1x1 or
  * 3x3 pad 1; grouped 32-filter tiles):
  *   0  fp32 (default; the reference's arithmetic on v_mfma_f32_32x32x2_f32);
