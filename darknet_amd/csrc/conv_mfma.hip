@@ -1355,25 +1355,33 @@ static int conv_mode(int c, int groups, int size, int stride, int pad, long in_b
  * 128-wide tiles than the chip has CUs (batch 1): twice the workgroups before any cut along K,
  * and fewer padded columns (192 instead of 256 for the 169 pixels of a 13x13 image).  Measured on
  * every such layer of yolov3 at batch 1: 8-25% less time than the wide tile at its best split. */
-/* 64x64 tiles (four waves of 32x32) for the smallest layers: those of 33..64 filters whose 64x256
- * tiles number fewer than the CUs (the early layers at batch 1: 23 instead of 34-37 microseconds for
- * the 3x3 32->64 layers at 208x208, 7 instead of 15 for 1x1 128->64 at 104x104), and 1x1 layers of
- * more filters that do not fill the chip with 128x64 tiles either (K up to 1024: 9-10 instead of
- * 11-12 microseconds each; for the 3x3 layers, with nine times the K, the two tiles tie). */
-static bool conv_small_tile(long columns, int n, int kch)
+/* 64x64 tiles (four waves of 32x32, eight workgroups per CU) for layers of 33..64 filters and for
+ * 1x1 layers of any more: with so little K per tile (16..64 chunks) the load latency at the start
+ * of a tile and its epilogue weigh as much as the MFMAs, and many small workgroups per CU overlap
+ * them better than three large ones.  Measured at batch 64 (min of three interleaved runs): 3x3
+ * 32->64 at 208x208 898 against 974 microseconds with 64x256 tiles, 1x1 128->64 at 104x104 137
+ * against 161, 1x1 1024->512 at 13x13 104 against 112; at batch 1 (tiles fewer than CUs) 23 instead
+ * of 34-37 microseconds for the 3x3 32->64 layers and 9-10 instead of 11-12 for the 1x1 layers. */
+static bool conv_small_tile(long columns, int n, int kch, int size)
 {
+    (void)columns;
+    (void)kch;
     if (g_tune_bn) return g_tune_bn == 1 || (g_tune_bn == 64 && n <= 64);
-    if (n <= 64) return (columns + 255) / 256 < 256;
-    return kch <= 64 && ((columns + 63) / 64) * ((n + 127) / 128) < 256;
+    return n <= 64 || size == 1;
 }
 
-static bool conv_narrow_tile(long columns, int n)
+/* 128x64 tiles for the other layers when the wide tile would not fill the chip, and for 3x3
+ * layers of up to 256 input channels in any case (four workgroups per CU instead of three:
+ * 756 against 772 microseconds for 256->512 at 26x26, batch 64, 805 against 830 for 64->128 at
+ * 104x104).  With 512 input channels the wide tile wins (779 against 857 at 13x13): every tile
+ * streams 18 MB of weights, and the narrow tile reads them twice as often per output. */
+static bool conv_narrow_tile(long columns, int n, int kch, int size)
 {
     if (g_tune_bn) return g_tune_bn == 64;
+    if (size == 3 && kch <= 144) return true;
     const long tiles = ((columns + 127) / 128) * ((n + 127) / 128);
     return tiles < 256;
 }
-
 
 extern "C" const char *conv_kernel_name_columns(int n, int c, int groups, int size, long columns)
 {
@@ -1392,11 +1400,11 @@ extern "C" const char *conv_kernel_name_columns(int n, int c, int groups, int si
     if (bf16 && bm == 128 && n > 128) bm = 256;
     if (x3 && bm == 128)
         snprintf(name, sizeof name, "conv_mfma_kernel<128,128,128,32,%d,3>", mode);
-    else if (bm == 128 && g_precision == 0 && columns > 0 && conv_small_tile(columns, n, (c * size * size + 15) / 16))
+    else if (bm == 128 && g_precision == 0 && columns > 0 && conv_small_tile(columns, n, (c * size * size + 15) / 16, size))
         snprintf(name, sizeof name, "conv_mfma_kernel<64,64,32,32,%d>", mode);
-    else if (bm == 128 && g_precision == 0 && columns > 0 && conv_narrow_tile(columns, n))
+    else if (bm == 128 && g_precision == 0 && columns > 0 && conv_narrow_tile(columns, n, (c * size * size + 15) / 16, size))
         snprintf(name, sizeof name, "conv_mfma_kernel<128,64,64,32,%d>", mode);
-    else if (bm == 64 && g_precision == 0 && columns > 0 && conv_small_tile(columns, n, (c * size * size + 15) / 16))
+    else if (bm == 64 && g_precision == 0 && columns > 0 && conv_small_tile(columns, n, (c * size * size + 15) / 16, size))
         snprintf(name, sizeof name, "conv_mfma_kernel<64,64,32,32,%d>", mode);
     else
         snprintf(name, sizeof name, "conv_mfma_kernel<%d,%d,%d,64,%d%s>", bm, bm >= 128 ? 128 : 256,
@@ -1498,7 +1506,7 @@ static long plan_split(long tiles, int kch, int cus, int *split, double fixed_sc
         return *split > 1 ? whole : tiles;
     }
     if (tail * 10 >= (long)cus * 9) return tiles; /* a nearly full round: leave it */
-    if (whole == 0 && fixed_scale == 1.0) {
+    if (whole == 0 && (fixed_scale == 1.0 || bn == 64)) {
         /* The layer does not fill the chip even once (batch 1).  Times in microseconds, fitted to a
          * sweep of the split factor over the layers of yolov3 at batch 1: a workgroup alone on its
          * CU cannot hide its LDS reads and barriers behind another one's MFMAs and takes `lone`
@@ -1628,7 +1636,8 @@ static void launch_tile(const mfma_args &a0, int mode)
     if (!kernel) dn_fatal("conv dispatch: no kernel for this tile shape and mode");
     int split = 1;
     /* a bf16 chunk takes a small fraction of an fp32 chunk's time; the fixed costs do not shrink */
-    const long whole = plan_split(total, a.KCH, g_cus, &split, bf16 ? 6.0 : x3 ? 2.0 : 1.0, BM, BN);
+    /* ... and a chunk of a 64-column tile is half or a quarter of the 128x128 chunk the fixed costs are counted in */
+    const long whole = plan_split(total, a.KCH, g_cus, &split, bf16 ? 6.0 : x3 ? 2.0 : BN == 64 ? 16384.0 / (BM * BN) : 1.0, BM, BN);
     const long tail = total - whole;
     a.whole_tiles = (int)whole;
     a.split = split;
@@ -1848,14 +1857,14 @@ static void conv_forward(const float *input, const float *weights, const float *
         launch_tile<32, 256, 32, 64>(a, mode);
     else if (n > 128 && g_precision == 1 && mode >= 10)
         launch_tile<256, 128, 128, 64>(a, mode);
-    else if (g_precision == 0 && conv_small_tile(a.Ntotal, n, a.KCH))
+    else if (g_precision == 0 && conv_small_tile(a.Ntotal, n, a.KCH, size))
         launch_tile<64, 64, 32, 32>(a, mode);
     else if (n <= 64)
         launch_tile<64, 256, 64, 64>(a, mode);
     else if (g_precision == 2 && mode >= 10)
         /* four waves side by side, 128 rows x 32 columns each: no two waves split the same activations */
         launch_tile<128, 128, 128, 32>(a, mode);
-    else if (g_precision == 0 && conv_narrow_tile(a.Ntotal, n))
+    else if (g_precision == 0 && conv_narrow_tile(a.Ntotal, n, a.KCH, size))
         launch_tile<128, 64, 64, 32>(a, mode);
     else
         launch_tile<128, 128, 64, 64>(a, mode);
