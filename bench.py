@@ -359,8 +359,11 @@ def measure(L, api, synth, workload, batch, precision, steps, warmup, per_layer=
         row["fused"] = row["fused"] or bool(Ly["type"] == "yolo" and prev and prev["type"] == "convolutional"
                                             and not prev["xnor"] and prev["n"] == Ly["n"] * (5 + Ly["classes"])
                                             and (prev["out_w"], prev["out_h"]) == (Ly["w"], Ly["h"]))
+        # a route of one source is a view of that source's buffer: no launch, no traffic
+        view = Ly["type"] == "route" and len(Ly.get("input_layers", [])) == 1
+        row["fused"] = row["fused"] or view
         row["gbs"] = row["bytes"] / ms / 1e6 if ms > 0 and not row["fused"] else 0.0
-        if row["fused"]:
+        if row["fused"] and not view:
             # the conv kernel reads the shortcut's second operand and writes the fused layer's output
             # beside its own (both layer outputs stay observable, as in the reference)
             extra = 4 * Ly["batch"] * Ly["outputs"] * (2 if Ly["type"] == "shortcut" else 1)
@@ -414,7 +417,7 @@ def measure(L, api, synth, workload, batch, precision, steps, warmup, per_layer=
         mem = {"ms_per_step": round(mm, 4), "gbs": round(mb / mm / 1e6, 1), "frac_of_hbm_peak": round(mb / mm / 1e6 / PEAK_HBM_GBS, 4)}
         log(f"[{workload} b{batch}] memory-bound layers: {mm:.3f} ms/step, {mb / mm / 1e6:.0f} GB/s "
             f"({mb / mm / 1e6 / PEAK_HBM_GBS:.1%} of HBM peak; {sum(r['fused'] for r in rows)} shortcuts "
-            f"and yolo heads run inside the preceding convolution and are not counted); conv layers {conv_ms:.3f} ms/step, "
+            f"and yolo heads that run inside the preceding convolution and one-source routes, which are views, are not counted); conv layers {conv_ms:.3f} ms/step, "
             f"{conv_tflops:.1f} TFLOP/s")
     net.free()
     return {"value": round(value, 2), "ms_per_step": round(ms_per_step, 4), "batch": batch,

@@ -216,6 +216,12 @@ static layer parse_route(cfg_section *o, size_params p, network *net)
     }
     r = make_route_layer(p.batch, n, layers, sizes);
     first = net->layers[layers[0]];
+    if (n == 1 && r.output_gpu && first.output_gpu) {
+        /* one source: the reference copies it (src/route_layer.c:74-87); here the layer's output is a
+         * view of the source's buffer - the same values at no cost (free_network knows) */
+        hip_free(r.output_gpu);
+        r.output_gpu = first.output_gpu;
+    }
     r.out_w = first.out_w;
     r.out_h = first.out_h;
     r.out_c = first.out_c;

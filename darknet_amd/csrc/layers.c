@@ -213,6 +213,7 @@ void forward_route_layer_gpu(layer l, network net)
     int i;
     if (l.n > 8) dn_fatal("route layer: more than 8 sources");
     for (i = 0; i < l.n; ++i) srcs[i] = net.layers[l.input_layers[i]].output_gpu;
+    if (l.n == 1 && srcs[0] == l.output_gpu) return; /* a view of its one source (parse_network_cfg) */
     forward_route_gpu(srcs, l.input_sizes, l.n, l.output_gpu, l.batch);
 }
 

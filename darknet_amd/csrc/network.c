@@ -27,7 +27,12 @@ void free_network(network *net)
 {
     int i;
     if (!net) return;
-    for (i = 0; i < net->n; ++i) free_layer(net->layers[i]);
+    for (i = 0; i < net->n; ++i) {
+        layer l = net->layers[i];
+        /* a route of one source may be a view of that source's buffer, which its owner frees */
+        if (l.type == ROUTE && l.n == 1 && l.output_gpu == net->layers[l.input_layers[0]].output_gpu) l.output_gpu = 0;
+        free_layer(l);
+    }
     free(net->layers);
     free(net->input);
     free(net->seen);

@@ -182,6 +182,25 @@ def test_set_batch_network_shrinks_and_grows_back(dn):
     net.free()
 
 
+def test_one_source_route_is_a_view_of_its_source(dn):
+    """`[route] layers=-4` copies one layer in the reference (src/route_layer.c:74-87); here the
+    route's output is the source's buffer: the same bits, no launch, and the two-source routes of the
+    same network still concatenate."""
+    net = api.Network(cfg_text=cfgs.yolov3(2, 160))
+    fill_params(net.set_conv, net.layers)
+    x = synth.uniform01(23, net.inputs * 2)
+    net.predict(x)
+    seen = 0
+    for i, L in enumerate(net.layers):
+        if L["type"] != "route":
+            continue
+        parts = [net.layer_output(j).reshape(2, -1) for j in L["input_layers"]]
+        assert np.array_equal(net.layer_output(i).reshape(2, -1), np.concatenate(parts, axis=1)), i
+        seen += len(parts) == 1
+    assert seen == 2
+    net.free()
+
+
 def test_shortcut_fusion_changes_no_bit(dn):
     """forward_network_device folds each residual add into the convolution before it; with the
     fusion switched off every layer output must hold the same bits."""
