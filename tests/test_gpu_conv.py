@@ -141,6 +141,46 @@ def test_conv_random_geometries(dn, orc, b, c, h, w, n, size, stride, pad, group
     assert norm_err(got, want) <= REL_TOL, dn.conv_kernel_name(n, c, groups, size)
 
 
+TILE_CASES = [  # b, c, h, w, n, size, stride: enough columns for whole rounds of tiles plus a K-split tail
+    (24, 64, 40, 40, 160, 3, 1),     # ragged filter tiles, 3x3 tap-blocked
+    (24, 96, 40, 40, 64, 1, 1),      # up to 64 filters, 1x1
+    (16, 80, 52, 52, 192, 1, 1),     # 1x1, more than 64 filters
+    (12, 20, 36, 36, 48, 3, 2),      # reference K order (c % 16 != 0), stride 2
+]
+
+
+@pytest.mark.parametrize("b,c,h,w,n,size,stride", TILE_CASES)
+def test_every_tile_shape_split_and_band_count_computes_the_same_layer(dn, orc, b, c, h, w, n, size, stride):
+    """The tuning hooks pick the tile (0 = the library's rule, 128 = wide, 64 = narrow, 1 = 64x64),
+    the K-split factor and the band count of the tile order; none may change a layer beyond the
+    summation order over K.  Image 0 and the last image against the checker, every variant against
+    the default."""
+    pad = size // 2
+    x = synth.uniform(41, b * c * h * w).reshape(b, c, h, w)
+    wt = synth.conv_weights(42, n, c, size)
+    bias, sc, mu, var = synth.bn_random(43, n)
+    kw = dict(n=n, size=size, stride=stride, pad=pad, groups=1)
+    base = run_conv(dn, x, wt, bias, sc, mu, var, bn=1, act="leaky", **kw)
+    for k in (0, b - 1):
+        want = orc.conv(x[k:k + 1], wt, bias, sc, mu, var, batch_normalize=1, activation="leaky", **kw)
+        assert norm_err(base[k:k + 1], want) <= REL_TOL, k
+    names = set()
+    try:
+        for tile_n in (0, 128, 64, 1):
+            for split in (0, 1, 3):
+                for bands in (0, 1, 2, 8):
+                    dn.conv_set_ksplit(split, tile_n)
+                    dn.conv_set_bands(bands)
+                    oh = (h + 2 * pad - size) // stride + 1
+                    names.add(dn.conv_kernel_name_columns(n, c, 1, size, b * oh * oh))
+                    got = run_conv(dn, x, wt, bias, sc, mu, var, bn=1, act="leaky", **kw)
+                    assert norm_err(got, base) <= 2e-5, (tile_n, split, bands)
+    finally:
+        dn.conv_set_ksplit(0, 0)
+        dn.conv_set_bands(0)
+    assert len(names) >= 2      # the hooks did switch kernels
+
+
 def test_mfma_kernel_agrees_with_direct_kernel_and_unpacked_call(dn):
     b, c, h, w, n = 2, 64, 20, 20, 96
     x = synth.uniform(1, b * c * h * w).reshape(b, c, h, w)
