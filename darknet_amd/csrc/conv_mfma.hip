@@ -413,9 +413,13 @@ __device__ __forceinline__ void conv_reduce_unit(const mfma_args &a, int t, int 
  * pre-split into three packed copies, the activations split in registers from the fp32 LDS tile,
  * and a product is the six piece-products down to 2^-16 relative (hi*hi, hi*mid, mid*hi, hi*lo,
  * lo*hi, mid*mid; the three dropped ones are below 2^-24), accumulated in fp32. */
-template <int BM, int BN, int WM, int WN, int MODE, int BF16 = 0>
+template <int BM, int BN, int WM, int WN, int MODE_V, int BF16 = 0>
 __global__ __launch_bounds__(DN_THREADS, ((BM == 128 && BF16 != 3) ? 3 : 2)) void conv_mfma_kernel(mfma_args a)
 {
+    /* MODE_V = K order and kernel size, plus 100 for the variant that serves launches too small to
+     * fill the chip (see the two forms of the fp32 loop below) */
+    constexpr int MODE = MODE_V % 100;
+    constexpr bool SPARSE_LAUNCH = MODE_V >= 100;
     constexpr int TM = WM / 32, TN = WN / 32;
     constexpr int WAVES_N = BN / WN;
     static_assert((BM / WM) * (BN / WN) == 4, "four waves per workgroup");
@@ -888,6 +892,32 @@ __global__ __launch_bounds__(DN_THREADS, ((BM == 128 && BF16 != 3) ? 3 : 2)) voi
             if (kc + 2 < kc_end) bstep(kc + 2, 2, 0);
             if (kc + 3 < kc_end) bstep(kc + 3, 3, 1);
         }
+    } else if constexpr (!BF16 && !X3 && BM >= 128 && !SPARSE_LAUNCH) {
+        /* fp32, 128-row tiles in launches that fill the chip: the step with the number of chunks still
+         * to come as a run-time scalar instead of a peeled last chunk.  The compiler then keeps 71 (128x64)
+         * and 115 (128x128) vector registers live instead of 102 and 168, so a CU holds five and four
+         * workgroups instead of four and three, and its matrix pipe idles less while one of them is in
+         * its prologue or epilogue: 2-3% less time per 3x3 layer at batch 64, 12% on 512->1024 at 13x13
+         * with the 128x64 tile.  A workgroup alone on its CU (batch 1) is 1-4% faster with the peeled
+         * form below, which the +100 variants keep; so are the 64- and 32-row tiles (no more workgroups
+         * fit: 64x64 already holds eight). */
+        auto fstep = [&](int kcur, int buf) {
+            const int rem = kc_end - 1 - kcur; /* chunks after this one (wave-uniform) */
+            read_operands(buf, 0);
+            __builtin_amdgcn_sched_barrier(0);
+            if (rem >= 1) load_chunk(kcur + 1, buf ^ 1);
+            __builtin_amdgcn_sched_barrier(0);
+            mfma_chunk(0);
+            __builtin_amdgcn_sched_barrier(0);
+            if (rem >= 1) {
+                __builtin_amdgcn_s_waitcnt(0);
+                __syncthreads();
+            }
+        };
+        for (int kc = kc_begin; kc < kc_end; kc += 2) {
+            fstep(kc, 0);
+            if (kc + 1 < kc_end) fstep(kc + 1, 1);
+        }
     } else {
     int kc = kc_begin;
     /* two chunks per trip so the LDS buffer index is a compile-time constant in each half */
@@ -1331,6 +1361,7 @@ extern "C" void conv_profile_next(void *start_event, void *stop_event)
 extern "C" int conv_profile_pending(void) { return g_prof_start != 0; }
 
 static int g_algo = 0;
+static int g_cus = 0; /* compute units of the current device (conv_device_setup) */
 /* Tuning and test hooks of the K-split (conv_set_ksplit): 0 / default = automatic. */
 static int g_tune_split = 0;   /* > 0: this many slices for every tail tile (1 = none) */
 static int g_tune_bn = 0;      /* 64 or 128: column width of the 128-row fp32 tile */
@@ -1370,15 +1401,14 @@ static bool conv_small_tile(long columns, int n, int kch, int size)
     return n <= 64 || size == 1;
 }
 
-/* 128x64 tiles for the other layers when the wide tile would not fill the chip, and for 3x3
- * layers of up to 256 input channels in any case (four workgroups per CU instead of three:
- * 756 against 772 microseconds for 256->512 at 26x26, batch 64, 805 against 830 for 64->128 at
- * 104x104).  With 512 input channels the wide tile wins (779 against 857 at 13x13): every tile
- * streams 18 MB of weights, and the narrow tile reads them twice as often per output. */
+/* 128x64 tiles (five workgroups per CU) for every other 3x3 layer, and for any layer whose 128x128
+ * tiles would number fewer than the CUs.  Measured at batch 64 against the 128x128 tile (four per CU):
+ * 742 against 762 microseconds for 256->512 at 26x26, 748 against 774 for 128->256 at 52x52, 777
+ * against 803 for 64->128 at 104x104, 749 against 784 for 512->1024 at 13x13. */
 static bool conv_narrow_tile(long columns, int n, int kch, int size)
 {
     if (g_tune_bn) return g_tune_bn == 64;
-    if (size == 3 && kch <= 144) return true;
+    if (size == 3) return true;
     const long tiles = ((columns + 127) / 128) * ((n + 127) / 128);
     return tiles < 256;
 }
@@ -1402,8 +1432,11 @@ extern "C" const char *conv_kernel_name_columns(int n, int c, int groups, int si
         snprintf(name, sizeof name, "conv_mfma_kernel<128,128,128,32,%d,3>", mode);
     else if (bm == 128 && g_precision == 0 && columns > 0 && conv_small_tile(columns, n, (c * size * size + 15) / 16, size))
         snprintf(name, sizeof name, "conv_mfma_kernel<64,64,32,32,%d>", mode);
-    else if (bm == 128 && g_precision == 0 && columns > 0 && conv_narrow_tile(columns, n, (c * size * size + 15) / 16, size))
-        snprintf(name, sizeof name, "conv_mfma_kernel<128,64,64,32,%d>", mode);
+    else if (bm == 128 && g_precision == 0 && columns > 0 && conv_narrow_tile(columns, n, (c * size * size + 15) / 16, size)) {
+        const long tiles = ((columns + 63) / 64) * ((n + 127) / 128);
+        const int sparse = tiles < (g_cus > 0 ? g_cus : 256) && mode >= 11; /* the variant of launches that do not fill the chip */
+        snprintf(name, sizeof name, "conv_mfma_kernel<128,64,64,32,%d>", mode + 100 * sparse);
+    }
     else if (bm == 64 && g_precision == 0 && columns > 0 && conv_small_tile(columns, n, (c * size * size + 15) / 16, size))
         snprintf(name, sizeof name, "conv_mfma_kernel<64,64,32,32,%d>", mode);
     else
@@ -1422,7 +1455,6 @@ static size_t g_scratch_floats = 0;
 
 static float *g_partial = 0; /* K-slice accumulators of tail tiles, grown on demand */
 static size_t g_partial_floats = 0;
-static int g_cus = 0;
 
 /* ---- allocation-free calls ----------------------------------------------------------------
  * forward_convolutional_noalloc_gpu serves callers that cannot allocate device memory (stream
@@ -1549,7 +1581,7 @@ typedef void (*conv_kernel_t)(mfma_args);
 
 /* The kernel instance for a tile shape, K order and precision; null when it is not built. */
 template <int BM, int BN, int WM, int WN>
-static conv_kernel_t pick_kernel(int mode, int bf16, int x3)
+static conv_kernel_t pick_kernel(int mode, int bf16, int x3, int sparse)
 {
     constexpr bool X3_ONLY = WM == 128 && WN == 32; /* the 128x32 wave tile is built for the three-piece mode alone ... */
     constexpr bool NO_X3 = BM == 128 && WN == 64;   /* ... which never runs the 128x128 tile with 64x64 wave tiles */
@@ -1559,6 +1591,10 @@ static conv_kernel_t pick_kernel(int mode, int bf16, int x3)
     if (X3_ONLY && !x3) dn_fatal("conv dispatch: the 128x32 wave tile is only built for the three-piece mode");
     if (FP32_ONLY && (bf16 || x3)) dn_fatal("conv dispatch: the 64-column tiles are only built for fp32 operands");
     if constexpr (FP32_ONLY) {
+        if constexpr (BM == 128) {
+            if (sparse && mode == 11) return conv_mfma_kernel<BM, BN, WM, WN, 111>;
+            if (sparse && mode == 13) return conv_mfma_kernel<BM, BN, WM, WN, 113>;
+        }
         switch (mode) {
         case 11: return conv_mfma_kernel<BM, BN, WM, WN, 11>;
         case 13: return conv_mfma_kernel<BM, BN, WM, WN, 13>;
@@ -1632,13 +1668,13 @@ static void launch_tile(const mfma_args &a0, int mode)
     g_cus = g_cus_dev[dev];
     const int bf16 = g_precision == 1 && mode >= 10;
     const int x3 = g_precision == 2 && mode >= 10;
-    const conv_kernel_t kernel = pick_kernel<BM, BN, WM, WN>(mode, bf16, x3);
-    if (!kernel) dn_fatal("conv dispatch: no kernel for this tile shape and mode");
     int split = 1;
     /* a bf16 chunk takes a small fraction of an fp32 chunk's time; the fixed costs do not shrink */
     /* ... and a chunk of a 64-column tile is half or a quarter of the 128x128 chunk the fixed costs are counted in */
     const long whole = plan_split(total, a.KCH, g_cus, &split, bf16 ? 6.0 : x3 ? 2.0 : BN == 64 ? 16384.0 / (BM * BN) : 1.0, BM, BN);
     const long tail = total - whole;
+    const conv_kernel_t kernel = pick_kernel<BM, BN, WM, WN>(mode, bf16, x3, total < g_cus);
+    if (!kernel) dn_fatal("conv dispatch: no kernel for this tile shape and mode");
     a.whole_tiles = (int)whole;
     a.split = split;
     a.per_xcd = (int)((whole + 7) / 8);
