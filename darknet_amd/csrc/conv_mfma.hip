@@ -839,7 +839,26 @@ __global__ __launch_bounds__(DN_THREADS, ((BM == 128 && BF16 != 3) ? 3 : 2)) voi
      *      consumed that buffer); the two swap places for the tiles with 256 columns
      *   3. the MFMAs of chunk kc
      *   4. wait for this wave's loads (vmcnt), barrier: chunk kc+1 is now visible to all waves */
+    /* loads a wave issues per chunk in the fp32 kernels, and the MFMAs of the chunk that go in front of each */
+    constexpr int LPC_F = A_PER_WAVE + 4 * NG_PER_WAVE;
+    constexpr int MFMA_PER_LOAD = (8 * TM * TN) / (LPC_F + 1) > 0 ? (8 * TM * TN) / (LPC_F + 1) : 1;
     auto step = [&](int kc_next, int buf) {
+        if constexpr (!BF16) {
+            /* fp32: the next chunk's loads are issued between this chunk's MFMAs */
+            read_operands(buf, 0);
+            __builtin_amdgcn_sched_barrier(0);
+            load_chunk(kc_next, buf ^ 1);
+            mfma_chunk(0);
+#pragma unroll
+            for (int g = 0; g < LPC_F; ++g) {
+                __builtin_amdgcn_sched_group_barrier(0x008, MFMA_PER_LOAD, 0);
+                __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);
+            }
+            __builtin_amdgcn_sched_barrier(0);
+            __builtin_amdgcn_s_waitcnt(0);
+            __syncthreads();
+            return;
+        }
         /* the 128-row tiles gain 1-5% from having their reads under way while the loads are issued;
          * the 256-column tiles, with twice the loads per wave, lose 7% and keep loads first */
         if constexpr (BM >= 128) {
@@ -905,9 +924,15 @@ __global__ __launch_bounds__(DN_THREADS, ((BM == 128 && BF16 != 3) ? 3 : 2)) voi
             const int rem = kc_end - 1 - kcur; /* chunks after this one (wave-uniform) */
             read_operands(buf, 0);
             __builtin_amdgcn_sched_barrier(0);
-            if (rem >= 1) load_chunk(kcur + 1, buf ^ 1);
-            __builtin_amdgcn_sched_barrier(0);
+            /* the next chunk's loads go between this chunk's MFMAs (the last step requests its own
+             * chunk again: no branch inside the schedule region) */
+            load_chunk(rem >= 1 ? kcur + 1 : kcur, buf ^ 1);
             mfma_chunk(0);
+#pragma unroll
+            for (int g = 0; g < LPC_F; ++g) {
+                __builtin_amdgcn_sched_group_barrier(0x008, MFMA_PER_LOAD, 0);
+                __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);
+            }
             __builtin_amdgcn_sched_barrier(0);
             if (rem >= 1) {
                 __builtin_amdgcn_s_waitcnt(0);
@@ -1401,14 +1426,16 @@ static bool conv_small_tile(long columns, int n, int kch, int size)
     return n <= 64 || size == 1;
 }
 
-/* 128x64 tiles (five workgroups per CU) for every other 3x3 layer, and for any layer whose 128x128
- * tiles would number fewer than the CUs.  Measured at batch 64 against the 128x128 tile (four per CU):
- * 742 against 762 microseconds for 256->512 at 26x26, 748 against 774 for 128->256 at 52x52, 777
- * against 803 for 64->128 at 104x104, 749 against 784 for 512->1024 at 13x13. */
+/* 128x64 tiles (five workgroups per CU against four of 128x128) for 3x3 layers of 128 to 256 input
+ * channels, and for any layer whose 128x128 tiles would number fewer than the CUs.  Measured at batch
+ * 64, narrow against wide, microseconds: 706 / 718 for 256->512 at 26x26, 713 / 719 for 128->256 at
+ * 52x52, 747 / 759 for 128->256 stride 2 at 104x104; but 753 / 737 for 64->128 at 104x104 (twice the
+ * prologues and epilogues per MFMA weigh more on a short K) and 740 / 728 for 512->1024 at 13x13
+ * (every tile streams 18 MB of weights, the narrow one twice as often per output). */
 static bool conv_narrow_tile(long columns, int n, int kch, int size)
 {
     if (g_tune_bn) return g_tune_bn == 64;
-    if (size == 3) return true;
+    if (size == 3 && kch >= 72 && kch <= 144) return true;
     const long tiles = ((columns + 127) / 128) * ((n + 127) / 128);
     return tiles < 256;
 }
