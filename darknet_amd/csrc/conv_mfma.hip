@@ -934,10 +934,10 @@ __global__ __launch_bounds__(DN_THREADS, ((BM == 128 && BF16 != 3) ? 3 : 2)) voi
                 __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);
             }
             __builtin_amdgcn_sched_barrier(0);
-            if (rem >= 1) {
-                __builtin_amdgcn_s_waitcnt(0);
-                __syncthreads();
-            }
+            /* also after the last chunk: its repeated request must have landed before the workgroup
+             * reuses its LDS in the epilogue or, as a K-slice, ends and gives it back */
+            __builtin_amdgcn_s_waitcnt(0);
+            if (rem >= 1) __syncthreads();
         };
         for (int kc = kc_begin; kc < kc_end; kc += 2) {
             fstep(kc, 0);
