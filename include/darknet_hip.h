@@ -201,8 +201,11 @@ void conv_pack_weights_gpu(const float *weights, float *packed, int n, int c, in
 /* Name of the kernel forward_convolutional_gpu launches for this geometry, as it appears in a
  * profiler trace (e.g. "conv_mfma_kernel<128,128,64,64,3>"); for reports only. */
 const char *conv_kernel_name(int n, int c, int groups, int size);
-/* The same for a layer of `columns` = batch*out_h*out_w output columns: small layers (batch 1) of
- * more than 64 filters run a narrower tile, which the name shows. */
+/* The same for a layer of `columns` = batch*out_h*out_w output columns: the tile depends on the
+ * number of columns (1x1 layers and layers of up to 64 filters run 64x64 tiles, 3x3 layers of 128 to
+ * 256 channels and layers whose wide tiles would not fill the chip 128x64 tiles), and a launch that
+ * does not fill the chip runs the variant whose K-order number carries +100 (e.g.
+ * "conv_mfma_kernel<128,64,64,32,113>"). */
 const char *conv_kernel_name_columns(int n, int c, int groups, int size, long columns);
 
 /* Kernel timing for reports: the next forward_convolutional[_shortcut]_gpu call that runs on the
