@@ -181,6 +181,26 @@ def test_every_tile_shape_split_and_band_count_computes_the_same_layer(dn, orc, 
     assert len(names) >= 2      # the hooks did switch kernels
 
 
+def test_small_and_chip_filling_launches_run_their_own_variant_and_agree(dn, orc):
+    """A 3x3 layer of 128..256 channels runs the 128x64 tile; a launch with fewer tiles than the chip
+    has CUs takes the variant whose K-order number carries +100 (another form of the same loop).  The
+    same image through both against the checker and against each other."""
+    c, h, w, n = 128, 26, 26, 256
+    x = synth.uniform(51, 32 * c * h * w).reshape(32, c, h, w)
+    wt = synth.conv_weights(52, n, c, 3)
+    bias, sc, mu, var = synth.bn_random(53, n)
+    kw = dict(n=n, size=3, stride=1, pad=1, groups=1)
+    small_name = dn.conv_kernel_name_columns(n, c, 1, 3, 1 * h * w).decode()
+    big_name = dn.conv_kernel_name_columns(n, c, 1, 3, 32 * h * w).decode()
+    assert small_name == "conv_mfma_kernel<128,64,64,32,113>" and big_name == "conv_mfma_kernel<128,64,64,32,13>"
+    big = run_conv(dn, x, wt, bias, sc, mu, var, bn=1, act="leaky", **kw)
+    for k in (0, 31):
+        small = run_conv(dn, x[k:k + 1], wt, bias, sc, mu, var, bn=1, act="leaky", **kw)
+        want = orc.conv(x[k:k + 1], wt, bias, sc, mu, var, batch_normalize=1, activation="leaky", **kw)
+        assert norm_err(small, want) <= REL_TOL and norm_err(big[k:k + 1], want) <= REL_TOL, k
+        assert norm_err(small, big[k:k + 1]) <= 2e-5, k
+
+
 def test_mfma_kernel_agrees_with_direct_kernel_and_unpacked_call(dn):
     b, c, h, w, n = 2, 64, 20, 20, 96
     x = synth.uniform(1, b * c * h * w).reshape(b, c, h, w)
