@@ -3,8 +3,8 @@ compiled or run): every function this library declares under a name the referenc
 has the reference's return type and argument types; the ACTIVATION / LAYER_TYPE enums have the
 reference's members in the reference's order; every member of this library's `layer` / `network`
 exists in the reference's structs with the same type (apart from the documented additions); and
-the adapter stubs in INTEGRATION.md only touch struct members and device-layer functions that
-exist.  Skipped where the reference tree is not mounted."""
+the adapter stubs of the integration guide only touch struct members and device-layer functions
+that exist.  Skipped where the reference tree is not mounted."""
 import glob
 import os
 import re
@@ -15,12 +15,13 @@ from util import have_reference_tree
 
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 REF = "/root/reference"
+GUIDE = "INTEGRATION.md"   # the guide for binders at the repository root
 pytestmark = pytest.mark.skipif(not have_reference_tree(), reason="needs the reference's headers")
 
 # typedefs of the reference that stand for `layer` (include/darknet.h and src/*_layer.h)
 LAYER_ALIASES = {"convolutional_layer", "maxpool_layer", "route_layer", "avgpool_layer", "softmax_layer",
                  "dropout_layer", "crop_layer", "cost_layer", "local_layer", "detection_layer", "connected_layer"}
-# members this library adds to the reference's structs (INTEGRATION.md tells a binder to add them)
+# members this library adds to the reference's structs (the integration guide tells a binder to add them)
 LAYER_ADDITIONS = {"weights_packed_gpu", "xnor_wbits_gpu", "xnor_xbits_gpu", "xnor_wmean_gpu"}
 NETWORK_ADDITIONS = {"det_rows_gpu", "det_count_gpu", "det_max_rows", "max_batch"}
 # same name, deliberately another signature
@@ -180,7 +181,7 @@ def test_struct_members_exist_in_the_reference_with_the_same_type(ref_headers, o
 
 
 def test_integration_adapters_use_members_and_functions_that_exist(ref_headers, own_headers):
-    doc = open(os.path.join(ROOT, "INTEGRATION.md")).read()
+    doc = open(os.path.join(ROOT, GUIDE)).read()
     code = "\n".join(re.findall(r"```c\n(.*?)```", doc, flags=re.S))
     assert "forward_convolutional_layer_gpu" in code and "forward_maxpool_layer_gpu" in code
     ref = ref_headers[REF + "/include/darknet.h"]
@@ -199,7 +200,7 @@ def test_integration_adapters_use_members_and_functions_that_exist(ref_headers, 
     defined_in_doc = set(re.findall(r"^void\s+(\w+)\s*\(", code_nc, flags=re.M))
     checked = 0
     for name in set(called) - defined_in_doc:
-        assert name in own, name + " is called by an INTEGRATION.md stub but not declared in darknet_hip.h"
+        assert name in own, name + " is called by a stub of the integration guide but not declared in darknet_hip.h"
         checked += 1
     assert checked >= 15
     # argument counts of the calls written out in full
@@ -212,4 +213,4 @@ def test_integration_adapters_use_members_and_functions_that_exist(ref_headers, 
             depth += ch in "(["
             depth -= ch in ")]"
             count += ch == "," and depth == 0
-        assert count == len(own[name][1]), f"{name}: {count} arguments in INTEGRATION.md, {len(own[name][1])} declared"
+        assert count == len(own[name][1]), f"{name}: {count} arguments in the integration guide, {len(own[name][1])} declared"
