@@ -146,6 +146,8 @@ TILE_CASES = [  # b, c, h, w, n, size, stride: enough columns for whole rounds o
     (24, 96, 40, 40, 64, 1, 1),      # up to 64 filters, 1x1
     (16, 80, 52, 52, 192, 1, 1),     # 1x1, more than 64 filters
     (12, 20, 36, 36, 48, 3, 2),      # reference K order (c % 16 != 0), stride 2
+    (12, 20, 40, 40, 160, 3, 1),     # reference K order on the 128-row tiles
+    (8, 24, 48, 48, 136, 1, 1),      # 1x1 in reference K order, ragged filter tiles
 ]
 
 
