@@ -330,8 +330,8 @@ def measure(L, api, synth, workload, batch, precision, steps, warmup, per_layer=
         if Ly["type"] == "convolutional":
             fl = 2.0 * Ly["n"] * Ly["size"] ** 2 * (Ly["c"] // Ly["groups"]) * Ly["out_h"] * Ly["out_w"] * Ly["batch"]
             name = ("xnor_conv_kernel" if Ly["xnor"] else
-                    L.conv_kernel_name_columns(Ly["n"], Ly["c"], Ly["groups"], Ly["size"],
-                                               Ly["batch"] * Ly["out_h"] * Ly["out_w"]).decode())
+                    L.conv_kernel_name_geometry(Ly["batch"], Ly["c"], Ly["h"], Ly["w"], Ly["n"], Ly["groups"],
+                                                Ly["size"], Ly["stride"], Ly["pad"]).decode())
             # what bounds the layer: the matrix cores, or HBM at its arithmetic intensity
             ceiling = min(peak, fl / row["bytes"] * PEAK_HBM_GBS / 1e3)
             tfl = fl / ms / 1e9 if ms > 0 else 0.0

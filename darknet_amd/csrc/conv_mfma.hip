@@ -1440,18 +1440,42 @@ static bool conv_narrow_tile(long columns, int n, int kch, int size)
     return tiles < 256;
 }
 
+static const char *kernel_name(int n, int c, int groups, int size, long columns, int patch, int mode);
+
+/* Without the layer's geometry the first-layer kernel cannot be told from the generic one: the name
+ * assumes stride 1, pad size/2 and never names conv_patch_kernel (conv_kernel_name_geometry does). */
 extern "C" const char *conv_kernel_name_columns(int n, int c, int groups, int size, long columns)
 {
-    static char name[96];
     int mode = conv_mode(c, groups, size, 1, size / 2, 0);
+    if (conv_grouped_tile(n, c, groups, size) && g_algo != 1) mode = 10 + size;
+    return kernel_name(n, c, groups, size, columns, 0, mode);
+}
+
+/* The name for a whole layer, decided by the predicates the dispatch itself uses (conv_forward). */
+extern "C" const char *conv_kernel_name_geometry(int batch, int c, int h, int w, int n, int groups, int size,
+                                                 int stride, int pad)
+{
+    const int out_h = (h + 2 * pad - size) / stride + 1, out_w = (w + 2 * pad - size) / stride + 1;
+    /* a batch beyond the 32-bit offsets runs in slices of whole images */
+    const long in_img = (long)c * h * w * 4;
+    const long by_bytes = ((1L << 32) - (2L << 20)) / in_img, by_cols = ((1L << 31) - 1024) / ((long)out_h * out_w);
+    const long per = by_bytes < by_cols ? by_bytes : by_cols;
+    if (g_algo != 1 && per >= 1 && per < batch) batch = (int)per;
+    const long columns = (long)batch * out_h * out_w;
+    int mode = conv_mode(c, groups, size, stride, pad, (long)batch * in_img);
+    if (g_algo != 1 && !(size == 3 && pad != 1) && conv_grouped_tile(n, c, groups, size)) mode = 10 + size;
+    if (columns >= (1L << 31) - 512) mode = -1;
+    const int patch = g_algo == 0 && mode == 3 && conv_patch_floats(c, h, w, n, groups, size, stride, pad) > 0;
+    return kernel_name(n, c, groups, size, columns, patch, mode);
+}
+
+static const char *kernel_name(int n, int c, int groups, int size, long columns, int patch, int mode)
+{
+    static char name[96];
     int bm = n <= 32 ? 32 : n <= 64 ? 64 : 128;
-    if (conv_grouped_tile(n, c, groups, size) && g_algo != 1) {
-        mode = size == 3 ? 13 : 11;
-        bm = 32;
-    }
+    if (mode >= 10 && groups > 1) bm = 32;
     if (mode < 0) return "conv_direct_kernel";
-    if (g_algo == 0 && mode == 3 && c == 3 && n <= 64 && columns > 0 && columns % 256 == 0)
-        return n <= 32 ? "conv_patch_kernel<1,3>" : "conv_patch_kernel<2,3>"; /* for the stride-1 pad-1 layers it serves */
+    if (patch) return n <= 32 ? "conv_patch_kernel<1,3>" : "conv_patch_kernel<2,3>";
     const int bf16 = g_precision == 1 && mode >= 10;
     const int x3 = g_precision == 2 && mode >= 10;
     if (bf16 && bm == 128 && n > 128) bm = 256;

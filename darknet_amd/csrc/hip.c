@@ -127,9 +127,79 @@ int *hip_make_int_array(int *x, size_t n)
     return x_gpu;
 }
 
+/* Packed-weights cache for binders whose `layer` has no member for the packed copy (a darknet tree
+ * that keeps the reference's struct): keyed by the device address of the weights and the layer's
+ * geometry.  An entry is dropped when its weights are freed through hip_free or written through
+ * hip_push_array, so a cached copy is never older than the weights it was made from as long as
+ * the weights change through this shim (inference does not change them any other way).  Like the
+ * reference's per-device handles (src/cuda.c:67-68,80-81) the table is not synchronised: one host
+ * thread at a time. */
+typedef struct {
+    const float *weights;
+    float *packed;
+    size_t nweights;
+    int n, c, groups, size;
+} packed_entry;
+static packed_entry *g_packed = 0;
+static int g_npacked = 0, g_cap_packed = 0;
+
+static void packed_drop_range(const float *lo, size_t n)
+{
+    int i = 0;
+    while (i < g_npacked) {
+        const float *w = g_packed[i].weights;
+        if (w + g_packed[i].nweights > lo && w < lo + (n ? n : 1)) {
+            hip_check_error(hipFree(g_packed[i].packed));
+            g_packed[i] = g_packed[--g_npacked];
+        } else {
+            ++i;
+        }
+    }
+}
+
+void conv_packed_forget(const float *weights)
+{
+    if (g_npacked) packed_drop_range(weights, 1);
+}
+
+int conv_packed_cached_count(void) { return g_npacked; }
+
+const float *conv_packed_cached_gpu(const float *weights, int n, int c, int groups, int size)
+{
+    const size_t floats = conv_packed_floats(n, c, groups, size);
+    packed_entry e;
+    int i;
+    if (!floats) return 0;
+    hip_require_device("conv_packed_cached_gpu");
+    for (i = 0; i < g_npacked; ++i) {
+        const packed_entry *p = &g_packed[i];
+        if (p->weights == weights) {
+            if (p->n == n && p->c == c && p->groups == groups && p->size == size) return p->packed;
+            break; /* same address, another layer: the old copy belongs to freed weights */
+        }
+    }
+    conv_packed_forget(weights);
+    e.weights = weights;
+    e.nweights = (size_t)n * (size_t)(c / groups) * (size_t)size * (size_t)size;
+    e.n = n;
+    e.c = c;
+    e.groups = groups;
+    e.size = size;
+    e.packed = hip_make_array(0, floats);
+    conv_pack_weights_gpu(weights, e.packed, n, c, groups, size);
+    if (g_npacked == g_cap_packed) {
+        g_cap_packed = g_cap_packed ? 2 * g_cap_packed : 64;
+        g_packed = realloc(g_packed, sizeof(*g_packed) * (size_t)g_cap_packed);
+        if (!g_packed) dn_fatal("Malloc error");
+    }
+    g_packed[g_npacked++] = e;
+    return e.packed;
+}
+
 void hip_free(float *x_gpu)
 {
     if (g_parse_only) return;
+    if (g_npacked && x_gpu) packed_drop_range(x_gpu, 1);
     hip_check_error(hipFree(x_gpu));
 }
 
@@ -251,6 +321,7 @@ static void staged_copy(char *dev, char *host, size_t bytes, int to_device)
 void hip_push_array(float *x_gpu, float *x, size_t n)
 {
     if (g_parse_only) return; /* the host copy is the only copy */
+    if (g_npacked) packed_drop_range(x_gpu, n);
     if (sizeof(float) * n >= DN_STAGE_MIN && !host_is_pinned(x, sizeof(float) * n)) {
         staged_copy((char *)x_gpu, (char *)x, sizeof(float) * n, 1);
         return;

@@ -56,7 +56,7 @@ def time_layer(batch, c, h, w, n, size, stride, pad=None, groups=1, bn=1, act=7,
     flops = 2.0 * n * size * size * (c // groups) * oh * ow * batch
     byts = 4.0 * (batch * c * h * w + batch * n * oh * ow + n * (c // groups) * size * size)
     return {"batch": batch, "shape": f"{size}x{size}/{stride} {c}->{n} @{w}x{h} g{groups}",
-            "kernel": L.conv_kernel_name_columns(n, c, groups, size, batch * oh * ow).decode(), "ms": round(ms, 4),
+            "kernel": L.conv_kernel_name_geometry(batch, c, h, w, n, groups, size, stride, pad).decode(), "ms": round(ms, 4),
             "tflops": round(flops / ms / 1e9, 2), "frac_of_fp32_mfma_peak": round(flops / ms / 1e9 / PEAK, 4),
             "algorithmic_gbs": round(byts / ms / 1e6, 1)}
 

@@ -52,6 +52,8 @@ SIGNATURES = {
     "forward_convolutional_noalloc_gpu": (i, [V] * 8 + [i] * 11),
     "forward_convolutional_yolo_gpu": (None, [V] * 8 + [i] * 11 + [V, i, i]),
     "conv_packed_floats": (z, [i, i, i, i]), "conv_pack_weights_gpu": (None, [V, V, i, i, i, i]),
+    "conv_packed_cached_gpu": (V, [V, i, i, i, i]), "conv_packed_forget": (None, [V]),
+    "conv_packed_cached_count": (i, []),
     "conv_set_algo": (None, [i]), "conv_set_ksplit": (None, [i, i]), "conv_set_bands": (None, [i]),
     "xnor_weight_words": (z, [i, i, i]), "xnor_input_words": (z, [i, i, i, i]),
     "xnor_pack_weights_gpu": (None, [V, V, V, i, i, i]),
@@ -99,7 +101,8 @@ SIGNATURES = {
     "conv_set_precision": (None, [i]), "conv_get_precision": (i, []),
     "conv_profile_next": (None, [V, V]), "conv_profile_pending": (i, []),
     "conv_kernel_name": (C.c_char_p, [i, i, i, i]),
-    "conv_kernel_name_columns": (C.c_char_p, [i, i, i, i, C.c_long]), "layer_output_host": (F, [V, i]),
+    "conv_kernel_name_columns": (C.c_char_p, [i, i, i, i, C.c_long]),
+    "conv_kernel_name_geometry": (C.c_char_p, [i] * 9), "layer_output_host": (F, [V, i]),
     "layer_indexes_host": (I, [V, i]), "network_set_verbose": (None, [i]),
     "network_set_conv": (None, [V, i, F, F, F, F, F]),
     "network_layer_info": (None, [V, i, I, F]), "network_route_inputs": (i, [V, i, I, I, i]),

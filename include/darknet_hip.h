@@ -96,7 +96,9 @@ void   hip_event_destroy(void *ev);
 void fill_gpu(int N, float ALPHA, float *X, int INCX);                       /* blas.h:100 */
 void copy_gpu(int N, float *X, int INCX, float *Y, int INCY);                /* blas.h:53  */
 void copy_gpu_offset(int N, float *X, int OFFX, int INCX, float *Y, int OFFY, int INCY); /* :54 */
+#ifndef DARKNET_API  /* inside a darknet tree src/activations.h:15 declares it with the ACTIVATION enum */
 void activate_array_gpu(float *x, int n, int activation);                    /* activations.h:15 */
+#endif
 void normalize_gpu(float *x, float *mean, float *variance, int batch, int filters, int spatial); /* blas.h:65 */
 void scale_bias_gpu(float *output, float *scales, int batch, int n, int size);  /* blas.h:76 */
 void add_bias_gpu(float *output, float *biases, int batch, int n, int size);    /* blas.h:79 */
@@ -198,6 +200,17 @@ int forward_convolutional_noalloc_gpu(const float *input, const float *weights, 
 size_t conv_packed_floats(int n, int c, int groups, int size);
 void conv_pack_weights_gpu(const float *weights, float *packed, int n, int c, int groups, int size);
 
+/* The packed copy for binders whose `layer` struct has no member to keep it in (a darknet tree that
+ * keeps the reference's include/darknet.h:115-422 as it is).  No counterpart in the reference.
+ * conv_packed_cached_gpu returns the packed copy of the weights at device address `weights`, packing
+ * them on the first call for that address and geometry; NULL when conv_packed_floats() == 0.  The
+ * library owns the copy and drops it when those weights are freed through hip_free / cuda_free or
+ * written through hip_push_array / cuda_push_array; a binder that writes the weights any other way
+ * calls conv_packed_forget(weights) afterwards.  One host thread at a time, like the rest of the shim. */
+const float *conv_packed_cached_gpu(const float *weights, int n, int c, int groups, int size);
+void conv_packed_forget(const float *weights);
+int conv_packed_cached_count(void);
+
 /* Name of the kernel forward_convolutional_gpu launches for this geometry, as it appears in a
  * profiler trace (e.g. "conv_mfma_kernel<128,128,64,64,3>"); for reports only. */
 const char *conv_kernel_name(int n, int c, int groups, int size);
@@ -207,6 +220,12 @@ const char *conv_kernel_name(int n, int c, int groups, int size);
  * does not fill the chip runs the variant whose K-order number carries +100 (e.g.
  * "conv_mfma_kernel<128,64,64,32,113>"). */
 const char *conv_kernel_name_columns(int n, int c, int groups, int size, long columns);
+/* The same for a layer whose whole geometry is known, decided by the very predicates the dispatch
+ * uses; the only form that can name the first-layer kernel ("conv_patch_kernel<1,3>": 3 channels,
+ * 3x3, stride 1, pad 1, up to 64 filters, image a multiple of 256 pixels and its width of 4) and
+ * the direct kernel of geometries the MFMA kernels do not serve. */
+const char *conv_kernel_name_geometry(int batch, int c, int h, int w, int n, int groups, int size,
+                                      int stride, int pad);
 
 /* Kernel timing for reports: the next forward_convolutional[_shortcut]_gpu call that runs on the
  * MFMA kernel attaches these two events (hip_event_create) to its main kernel's dispatch, so

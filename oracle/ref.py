@@ -29,8 +29,15 @@ _IV = ["type", "batch", "h", "w", "c", "out_h", "out_w", "out_c", "n", "size", "
 _FV = ["alpha", "beta", "scale", "temperature"]
 
 
+_HARNESS = {"fast": "librefh.so", "o2": "librefh_o2.so", "hip": "librefh_hip.so"}
+_LIBRARY = {"fast": "libdarknet_ref.so", "o2": "libdarknet_ref_o2.so", "hip": "libdarknet_ref_hip.so"}
+
+
 def _path(variant: str) -> str:
-    return os.path.join(_HERE, "_ref", "librefh.so" if variant == "fast" else "librefh_o2.so")
+    """fast / o2: the reference's CPU build.  hip: the reference's own host files built with -DGPU
+    and bound to darknet_amd/libdarknet_hip.so through integration/adapters.c - the same calls then
+    run the reference's parse_network_cfg / network_predict / forward_network_gpu on the HIP kernels."""
+    return os.path.join(_HERE, "_ref", _HARNESS[variant])
 
 
 def available(variant: str = "o2") -> bool:
@@ -39,8 +46,7 @@ def available(variant: str = "o2") -> bool:
 
 def raw(variant: str = "o2"):
     """The reference library itself (plain-pointer functions such as im2col_cpu, gemm)."""
-    name = "libdarknet_ref.so" if variant == "fast" else "libdarknet_ref_o2.so"
-    return C.CDLL(os.path.join(_HERE, "_ref", name))
+    return C.CDLL(os.path.join(_HERE, "_ref", _LIBRARY[variant]))
 
 
 def _harness(variant="o2"):
@@ -66,12 +72,17 @@ def letterbox_image(im, bw, bh, variant="o2"):
 
 
 class RefNet:
-    """A network parsed and run by the compiled reference (CPU build)."""
+    """A network parsed and run by the compiled reference (CPU build, or variant "hip")."""
 
-    def __init__(self, cfg_path: str, variant: str = "o2"):
-        raw(variant)
+    def __init__(self, cfg_path: str, variant: str = "o2", gpu: int | None = 0):
+        self.lib = raw(variant)
         self.h = C.CDLL(_path(variant))
         H = self.h
+        for f in (self.lib.load_weights, self.lib.save_weights):
+            f.restype = None
+            f.argtypes = [C.c_void_p, C.c_char_p]
+        if variant == "hip" and gpu is not None:
+            H.refh_set_gpu(gpu)
         H.refh_load.restype = C.c_void_p
         H.refh_load.argtypes = [C.c_char_p]
         H.refh_free.argtypes = [C.c_void_p]
@@ -149,6 +160,19 @@ class RefNet:
         rows = np.zeros((max(cap, 1), 5 + classes), np.float32)
         n = self.h.refh_get_boxes(self.net, w, h, thresh, relative, nms, rows.ctypes.data_as(_F), cap)
         return rows[:n].copy()
+
+    def load_weights(self, path):
+        """load_weights of the reference (src/parser.c:1308); its GPU build ends each layer's load with
+        push_convolutional_layer (:1210-1214)."""
+        self.lib.load_weights(self.net, path.encode())
+
+    def save_weights(self, path):
+        self.lib.save_weights(self.net, path.encode())
+
+    def free(self):
+        if self.net:
+            self.h.refh_free(self.net)
+            self.net = None
 
     def predict(self, x):
         x = np.ascontiguousarray(x, np.float32)

@@ -9,6 +9,19 @@
 #include "darknet.h"
 #include <string.h>
 
+/* Built a second time with -DGPU against the reference tree as bound to the HIP library
+ * (oracle/Makefile, target ref_hip): the same calls then drive the reference's own
+ * parse_network_cfg / network_predict / forward_network_gpu over the adapters, parameters are
+ * pushed to the device after they are written and layer outputs are pulled before they are read. */
+#ifdef GPU
+#include "convolutional_layer.h"
+#include "batchnorm_layer.h"
+void refh_set_gpu(int n) { cuda_set_device(n); }
+int refh_is_gpu_build(void) { return 1; }
+#else
+int refh_is_gpu_build(void) { return 0; }
+#endif
+
 enum { REFH_NI = 28, REFH_NF = 4 };
 
 network *refh_load(char *cfg)
@@ -105,6 +118,9 @@ void refh_set_conv(network *net, int i, const float *weights, const float *biase
         if (mean) memcpy(l.rolling_mean, mean, sizeof(float) * (size_t)l.n);
         if (variance) memcpy(l.rolling_variance, variance, sizeof(float) * (size_t)l.n);
     }
+#ifdef GPU
+    push_convolutional_layer(l);
+#endif
 }
 
 /* The same for a [batchnorm] layer: c values per vector, no weights (src/batchnorm_layer.c:20-33). */
@@ -116,6 +132,9 @@ void refh_set_batchnorm(network *net, int i, const float *biases, const float *s
     if (scales) memcpy(l.scales, scales, sizeof(float) * (size_t)l.c);
     if (mean) memcpy(l.rolling_mean, mean, sizeof(float) * (size_t)l.c);
     if (variance) memcpy(l.rolling_variance, variance, sizeof(float) * (size_t)l.c);
+#ifdef GPU
+    push_batchnorm_layer(l);
+#endif
 }
 
 /* The same for a connected layer (its parameter vectors are sized by outputs / inputs). */
@@ -147,8 +166,23 @@ float *refh_predict(network *net, float *input)
     return network_predict(net, input);
 }
 
-float *refh_layer_output(network *net, int i) { return net->layers[i].output; }
-int *refh_layer_indexes(network *net, int i) { return net->layers[i].indexes; }
+float *refh_layer_output(network *net, int i)
+{
+    layer l = net->layers[i];
+#ifdef GPU
+    if (l.output_gpu && l.output) cuda_pull_array(l.output_gpu, l.output, (size_t)l.outputs * l.batch);
+#endif
+    return l.output;
+}
+
+int *refh_layer_indexes(network *net, int i)
+{
+    layer l = net->layers[i];
+#ifdef GPU
+    if (l.indexes_gpu && l.indexes) hip_pull_int_array(l.indexes_gpu, l.indexes, (size_t)l.outputs * l.batch);
+#endif
+    return l.indexes;
+}
 float *refh_layer_weights(network *net, int i) { return net->layers[i].weights; }
 float *refh_layer_binary_weights(network *net, int i) { return net->layers[i].binary_weights; }
 float *refh_layer_binary_input(network *net, int i) { return net->layers[i].binary_input; }

@@ -183,7 +183,12 @@ def test_struct_members_exist_in_the_reference_with_the_same_type(ref_headers, o
 def test_integration_adapters_use_members_and_functions_that_exist(ref_headers, own_headers):
     doc = open(os.path.join(ROOT, GUIDE)).read()
     code = "\n".join(re.findall(r"```c\n(.*?)```", doc, flags=re.S))
-    assert "forward_convolutional_layer_gpu" in code and "forward_maxpool_layer_gpu" in code
+    # the adapters a tree needs are a compiled file (tests/test_integration_link.py links it into the
+    # reference tree); the guide's own blocks are the optional replacements, checked here as text
+    adapters = open(os.path.join(ROOT, "integration", "adapters.c")).read()
+    assert "forward_convolutional_layer_gpu" in adapters and "forward_maxpool_layer_gpu" in adapters
+    assert "forward_connected_layer_gpu" in code and "forward_route_layer_gpu" in code
+    code = code + "\n" + adapters
     ref = ref_headers[REF + "/include/darknet.h"]
     layer = set(struct_members(ref, "struct layer{")) | LAYER_ADDITIONS
     network = set(struct_members(ref, "typedef struct network{")) | NETWORK_ADDITIONS
