@@ -214,13 +214,15 @@ static layer parse_route(cfg_section *o, size_params p, network *net)
         layers[i] = index;
         sizes[i] = net->layers[index].outputs;
     }
-    r = make_route_layer(p.batch, n, layers, sizes);
     first = net->layers[layers[0]];
-    if (n == 1 && r.output_gpu && first.output_gpu) {
+    if (n == 1 && first.output_gpu) {
         /* one source: the reference copies it (src/route_layer.c:74-87); here the layer's output is a
-         * view of the source's buffer - the same values at no cost (free_network knows) */
-        hip_free(r.output_gpu);
-        r.output_gpu = first.output_gpu;
+         * view of the source's buffer - the same values, no launch, no second buffer */
+        r = make_route_view(p.batch, layers[0], sizes[0], first.output_gpu);
+        free(layers);
+        free(sizes);
+    } else {
+        r = make_route_layer(p.batch, n, layers, sizes);
     }
     r.out_w = first.out_w;
     r.out_h = first.out_h;

@@ -2019,5 +2019,6 @@ extern "C" int forward_convolutional_noalloc_gpu(const float *input, const float
     conv_forward(input, weights, packed, biases, scales, rolling_mean, rolling_variance, output, batch, c, h, w,
                  n, groups, size, stride, pad, batch_normalize, activation, 0, 0, 0.f, 0.f, DN_LINEAR, 0);
     g_noalloc = 0;
+    if (g_noalloc_error) g_prof_start = g_prof_stop = 0; /* a pending timing pair must not stamp a later, unrelated call */
     return g_noalloc_error ? -1 : 0;
 }

@@ -36,6 +36,8 @@ float cfg_find_float(cfg_section *s, const char *key, float def);
 float cfg_find_float_quiet(cfg_section *s, const char *key, float def);
 void cfg_report_unused(cfg_section *s);
 
+layer make_route_view(int batch, int input_layer, int input_size, float *source_output_gpu);
+
 extern int dn_verbose;
 void *dn_calloc(size_t n, size_t size);
 

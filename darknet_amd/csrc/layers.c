@@ -184,7 +184,7 @@ void forward_maxpool_layer_gpu(layer l, network net)
 }
 
 /* ---- route: src/route_layer.c:7-38 --------------------------------------------------------- */
-layer make_route_layer(int batch, int n, int *input_layers, int *input_sizes)
+static layer route_layer_without_output(int batch, int n, int *input_layers, int *input_sizes)
 {
     layer l;
     int i, outputs = 0;
@@ -203,7 +203,27 @@ layer make_route_layer(int batch, int n, int *input_layers, int *input_sizes)
     l.outputs = outputs;
     l.inputs = outputs;
     l.forward_gpu = forward_route_layer_gpu;
-    l.output_gpu = hip_make_array(0, (size_t)outputs * batch);
+    return l;
+}
+
+layer make_route_layer(int batch, int n, int *input_layers, int *input_sizes)
+{
+    layer l = route_layer_without_output(batch, n, input_layers, input_sizes);
+    l.output_gpu = hip_make_array(0, (size_t)l.outputs * batch);
+    return l;
+}
+
+/* A route of one source as a view of that source's device buffer: what the reference copies
+ * (src/route_layer.c:74-87) is already there.  The buffer stays the source's: free_layer leaves it. */
+layer make_route_view(int batch, int input_layer, int input_size, float *source_output_gpu)
+{
+    int *layers = (int *)dn_calloc(1, sizeof(int)), *sizes = (int *)dn_calloc(1, sizeof(int));
+    layer l;
+    layers[0] = input_layer;
+    sizes[0] = input_size;
+    l = route_layer_without_output(batch, 1, layers, sizes);
+    l.output_gpu = source_output_gpu;
+    l.output_gpu_is_view = 1;
     return l;
 }
 
@@ -213,7 +233,7 @@ void forward_route_layer_gpu(layer l, network net)
     int i;
     if (l.n > 8) dn_fatal("route layer: more than 8 sources");
     for (i = 0; i < l.n; ++i) srcs[i] = net.layers[l.input_layers[i]].output_gpu;
-    if (l.n == 1 && srcs[0] == l.output_gpu) return; /* a view of its one source (parse_network_cfg) */
+    if (l.output_gpu_is_view) return; /* its one source's buffer is its output (make_route_view) */
     forward_route_gpu(srcs, l.input_sizes, l.n, l.output_gpu, l.batch);
 }
 
@@ -802,7 +822,7 @@ void free_layer(layer l)
     if (l.scales_gpu) hip_free(l.scales_gpu);
     if (l.rolling_mean_gpu) hip_free(l.rolling_mean_gpu);
     if (l.rolling_variance_gpu) hip_free(l.rolling_variance_gpu);
-    if (l.output_gpu) hip_free(l.output_gpu);
+    if (l.output_gpu && !l.output_gpu_is_view) hip_free(l.output_gpu);
     if (l.binary_weights_gpu) hip_free(l.binary_weights_gpu);
     if (l.binary_input_gpu) hip_free(l.binary_input_gpu);
     if (l.weights_packed_gpu) hip_free(l.weights_packed_gpu);

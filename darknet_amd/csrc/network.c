@@ -29,9 +29,7 @@ void free_network(network *net)
     if (!net) return;
     for (i = 0; i < net->n; ++i) {
         layer l = net->layers[i];
-        /* a route of one source may be a view of that source's buffer, which its owner frees */
-        if (l.type == ROUTE && l.n == 1 && l.output_gpu == net->layers[l.input_layers[0]].output_gpu) l.output_gpu = 0;
-        free_layer(l);
+        free_layer(l); /* leaves the buffers a layer only borrows: dropout, one-source routes */
     }
     free(net->layers);
     free(net->input);

@@ -138,6 +138,7 @@ struct layer {
 
     /* additions of this library */
     float *weights_packed_gpu; /* MFMA layout of weights_gpu; refreshed by push_convolutional_layer */
+    int output_gpu_is_view;    /* output_gpu belongs to another layer (a one-source route): free_layer leaves it */
     unsigned *xnor_wbits_gpu;  /* xnor layers: packed sign(w), packed sign(x), mean|w| per filter */
     unsigned *xnor_xbits_gpu;
     float *xnor_wmean_gpu;

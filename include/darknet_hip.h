@@ -130,7 +130,14 @@ void binarize_weights_gpu(float *weights, int n, int size, float *binary); /* co
  *   packed: NULL, or the buffer written by conv_pack_weights_gpu for these weights (skips the
  *   per-call repack; must be refreshed whenever the weights change).
  * A 1x1 kernel must come with stride 1 and pad 0 (the reference feeds the image straight to
- * the GEMM in that case, src/convolutional_layer.c:468-469; every cfg in the tree obeys it). */
+ * the GEMM in that case, src/convolutional_layer.c:468-469; every cfg in the tree obeys it).
+ * Results are deterministic run to run.  The order in which K is summed depends on how the launch
+ * fills the chip, hence on the batch size: tiles of the last, partial round are cut along K and the
+ * slices summed in slice order.  The same image therefore gives the same values at every batch size
+ * only to rounding (measured <= 1e-5 of the layer's largest value, tests hold 2e-5), where the
+ * reference's per-image GEMM gives the same bits.  conv_set_algo(3), or conv_set_ksplit(1, 0),
+ * switches the cut off: then every output sums K in one fixed order and the bits no longer depend
+ * on the batch size (tested). */
 void forward_convolutional_gpu(const float *input, const float *weights, const float *packed,
                                const float *biases, const float *scales,
                                const float *rolling_mean, const float *rolling_variance,
@@ -181,7 +188,9 @@ void forward_convolutional_yolo_gpu(const float *input, const float *weights, co
  *   - a geometry whose K-split needs more than 64 MiB is refused (none of the benchmark
  *     networks comes near: their largest need is 48 MB).
  * Returns 0, or -1 after a message on stderr when the call was refused; a refused call launches
- * nothing.  The address of the array is looked up once per device (hip_set_device does it;
+ * nothing (one exception: a batch beyond the kernels' 32-bit offsets, 4 GiB of input, runs in
+ * slices of whole images, and a slice can be refused after earlier ones ran) and drops a pending
+ * conv_profile_next pair.  The address of the array is looked up once per device (hip_set_device does it;
  * otherwise the first call on that device, which should then precede any stream capture).
  * Every call on a device shares that device's array: calls that overlap on one device - two
  * streams, two host threads - race.  Calls on one stream are ordered and safe. */

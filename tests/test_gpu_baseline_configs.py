@@ -88,6 +88,15 @@ def test_yolov3_608_batch_8(dn):
     batch_equals_batch_1(lambda b: cfgs.yolov3(b, 608), 8, [2, 7])
 
 
+def test_yolov3_416_batch_64(dn):
+    """The headline configuration: three images of the batch, per layer at the same-image tolerance,
+    on the first layers, two layers of every scale (a 1x1 and a 3x3, with their fused shortcuts),
+    the neck and the three heads."""
+    batch_equals_batch_1(lambda b: cfgs.yolov3(b, 416), 64, [0, 40, 63],
+                         layers=[0, 1, 2, 3, 4, 5, 11, 12, 13, 14, 15, 36, 37, 38, 39, 40, 61, 62, 63, 64, 65, 74,
+                                 79, 80, 81, 82, 84, 85, 86, 87, 93, 94, 96, 97, 98, 99, 105, 106])
+
+
 def test_yolov3_608_batch_64(dn):
     """The largest configuration (30 GB of layer outputs): the three yolo heads, the first
     layers and one layer of every scale, for two images."""

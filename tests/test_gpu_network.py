@@ -182,6 +182,99 @@ def test_set_batch_network_shrinks_and_grows_back(dn):
     net.free()
 
 
+ROUTE_VIEWS = """[net]
+batch=2
+subdivisions=1
+width=12
+height=10
+channels=4
+
+[convolutional]
+filters=8
+size=3
+stride=1
+pad=1
+activation=leaky
+
+[route]
+layers=-1
+
+[route]
+layers=-1
+
+[dropout]
+probability=.5
+
+[convolutional]
+filters=6
+size=1
+stride=1
+pad=1
+activation=linear
+
+[route]
+layers=3
+
+[route]
+layers=-1,1
+
+[route]
+layers=4
+"""
+
+
+def test_views_of_views_and_of_dropout_layers(dn):
+    """A route of a route, a dropout behind a view, a route whose source is a dropout layer, a
+    two-source route that concatenates two views, and a view as the network's last layer: every
+    layer equals the checker's, and building and freeing the network three times returns the memory."""
+    import ctypes as C
+    hip = C.CDLL("libamdhip64.so")
+
+    def free_bytes():
+        free, total = C.c_size_t(), C.c_size_t()
+        assert hip.hipMemGetInfo(C.byref(free), C.byref(total)) == 0
+        return free.value
+
+    assert check_network(ROUTE_VIEWS) <= REL_TOL
+    before = free_bytes()
+    for _ in range(3):
+        check_network(ROUTE_VIEWS)
+    assert free_bytes() == before
+    net = api.Network(cfg_text=ROUTE_VIEWS)
+    kinds = [L["type"] for L in net.layers]
+    assert kinds == ["convolutional", "route", "route", "dropout", "convolutional", "route", "route", "route"]
+    net.free()
+
+
+@pytest.mark.parametrize("pin", ["algo3", "ksplit1"])
+def test_same_image_same_bits_at_any_batch_without_the_k_split(dn, pin):
+    """With the cut along K switched off every output sums K in one fixed order, whatever tile it
+    falls into: an image then gives the same bits at batch 1 and inside a batch of five, as the
+    reference's per-image GEMM does at any batch size."""
+    if pin == "algo3":
+        dn.conv_set_algo(3)
+    else:
+        dn.conv_set_ksplit(1, 0)
+        dn.conv_set_bands(1)
+    try:
+        net5 = api.Network(cfg_text=cfgs.yolov3(5, 160))
+        net1 = api.Network(cfg_text=cfgs.yolov3(1, 160))
+        fill_params(net5.set_conv, net5.layers)
+        fill_params(net1.set_conv, net1.layers)
+        x = synth.uniform01(9, net5.inputs * 5).reshape(5, -1)
+        net5.predict(x)
+        for k in (0, 3):
+            net1.predict(x[k])
+            for i in range(net5.n):
+                assert np.array_equal(net5.layer_output(i)[k], net1.layer_output(i)[0]), (pin, k, i)
+        net5.free()
+        net1.free()
+    finally:
+        dn.conv_set_algo(0)
+        dn.conv_set_ksplit(0, 0)
+        dn.conv_set_bands(0)
+
+
 def test_one_source_route_is_a_view_of_its_source(dn):
     """`[route] layers=-4` copies one layer in the reference (src/route_layer.c:74-87); here the
     route's output is the source's buffer: the same bits, no launch, and the two-source routes of the

@@ -99,3 +99,35 @@ def test_noalloc_refuses_what_would_allocate(dn, capfd):
     assert dn.forward_convolutional_noalloc_gpu(*cs.args(cs.out_b)) == 0
     dn.forward_convolutional_gpu(*cs.args(cs.out_a))
     assert np.array_equal(cs.out_b.numpy(cs.shape()).view(np.uint32), cs.out_a.numpy(cs.shape()).view(np.uint32))
+
+
+def test_noalloc_refusals_decided_on_the_host(dn, capfd):
+    """A K-split that needs more than the fixed array, and the bf16 staging mode on a 3x3 layer: both
+    are refused before anything is launched, and a timing pair armed for the refused call does not
+    stay armed for the next one."""
+    cs = Case(dn, 51, 1, 128, 52, 52, 256, 3, 1, 1)       # 86 tiles of 128x64 at batch 1: all of them tail
+    sentinel = np.full(cs.out_b.n, 5.0, np.float32)
+    cs.out_b = D(sentinel)
+    e0, e1 = dn.hip_event_create(), dn.hip_event_create()
+    dn.conv_set_ksplit(32, 64)                            # 86 tiles x 32 slices x 128x64 floats = 90 MB > 64 MiB
+    try:
+        dn.conv_profile_next(e0, e1)
+        assert dn.forward_convolutional_noalloc_gpu(*cs.args(cs.out_b)) == -1
+    finally:
+        dn.conv_set_ksplit(0, 0)
+    assert "scratch" in capfd.readouterr().err
+    assert dn.conv_profile_pending() == 0
+    dn.conv_set_precision(1)
+    try:
+        assert dn.forward_convolutional_noalloc_gpu(*cs.args(cs.out_b)) == -1
+    finally:
+        dn.conv_set_precision(0)
+    assert "bf16" in capfd.readouterr().err
+    dn.hip_synchronize()
+    assert np.array_equal(cs.out_b.numpy((cs.out_b.n,)), sentinel)
+    dn.hip_event_destroy(e0)
+    dn.hip_event_destroy(e1)
+    # the same layer under the library's own choice of split fits and agrees with the allocating entry
+    assert dn.forward_convolutional_noalloc_gpu(*cs.args(cs.out_b)) == 0
+    dn.forward_convolutional_gpu(*cs.args(cs.out_a))
+    assert np.array_equal(cs.out_b.numpy(cs.shape()).view(np.uint32), cs.out_a.numpy(cs.shape()).view(np.uint32))
