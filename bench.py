@@ -409,6 +409,19 @@ def measure(L, api, synth, workload, batch, precision, steps, warmup, per_layer=
     pcie_pinned_ms = (time.perf_counter() - t0) * 1e3 / 2
     api.free_pinned_array(xp)
     del xp
+    # the same work with the copies overlapped: network_predict_submit / _collect keep two batches in
+    # flight, so the upload of batch n+1 and the download of batch n-1 run while batch n computes
+    # (pageable input, as network_predict takes it; the outputs are the same bits)
+    reps = 6 if batch > 1 else 40
+    net.submit(x)
+    net.collect(copy=False)
+    t0 = time.perf_counter()
+    net.submit(x)
+    for _ in range(reps - 1):
+        net.submit(x)
+        net.collect(copy=False)
+    net.collect(copy=False)
+    pcie_pipelined_ms = (time.perf_counter() - t0) * 1e3 / reps
 
     # ---- per-layer accounting, grouped by kernel
     kernels = {}
@@ -533,8 +546,12 @@ def measure(L, api, synth, workload, batch, precision, steps, warmup, per_layer=
             "gflop_per_image": round(flops_img / 1e9, 3), "device": dev,
             "wall_ms_per_step": round(wall_ms / steps, 4),
             "ms_per_step_with_layer_events": round(ms_per_step_events, 4),
-            "pcie_inclusive_ms_per_step": round(pcie_ms, 3),
-            "pcie_inclusive_images_per_s": round(batch / (pcie_ms / 1e3), 2),
+            "pcie_inclusive_ms_per_step": round(pcie_pipelined_ms, 3),
+            "pcie_inclusive_images_per_s": round(batch / (pcie_pipelined_ms / 1e3), 2),
+            "pcie_inclusive_note": "network_predict_submit/_collect, two batches in flight, pageable input; "
+                                   "the synchronous network_predict is the _sync_ figure",
+            "pcie_inclusive_sync_ms_per_step": round(pcie_ms, 3),
+            "pcie_inclusive_sync_images_per_s": round(batch / (pcie_ms / 1e3), 2),
             "pcie_inclusive_pinned_input_ms_per_step": round(pcie_pinned_ms, 3),
             "memory_bound_layers": mem, "roofline": roofline}
 
@@ -635,6 +652,8 @@ def main():
                           f"weights uniform(-1,1)*sqrt(2/(k*k*c)), BN mean 0 var 1 scale 1"}
     config.update({k: m[k] for k in ("gflop_per_image", "device", "wall_ms_per_step", "ms_per_step_with_layer_events",
                                      "pcie_inclusive_ms_per_step", "pcie_inclusive_images_per_s",
+                                     "pcie_inclusive_note", "pcie_inclusive_sync_ms_per_step",
+                                     "pcie_inclusive_sync_images_per_s",
                                      "pcie_inclusive_pinned_input_ms_per_step", "memory_bound_layers")})
     out = {
         "metric": "images/sec", "value": m["value"], "unit": "images/s", "n_gpus": 1,

@@ -240,6 +240,28 @@ class Network:
         last = [L for L in self.layers if L["type"] != "cost"][-1]   # get_network_output_layer
         return np.ctypeslib.as_array(out, shape=(self.batch, last["outputs"])).copy()
 
+    def submit(self, x):
+        """network_predict_submit: queue upload, forward and download of one batch (two may be in
+        flight).  A pinned array (pinned_array) is used where it is and must stay untouched until
+        the batch is collected; anything else is copied before the call returns."""
+        x = x if isinstance(x, np.ndarray) and x.dtype == np.float32 and x.flags.c_contiguous else \
+            np.ascontiguousarray(x, np.float32)
+        assert x.size == self.inputs * self.batch, (x.size, self.inputs, self.batch)
+        self.L.network_predict_submit(self.net, _fp(x))
+
+    def collect(self, copy=True):
+        """network_predict_collect: the output layer of the oldest batch in flight, [batch, outputs]."""
+        out = self.L.network_predict_collect(self.net)
+        last = [L for L in self.layers if L["type"] != "cost"][-1]
+        a = np.ctypeslib.as_array(out, shape=(self.batch, last["outputs"]))
+        return a.copy() if copy else a
+
+    def collected_output(self, i, copy=True):
+        """Host copy of layer i (a yolo head or the output layer) of the batch collected last."""
+        p = self.L.network_collected_output(self.net, i)
+        a = np.ctypeslib.as_array(p, shape=(self.batch, self.layers[i]["outputs"]))
+        return a.copy() if copy else a
+
     def push_input(self, x):
         """Place a batch in the network's device input buffer (for forward_device)."""
         x = np.ascontiguousarray(x, np.float32)

@@ -19,7 +19,7 @@ LIB = os.path.join(HERE, "libdarknet_hip.so")
 ROCM = os.environ.get("ROCM_PATH", "/opt/rocm")
 
 HIP_SOURCES = ["pointwise.hip", "pool.hip", "conv_direct.hip", "conv_mfma.hip", "xnor.hip", "detect.hip", "image.hip", "local.hip"]
-C_SOURCES = ["hip.c", "cfg_reader.c", "cfg_parser.c", "layers.c", "network.c", "weights_io.c", "boxes.c", "images.c"]
+C_SOURCES = ["hip.c", "cfg_reader.c", "cfg_parser.c", "layers.c", "network.c", "weights_io.c", "boxes.c", "images.c", "pipeline.c"]
 
 # -packed-fp32-ops: keep the compiler from forming packed fp32 instructions.
 HIP_FLAGS = ["--offload-arch=gfx950", "-O3", "-fPIC", "-ffp-contract=off", "-Wno-comment",

@@ -245,7 +245,7 @@ void hip_host_free(float *x)
     free(x);
 }
 
-static int host_is_pinned(const void *x, size_t bytes)
+int dn_host_is_pinned(const void *x, size_t bytes)
 {
     int i;
     for (i = 0; i < g_npinned; ++i)
@@ -266,7 +266,7 @@ static hipStream_t g_copy_stream;
 
 /* memcpy between pageable and pinned memory, split over the host cores: one core moves ~8 GB/s,
  * less than the link, so a single-threaded copy would be the bottleneck of every large transfer */
-static void host_copy(char *dst, const char *src, size_t bytes)
+void dn_host_copy(char *dst, const char *src, size_t bytes)
 {
     const size_t piece = (size_t)1 << 20;
     const long pieces = (long)((bytes + piece - 1) / piece);
@@ -296,7 +296,7 @@ static void staged_copy(char *dev, char *host, size_t bytes, int to_device)
         k = i & 1;
         if (to_device) {
             if (i >= 2) hip_check_error(hipEventSynchronize(g_stage_ev[k])); /* buffer k is free again */
-            host_copy((char *)g_stage[k], host + off, len);
+            dn_host_copy((char *)g_stage[k], host + off, len);
             hip_check_error(hipMemcpyAsync(dev + off, g_stage[k], len, hipMemcpyHostToDevice, g_copy_stream));
             hip_check_error(hipEventRecord(g_stage_ev[k], g_copy_stream));
         } else {
@@ -305,7 +305,7 @@ static void staged_copy(char *dev, char *host, size_t bytes, int to_device)
             hip_check_error(hipEventRecord(g_stage_ev[k], g_copy_stream));
             if (i >= 1) { /* while chunk i is in flight, hand chunk i-1 to the caller */
                 hip_check_error(hipEventSynchronize(g_stage_ev[k ^ 1]));
-                host_copy(host + prev_off, (const char *)g_stage[k ^ 1], prev_len);
+                dn_host_copy(host + prev_off, (const char *)g_stage[k ^ 1], prev_len);
             }
             prev_off = off;
             prev_len = len;
@@ -313,7 +313,7 @@ static void staged_copy(char *dev, char *host, size_t bytes, int to_device)
         off += len;
     }
     hip_check_error(hipStreamSynchronize(g_copy_stream));
-    if (!to_device && i >= 1) host_copy(host + prev_off, (const char *)g_stage[(i - 1) & 1], prev_len);
+    if (!to_device && i >= 1) dn_host_copy(host + prev_off, (const char *)g_stage[(i - 1) & 1], prev_len);
 }
 
 /* The copies are synchronous, like the reference's cudaMemcpy (src/cuda.c:153-165); work
@@ -322,7 +322,7 @@ void hip_push_array(float *x_gpu, float *x, size_t n)
 {
     if (g_parse_only) return; /* the host copy is the only copy */
     if (g_npacked) packed_drop_range(x_gpu, n);
-    if (sizeof(float) * n >= DN_STAGE_MIN && !host_is_pinned(x, sizeof(float) * n)) {
+    if (sizeof(float) * n >= DN_STAGE_MIN && !dn_host_is_pinned(x, sizeof(float) * n)) {
         staged_copy((char *)x_gpu, (char *)x, sizeof(float) * n, 1);
         return;
     }
@@ -333,7 +333,7 @@ void hip_push_array(float *x_gpu, float *x, size_t n)
 void hip_pull_array(float *x_gpu, float *x, size_t n)
 {
     if (g_parse_only) return;
-    if (sizeof(float) * n >= DN_STAGE_MIN && !host_is_pinned(x, sizeof(float) * n)) {
+    if (sizeof(float) * n >= DN_STAGE_MIN && !dn_host_is_pinned(x, sizeof(float) * n)) {
         staged_copy((char *)x_gpu, (char *)x, sizeof(float) * n, 0);
         return;
     }

@@ -21,6 +21,10 @@ void dn_check_launch(const char *what);
  * (hip_set_parse_only in darknet_hip.h). */
 void hip_require_device(const char *what);
 int hip_parse_only(void);
+/* memcpy split over the host cores (a single core moves less than the host link does), and whether
+ * [x, x+bytes) lies inside a buffer hip_host_alloc handed out */
+void dn_host_copy(char *dst, const char *src, size_t bytes);
+int dn_host_is_pinned(const void *x, size_t bytes);
 
 #ifdef __cplusplus
 }

@@ -38,6 +38,9 @@ void cfg_report_unused(cfg_section *s);
 
 layer make_route_view(int batch, int input_layer, int input_size, float *source_output_gpu);
 
+void dn_forward_gated(network *net, int gate_layer, void (*gate)(void *), void *gate_arg);
+void dn_pipeline_free(network *net);
+
 extern int dn_verbose;
 void *dn_calloc(size_t n, size_t size);
 

@@ -37,6 +37,7 @@ void free_network(network *net)
     if (net->input_gpu) hip_free(net->input_gpu);
     if (net->det_rows_gpu) hip_free(net->det_rows_gpu);
     if (net->det_count_gpu) hip_free((float *)net->det_count_gpu);
+    dn_pipeline_free(net);
     free(net);
 }
 
@@ -110,8 +111,10 @@ static int forward_conv_yolo_pair(network net, int i)
     return 1;
 }
 
-/* The layer loop of src/network.c:773-785 without the copies around it. */
-void forward_network_device(network *netp)
+/* The layer loop of src/network.c:773-785 without the copies around it.  `gate` (may be NULL) is
+ * called once, before the launch that first writes the output of a layer at or after `gate_layer`
+ * (a convolution writes the output of the shortcut or yolo layer fused behind it, hence i + 1). */
+void dn_forward_gated(network *netp, int gate_layer, void (*gate)(void *), void *gate_arg)
 {
     DN_NEED_DEVICE("forward_network_device");
     network net = *netp;
@@ -121,6 +124,10 @@ void forward_network_device(network *netp)
         layer l = net.layers[i];
         net.index = i;
         if (!l.forward_gpu) dn_fatal("layer without a GPU forward");
+        if (gate && gate_layer >= 0 && i + 1 >= gate_layer) {
+            gate(gate_arg);
+            gate = 0;
+        }
         if (forward_conv_shortcut_pair(net, i) || forward_conv_yolo_pair(net, i)) {
             ++i;
             l = net.layers[i];
@@ -130,6 +137,8 @@ void forward_network_device(network *netp)
         net.input_gpu = l.output_gpu;
     }
 }
+
+void forward_network_device(network *netp) { dn_forward_gated(netp, -1, 0, 0); }
 
 /* The same loop with a HIP event between consecutive layers; layer_ms[i] receives layer i's
  * time on the device (a shortcut that ran inside the convolution before it reports 0), and, when

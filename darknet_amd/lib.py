@@ -95,6 +95,8 @@ SIGNATURES = {
     "pull_network_output": (None, [V]), "network_width": (i, [V]), "network_height": (i, [V]),
     "forward_network_device": (None, [V]), "forward_network_profiled": (f, [V, F]),
     "network_set_fusion": (None, [i]),
+    "network_predict_submit": (None, [V, F]), "network_predict_collect": (F, [V]),
+    "network_collected_output": (F, [V, i]), "network_predict_in_flight": (i, [V]),
     "forward_network_profiled_kernels": (f, [V, F, F]),
     "hip_set_parse_only": (None, [i]), "hip_parse_only": (i, []),
     "hip_host_alloc": (F, [z]), "hip_host_free": (None, [F]),

@@ -175,6 +175,7 @@ typedef struct network {
     int *det_count_gpu;
     int det_max_rows;
     int max_batch;
+    void *pipeline;   /* state of network_predict_submit / _collect, made on first use */
 } network;
 
 /* include/darknet.h:515-526 */
@@ -272,6 +273,26 @@ float *network_output(network *net);                        /* src/network.c:755
 void pull_network_output(network *net);                     /* src/network.c:1123 */
 int network_width(network *net);                            /* src/network.c:674 */
 int network_height(network *net);                           /* src/network.c:675 */
+
+/* network_predict in two halves (no counterpart in the reference, whose network_predict uploads,
+ * computes and downloads one after the other, src/network.c:497-508, :766, :786, src/yolo_layer.c:360).
+ * Up to two batches are in flight: while batch n computes, the input of batch n+1 is uploaded and the
+ * outputs of batch n-1 are downloaded on two copy streams of their own.
+ *   network_predict_submit   takes `input` (net->inputs * net->batch floats; copied before the call
+ *                            returns unless it lies in hip_host_alloc memory, which must then stay
+ *                            untouched until that batch is collected) and queues upload, forward
+ *                            and download; ends the process if two batches are already in flight
+ *   network_predict_collect  waits for the oldest batch in flight and returns the host copy of the
+ *                            output layer, what network_predict returns, same bits
+ *   network_collected_output the host copy of layer i (a yolo head or the output layer) of the
+ *                            batch collected last
+ * The pointers stay valid until the next network_predict_submit.  Between a submit and its collect
+ * the device buffers of the network belong to the pipeline: no network_predict, set_batch_network or
+ * detection call on the same network in between.  One host thread per network, as everywhere. */
+void network_predict_submit(network *net, float *input);
+float *network_predict_collect(network *net);
+float *network_collected_output(network *net, int i);
+int network_predict_in_flight(network *net);
 
 /* ---- input side: include/darknet.h:508-513 and src/image.c / src/network.c:579 ------------- */
 typedef struct {

@@ -444,3 +444,57 @@ def test_free_network_returns_its_device_memory(dn):
         for t in texts:
             cycle(t)
     assert device_free_bytes() >= base - (4 << 20), (base, device_free_bytes())
+
+
+def test_pipelined_predict_gives_the_bits_of_network_predict(dn):
+    """network_predict_submit / _collect with two batches in flight: five different batches, pageable
+    and pinned inputs mixed, every yolo head and the output layer bit-equal to network_predict on the
+    same batch; the pointers of a collected batch stay intact while the next one is in flight."""
+    net = api.Network(cfg_text=cfgs.yolov3_tiny(8, 224))
+    fill_params(net.set_conv, net.layers)
+    heads = [i for i, L in enumerate(net.layers) if L["type"] == "yolo"]
+    xs = [synth.uniform01(100 + k, net.inputs * 8) for k in range(5)]
+    want = []
+    for x in xs:
+        final = net.predict(x)
+        want.append({i: net.layer_output(i) for i in heads})
+        assert np.array_equal(final, want[-1][heads[-1]])
+    pinned = api.pinned_array(xs[1].size)
+    pinned[:] = xs[1]
+    feed = [xs[0], pinned, xs[2], xs[3], xs[4]]
+    net.submit(feed[0])
+    assert dn.network_predict_in_flight(net.net) == 1
+    for k in range(1, 5):
+        net.submit(feed[k])                          # batch k uploads and computes ...
+        assert dn.network_predict_in_flight(net.net) == 2
+        final = net.collect()                        # ... while batch k-1 comes back
+        got = {i: net.collected_output(i) for i in heads}
+        for i in heads:
+            assert np.array_equal(got[i], want[k - 1][i]), (k - 1, i)
+        assert np.array_equal(final, want[k - 1][heads[-1]])
+    net.collect()
+    for i in heads:
+        assert np.array_equal(net.collected_output(i), want[4][i]), (4, i)
+    assert dn.network_predict_in_flight(net.net) == 0
+    # the synchronous call still works on the same network afterwards
+    assert np.array_equal(net.predict(xs[0]), want[0][heads[-1]])
+    api.free_pinned_array(pinned)
+    net.free()
+
+
+def test_pipelined_predict_on_a_classifier_and_at_a_smaller_batch(dn):
+    net = api.Network(cfg_text=cfgs.resnext50(4, 64))
+    fill_params(net.set_conv, net.layers)
+    xs = [synth.uniform01(300 + k, net.inputs * 4) for k in range(3)]
+    want = [net.predict(x) for x in xs]
+    net.submit(xs[0])
+    net.submit(xs[1])
+    assert np.array_equal(net.collect(), want[0])
+    net.submit(xs[2])
+    assert np.array_equal(net.collect(), want[1])
+    assert np.array_equal(net.collect(), want[2])
+    net.set_batch(2)
+    small = net.predict(xs[0][:net.inputs * 2])
+    net.submit(xs[0][:net.inputs * 2])
+    assert np.array_equal(net.collect(), small)
+    net.free()

@@ -23,7 +23,7 @@ LAYER_ALIASES = {"convolutional_layer", "maxpool_layer", "route_layer", "avgpool
                  "dropout_layer", "crop_layer", "cost_layer", "local_layer", "detection_layer", "connected_layer"}
 # members this library adds to the reference's structs (the integration guide tells a binder to add them)
 LAYER_ADDITIONS = {"weights_packed_gpu", "xnor_wbits_gpu", "xnor_xbits_gpu", "xnor_wmean_gpu", "output_gpu_is_view"}
-NETWORK_ADDITIONS = {"det_rows_gpu", "det_count_gpu", "det_max_rows", "max_batch"}
+NETWORK_ADDITIONS = {"det_rows_gpu", "det_count_gpu", "det_max_rows", "max_batch", "pipeline"}
 # same name, deliberately another signature
 SIGNATURE_EXCEPTIONS = {
     "check_error": "takes cudaError_t in the reference; the library's is hip_check_error(int)",
