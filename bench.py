@@ -609,6 +609,9 @@ def main():
     ap.add_argument("--precision", default="fp32", choices=["fp32", "bf16", "bf16x3"],
                     help="bf16: the tap-blocked MFMA kernels round their operands to bf16 (opt-in, not the "
                          "headline configuration; its error against fp32 is reported by the tests)")
+    ap.add_argument("--fusion", type=int, default=1, choices=[0, 1, 2],
+                    help="network_set_fusion: 0 layer by layer, 1 layer pairs in one launch with every layer's "
+                         "output written (default), 2 lean (maps only a fused maxpool reads are not written)")
     ap.add_argument("--no-cpu", action="store_true")
     ap.add_argument("--post", action="store_true",
                     help="time letterbox and detection decode + NMS around the forward pass instead")
@@ -628,6 +631,7 @@ def main():
     api.set_gpu(0)
     L = api._lib.load()
     log("device:", L.hip_device_name().decode())
+    L.network_set_fusion(args.fusion)
     if args.workload == "sweep":
         sweep_bench(args, L)
         return
@@ -649,7 +653,8 @@ def main():
 
     cfg_name, size = WORKLOADS[args.workload]
     config = {"workload": f"{args.workload} forward, batch {batch}, {args.precision}, input uniform[0,1), "
-                          f"weights uniform(-1,1)*sqrt(2/(k*k*c)), BN mean 0 var 1 scale 1"}
+                          f"weights uniform(-1,1)*sqrt(2/(k*k*c)), BN mean 0 var 1 scale 1",
+              "fusion": args.fusion}
     config.update({k: m[k] for k in ("gflop_per_image", "device", "wall_ms_per_step", "ms_per_step_with_layer_events",
                                      "pcie_inclusive_ms_per_step", "pcie_inclusive_images_per_s",
                                      "pcie_inclusive_note", "pcie_inclusive_sync_ms_per_step",

@@ -1028,8 +1028,14 @@ __global__ __launch_bounds__(DN_THREADS, 4) void conv_patch_kernel(mfma_args a)
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int W = a.W, H = a.H, P = a.P;
     const int tiles_per_image = P / 256; /* the host checks P % 256 == 0 */
-    const int b = blockIdx.x / tiles_per_image;
-    const int p0 = (blockIdx.x - b * tiles_per_image) * 256;
+    /* Workgroup ids go round the eight XCDs, each with an L2 of its own, and neighbouring tiles
+     * share input rows (a 256-pixel tile reads three or four rows to produce part of one): XCD x
+     * takes the x-th eighth of the tile order, so that neighbours meet in one L2 instead of each
+     * fetching those rows into its own. */
+    const int ntiles = gridDim.x, xq = ntiles >> 3, xr = ntiles & 7, xcd = blockIdx.x & 7;
+    const int tile = xcd * xq + (xcd < xr ? xcd : xr) + (blockIdx.x >> 3);
+    const int b = tile / tiles_per_image;
+    const int p0 = (tile - b * tiles_per_image) * 256;
     const int y0 = p0 / W, y1 = (p0 + 255) / W;
     const int nrows = y1 - y0 + 3, RS = W + 8; /* a row: four zeros, the W pixels, four zeros */
 
@@ -1113,6 +1119,12 @@ __global__ __launch_bounds__(DN_THREADS, 4) void conv_patch_kernel(mfma_args a)
 #pragma unroll
     for (int i = 0; i < TM; ++i) {
         const conv_row_t row = rows_s[i * 32 + li];
+        /* the tail arithmetic with every lane at work; only the turn through LDS below goes by halves */
+#pragma unroll
+        for (int j = 0; j < 2; ++j)
+#pragma unroll
+            for (int r = 0; r < 16; ++r)
+                acc[i][j][r] = conv_tail_one(acc[i][j][r], row, conv_f2{a.slope_hi, a.slope_lo});
 #pragma unroll
         for (int hf = 0; hf < 2; ++hf) {
             __syncthreads(); /* the buffer is free: pixels read (first pass), rows stored (later ones) */
@@ -1123,10 +1135,10 @@ __global__ __launch_bounds__(DN_THREADS, 4) void conv_patch_kernel(mfma_args a)
 #pragma unroll
                     for (int rg = 0; rg < 4; ++rg) {
                         float4 o;
-                        o.x = conv_tail_one(acc[i][j][rg * 4 + 0], row, conv_f2{a.slope_hi, a.slope_lo});
-                        o.y = conv_tail_one(acc[i][j][rg * 4 + 1], row, conv_f2{a.slope_hi, a.slope_lo});
-                        o.z = conv_tail_one(acc[i][j][rg * 4 + 2], row, conv_f2{a.slope_hi, a.slope_lo});
-                        o.w = conv_tail_one(acc[i][j][rg * 4 + 3], row, conv_f2{a.slope_hi, a.slope_lo});
+                        o.x = acc[i][j][rg * 4 + 0];
+                        o.y = acc[i][j][rg * 4 + 1];
+                        o.z = acc[i][j][rg * 4 + 2];
+                        o.w = acc[i][j][rg * 4 + 3];
                         const int q = wave * 16 + j * 8 + 2 * rg + kh; /* quad of four pixels within the tile */
                         *(float4 *)&buf[f16 * 256 + ((q ^ f16) << 2)] = o;
                     }

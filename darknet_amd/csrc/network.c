@@ -67,11 +67,93 @@ void set_batch_network(network *net, int b)
     for (i = 0; i < net->n; ++i) net->layers[i].batch = b;
 }
 
-static int g_fuse_shortcut = 1;
+static int g_fuse_shortcut = 1; /* 0 off, 1 on, 2 on and lean */
 
-/* 1 (default): a convolution followed directly by a same-geometry shortcut runs as one kernel
- * launch sequence; 0: every layer runs on its own.  Both layers' outputs are written either way. */
-void network_set_fusion(int on) { g_fuse_shortcut = on ? 1 : 0; }
+/* 0: every layer runs on its own, as in src/network.c:773-785.
+ * 1 (default): layer pairs run as one launch where a kernel serves both - a convolution and the
+ *    same-geometry shortcut or the yolo head behind it, an xnor convolution and the 2x2 stride-2
+ *    maxpool behind it - and an xnor convolution writes the sign bits the next xnor convolution
+ *    reads.  Every layer's output buffer is written and holds the bits of the unfused sequence.
+ * 2 (lean): as 1, but the map of an xnor convolution that only the maxpool fused behind it reads
+ *    is not written (its output buffer keeps whatever it held; layer_output_host refuses it). */
+void network_set_fusion(int on) { g_fuse_shortcut = on < 0 ? 0 : on > 2 ? 2 : on; }
+
+/* An xnor convolution and the maxpool behind it that the pooled kernel serves: 3x3 / stride 1 /
+ * pad 1 into an even-sized map, pooled 2x2 with stride 2 from the map's first pixel. */
+static int xnor_pool_pair(const network *net, int i)
+{
+    const layer *l, *m;
+    if (!g_fuse_shortcut || i < 0 || i + 1 >= net->n) return 0;
+    l = &net->layers[i];
+    m = &net->layers[i + 1];
+    if (l->type != CONVOLUTIONAL || !l->xnor || m->type != MAXPOOL) return 0;
+    if (l->size != 3 || l->stride != 1 || l->pad != 1 || (l->out_h & 1) || (l->out_w & 1)) return 0;
+    if (m->size != 2 || m->stride != 2 || m->pad / 2 != 0) return 0;
+    if (m->h != l->out_h || m->w != l->out_w || m->c != l->out_c || m->batch != l->batch) return 0;
+    if (m->out_h * 2 != m->h || m->out_w * 2 != m->w) return 0;
+    return 1;
+}
+
+/* The xnor convolution that reads layer q's output as its input and can take its sign bits from
+ * the kernel that wrote that output: the layer right behind it.  -1: none. */
+static int xnor_bits_consumer(const network *net, int q)
+{
+    const layer *p, *k;
+    if (!g_fuse_shortcut || q < 0 || q + 1 >= net->n) return -1;
+    p = &net->layers[q];
+    k = &net->layers[q + 1];
+    if (k->type != CONVOLUTIONAL || !k->xnor || !k->xnor_xbits_gpu) return -1;
+    if (k->c != p->out_c || k->h != p->out_h || k->w != p->out_w || k->batch != p->batch) return -1;
+    return q + 1;
+}
+
+/* Whether xnor convolution i finds its input's sign bits already written by the layer in front. */
+static int xnor_bits_ready(const network *net, int i)
+{
+    if (i >= 1 && net->layers[i - 1].type == CONVOLUTIONAL && net->layers[i - 1].xnor)
+        return xnor_bits_consumer(net, i - 1) == i;
+    if (i >= 2 && net->layers[i - 1].type == MAXPOOL && xnor_pool_pair(net, i - 2))
+        return xnor_bits_consumer(net, i - 1) == i;
+    return 0;
+}
+
+/* Whether anything but the layer right behind it reads layer i's output. */
+static int layer_output_read_elsewhere(const network *net, int i)
+{
+    int k, j;
+    if (i >= net->n - 1) return 1;
+    for (k = i + 1; k < net->n; ++k) {
+        const layer *l = &net->layers[k];
+        if (l->type == ROUTE)
+            for (j = 0; j < l->n; ++j)
+                if (l->input_layers[j] == i) return 1;
+        if (l->type == SHORTCUT && l->index == i) return 1;
+    }
+    return 0;
+}
+
+/* lean mode: the map of xnor convolution i is not written */
+static int xnor_map_skipped(const network *net, int i)
+{
+    return g_fuse_shortcut == 2 && xnor_pool_pair(net, i) && !layer_output_read_elsewhere(net, i);
+}
+
+/* Runs xnor convolution i, with the maxpool behind it when xnor_pool_pair says so.  Returns the
+ * number of layers it ran beyond i (0 or 1). */
+static int forward_xnor(network net, int i)
+{
+    const layer l = net.layers[i];
+    const int pooled = xnor_pool_pair(&net, i);
+    const int q = i + pooled;
+    const int k = xnor_bits_consumer(&net, q);
+    forward_convolutional_xnor_fused_gpu(net.input_gpu, l.xnor_wbits_gpu, l.xnor_wmean_gpu, l.xnor_xbits_gpu,
+                                         xnor_bits_ready(&net, i), l.biases_gpu, l.scales_gpu, l.rolling_mean_gpu,
+                                         l.rolling_variance_gpu, xnor_map_skipped(&net, i) ? 0 : l.output_gpu,
+                                         pooled ? net.layers[i + 1].output_gpu : 0,
+                                         k >= 0 ? net.layers[k].xnor_xbits_gpu : 0, l.batch, l.c, l.h, l.w, l.n, l.size,
+                                         l.stride, l.pad, l.batch_normalize, (int)l.activation);
+    return pooled;
+}
 
 /* Runs layers i and i+1 together when they are a convolution and the residual add of a
  * darknet53 block (src/shortcut_layer.c:77-83 with equal geometries).  Returns 1 if it did. */
@@ -128,7 +210,10 @@ void dn_forward_gated(network *netp, int gate_layer, void (*gate)(void *), void 
             gate(gate_arg);
             gate = 0;
         }
-        if (forward_conv_shortcut_pair(net, i) || forward_conv_yolo_pair(net, i)) {
+        if (l.type == CONVOLUTIONAL && l.xnor && g_fuse_shortcut) {
+            i += forward_xnor(net, i);
+            l = net.layers[i];
+        } else if (forward_conv_shortcut_pair(net, i) || forward_conv_yolo_pair(net, i)) {
             ++i;
             l = net.layers[i];
         } else {
@@ -176,7 +261,14 @@ float forward_network_profiled_kernels(network *netp, float *layer_ms, float *ke
             conv_profile_next(ks[i], ke[i]);
             timed = 1;
         }
-        if (forward_conv_shortcut_pair(net, i) || forward_conv_yolo_pair(net, i)) {
+        if (l.type == CONVOLUTIONAL && l.xnor && g_fuse_shortcut) {
+            if (forward_xnor(net, i)) {
+                hip_event_record(ev[i + 1]);
+                ++i;
+                if (kernel_ms) kernel_ms[i] = -1.f;
+                l = net.layers[i];
+            }
+        } else if (forward_conv_shortcut_pair(net, i) || forward_conv_yolo_pair(net, i)) {
             hip_event_record(ev[i + 1]);
             ++i;
             if (kernel_ms) kernel_ms[i] = -1.f;
@@ -281,6 +373,9 @@ float *layer_output_host(network *net, int i)
     l = &net->layers[i];
     /* a dropout layer's output is the buffer of the layer before it (src/parser.c:829-836) */
     if (l->type == DROPOUT && i > 0) return layer_output_host(net, i - 1);
+    if (xnor_map_skipped(net, i))
+        dn_fatal("layer_output_host: in lean mode (network_set_fusion(2)) this convolution's map is not written; "
+                 "only the maxpool behind it is");
     if (!l->output) {
         /* sized for the batch the network was built with: set_batch_network may come back up to it */
         const int cap = net->max_batch > l->batch ? net->max_batch : l->batch;
@@ -297,6 +392,8 @@ int *layer_indexes_host(network *net, int i)
     if (i < 0 || i >= net->n) dn_fatal("layer_indexes_host: layer index out of range");
     l = &net->layers[i];
     if (l->type != MAXPOOL || !l->indexes_gpu) dn_fatal("layer_indexes_host: layer has no indexes");
+    if (i > 0 && xnor_map_skipped(net, i - 1))
+        dn_fatal("layer_indexes_host: in lean mode (network_set_fusion(2)) the map this layer pools is not written");
     if (!l->indexes)
         l->indexes = (int *)dn_calloc((size_t)l->outputs * (net->max_batch > l->batch ? net->max_batch : l->batch), sizeof(int));
     /* the forward pass leaves the argmax out (only the backward pass reads it): compute it now from

@@ -304,6 +304,27 @@ void forward_convolutional_xnor_packed_gpu(const float *input, const unsigned *w
                                            float *output, int batch, int c, int h, int w, int n, int size,
                                            int stride, int pad, int batch_normalize, int activation);
 
+/* forward_convolutional_xnor_packed_gpu with what the layers around an xnor convolution otherwise do
+ * in passes of their own (no counterpart in the reference):
+ *   xbits_ready != 0  xbits already holds the sign bits of the input (the layer that produced the
+ *                     input wrote them through its own next_xbits); `input` is then not read
+ *   pool_output       NULL, or the output of the 2x2 stride-2 maxpool layer behind this one
+ *                     (src/maxpool_layer.c:79-114 with size 2, stride 2, padding 0 or 1), written from
+ *                     the same pass: [batch][n][out_h/2][out_w/2].  Needs size 3, stride 1, pad 1 and
+ *                     an even out_h, out_w.  `output` may then be NULL: the convolution's own map is
+ *                     not written
+ *   next_xbits        NULL, or where to write the sign bits (x > 0) of pool_output - of `output` when
+ *                     there is no pool_output - in the layout xnor_pack_input_gpu gives that tensor:
+ *                     xnor_input_words(batch, n, its height, its width) words
+ * Every buffer written holds the bits the separate calls (forward_convolutional_xnor_packed_gpu,
+ * forward_maxpool_gpu, xnor_pack_input_gpu) would write. */
+void forward_convolutional_xnor_fused_gpu(const float *input, const unsigned *wbits, const float *wmean,
+                                          unsigned *xbits, int xbits_ready, const float *biases,
+                                          const float *scales, const float *rolling_mean,
+                                          const float *rolling_variance, float *output, float *pool_output,
+                                          unsigned *next_xbits, int batch, int c, int h, int w, int n, int size,
+                                          int stride, int pad, int batch_normalize, int activation);
+
 /* forward_maxpool_layer_gpu (src/maxpool_layer_kernels.cu:87-99), CPU semantics of
  * src/maxpool_layer.c:79-114: window origin (-pad)/2, outside = -FLT_MAX, first maximum wins.
  * indexes may be NULL (inference never reads them). */
