@@ -69,6 +69,14 @@ extern "C" void conv_direct_forward(const float *, const float *, const float *,
                                     const float *, const float *, float *, int, int, int, int, int,
                                     int, int, int, int, int, int);
 
+/* conv_first.hip: the kernel of 3-channel first layers */
+extern "C" int conv_first_serves(int batch, int c, int h, int w, int n, int groups, int size, int stride, int pad);
+extern "C" const char *conv_first_kernel_name(int n, int pooled);
+extern "C" void conv_first_forward(const float *input, const float *weights, const float *biases, const float *scales,
+                                   const float *rolling_mean, const float *rolling_variance, float *out, float *pool,
+                                   unsigned *bits, int batch, int h, int w, int n, int batch_normalize, double slope,
+                                   int cus, void *start, void *stop);
+
 struct mfma_args {
     const float *in;
     const float *wp; /* packed weights */
@@ -1477,6 +1485,8 @@ extern "C" const char *conv_kernel_name_geometry(int batch, int c, int h, int w,
     int mode = conv_mode(c, groups, size, stride, pad, (long)batch * in_img);
     if (g_algo != 1 && !(size == 3 && pad != 1) && conv_grouped_tile(n, c, groups, size)) mode = 10 + size;
     if (columns >= (1L << 31) - 512) mode = -1;
+    if (g_algo == 0 && mode == 3 && conv_first_serves(batch, c, h, w, n, groups, size, stride, pad))
+        return conv_first_kernel_name(n, 0);
     const int patch = g_algo == 0 && mode == 3 && conv_patch_floats(c, h, w, n, groups, size, stride, pad) > 0;
     return kernel_name(n, c, groups, size, columns, patch, mode);
 }
@@ -1557,7 +1567,7 @@ extern "C" void conv_set_bands(int bands) { g_tune_bands = bands; }
 
 extern "C" void conv_set_ksplit(int split, int tile_n)
 {
-    if (split < 0 || (tile_n != 0 && tile_n != 1 && tile_n != 64 && tile_n != 128))
+    if (split < -32 || (tile_n != 0 && tile_n != 1 && tile_n != 64 && tile_n != 128))
         dn_fatal("conv_set_ksplit: split >= 0, tile_n 0, 1, 64 or 128");
     g_tune_split = split;
     g_tune_bn = tile_n;
@@ -1593,6 +1603,10 @@ static long plan_split(long tiles, int kch, int cus, int *split, double fixed_sc
 {
     *split = 1;
     if (g_algo == 3 || cus <= 0) return tiles;
+    if (g_tune_split < 0) { /* tuning hook: every tile cut into -split slices */
+        *split = -g_tune_split < kch ? -g_tune_split : kch;
+        return *split > 1 ? 0 : tiles;
+    }
     const long whole = tiles / cus * cus;
     const long tail = tiles - whole;
     if (tail == 0) return tiles;
@@ -1855,6 +1869,16 @@ static void conv_forward(const float *input, const float *weights, const float *
         return;
     }
 
+    /* first layers (3 channels, 3x3 / 1 / pad 1, even height, width a multiple of 32): their own kernel */
+    if (g_algo == 0 && mode == 3 && !sum && conv_first_serves(batch, c, h, w, n, groups, size, stride, pad)) {
+        const int dev = hip_get_device();
+        if (dev >= 0 && dev < DN_MAX_DEVICES && !g_cus_dev[dev]) conv_device_setup();
+        conv_first_forward(input, weights, biases, scales, rolling_mean, rolling_variance, output, 0, 0, batch, h, w, n,
+                           batch_normalize, slope, dev >= 0 && dev < DN_MAX_DEVICES ? g_cus_dev[dev] : 0,
+                           (void *)g_prof_start, (void *)g_prof_stop);
+        g_prof_start = g_prof_stop = 0;
+        return;
+    }
     const long patch = (g_algo == 0 && mode == 3 && !sum) ? conv_patch_floats(c, h, w, n, groups, size, stride, pad) : 0;
     if (g_noalloc && !patch && (!packed || (g_precision == 1 && mode == 13))) {
         fprintf(stderr, !packed ? "forward_convolutional_noalloc_gpu: this geometry runs on packed weights; pass the "
@@ -2033,4 +2057,39 @@ extern "C" int forward_convolutional_noalloc_gpu(const float *input, const float
     g_noalloc = 0;
     if (g_noalloc_error) g_prof_start = g_prof_stop = 0; /* a pending timing pair must not stamp a later, unrelated call */
     return g_noalloc_error ? -1 : 0;
+}
+
+/* Whether forward_convolutional_maxpool_gpu serves the pair: a 3-channel 3x3 / stride 1 / pad 1
+ * convolution of up to 64 filters with an activation its tail carries (leaky, linear, relu), over an
+ * image of even height and a width that is a multiple of 32. */
+extern "C" int conv_maxpool_fusable(int batch, int c, int h, int w, int n, int groups, int size, int stride, int pad,
+                                    int activation)
+{
+    double slope;
+    if (g_algo != 0 || !conv_inline_activation(activation, &slope)) return 0;
+    return conv_first_serves(batch, c, h, w, n, groups, size, stride, pad);
+}
+
+extern "C" void forward_convolutional_maxpool_gpu(const float *input, const float *weights, const float *biases,
+                                                  const float *scales, const float *rolling_mean,
+                                                  const float *rolling_variance, float *output, float *pool_output,
+                                                  unsigned *next_xbits, int batch, int c, int h, int w, int n,
+                                                  int groups, int size, int stride, int pad, int batch_normalize,
+                                                  int activation)
+{
+    hip_require_device("forward_convolutional_maxpool_gpu");
+    double slope = 1.;
+    if (!input || !weights || !biases || !pool_output) dn_fatal("forward_convolutional_maxpool_gpu: null pointer");
+    if (batch_normalize && (!scales || !rolling_mean || !rolling_variance))
+        dn_fatal("forward_convolutional_maxpool_gpu: batch_normalize needs scales, rolling_mean, rolling_variance");
+    if (!conv_inline_activation(activation, &slope) ||
+        !conv_first_serves(batch, c, h, w, n, groups, size, stride, pad))
+        dn_fatal("forward_convolutional_maxpool_gpu: serves 3-channel 3x3 / 1 / pad 1 layers of up to 64 filters with a "
+                 "leaky, linear or relu activation, even height and a width that is a multiple of 32 "
+                 "(conv_maxpool_fusable)");
+    const int dev = hip_get_device();
+    if (dev < 0 || dev >= DN_MAX_DEVICES) dn_fatal("forward_convolutional_maxpool_gpu: device index out of range");
+    if (!g_cus_dev[dev]) conv_device_setup();
+    conv_first_forward(input, weights, biases, scales, rolling_mean, rolling_variance, output, pool_output, next_xbits,
+                       batch, h, w, n, batch_normalize, slope, g_cus_dev[dev], 0, 0);
 }

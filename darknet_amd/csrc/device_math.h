@@ -112,4 +112,55 @@ __device__ __forceinline__ float dn_bn_apply(float acc, const dn_bn_row &r, int 
     return __fadd_rn(x, r.bias);
 }
 
+/* A double constant as an unevaluated sum of two floats: fmaf(x, hi, x*lo) reproduces
+ * (float)((double)x * c) except when the exact product lies within ~2^-48 (relative) of a float
+ * rounding boundary, at a third of the instructions of the convert / multiply / convert sequence. */
+struct dn_f2 {
+    float hi, lo;
+};
+
+__host__ __device__ inline dn_f2 dn_split(double c)
+{
+    dn_f2 r;
+    r.hi = (float)c;
+    r.lo = (float)(c - (double)r.hi);
+    return r;
+}
+
+__device__ __forceinline__ float dn_mul_f2(float x, dn_f2 c) { return fmaf(x, c.hi, __fmul_rn(x, c.lo)); }
+
+/* Per-filter constants of the convolution tail in that form, and the tail itself: normalize
+ * (src/blas.c:154, as a multiplication by the reciprocal of the double denominator), scale, bias
+ * (src/batchnorm_layer.c:151-154), each step rounded to float as the reference's separate passes
+ * do, then the activation y > 0 ? y : slope*y (leaky .1, linear 1, relu 0).  Without batch-norm the
+ * constants are neutral and change no bit. */
+struct dn_tail_row {
+    dn_f2 inv;
+    float mean, scale, bias;
+};
+
+__device__ __forceinline__ dn_tail_row dn_tail_make(int bn, float bias, float scale, float mean, float var)
+{
+    dn_tail_row r;
+    r.bias = bias;
+    if (bn) {
+        r.inv = dn_split(1.0 / (sqrt((double)var) + (double).000001f));
+        r.mean = mean;
+        r.scale = scale;
+    } else {
+        r.inv.hi = 1.f;
+        r.inv.lo = 0.f;
+        r.mean = 0.f;
+        r.scale = 1.f;
+    }
+    return r;
+}
+
+__device__ __forceinline__ float dn_tail(float acc, const dn_tail_row &row, dn_f2 slope)
+{
+    float x = dn_mul_f2(__fsub_rn(acc, row.mean), row.inv);
+    x = __fadd_rn(__fmul_rn(x, row.scale), row.bias);
+    return (x > 0) ? x : dn_mul_f2(x, slope);
+}
+
 #endif

@@ -94,6 +94,22 @@ static int xnor_pool_pair(const network *net, int i)
     return 1;
 }
 
+/* A first layer (3 channels, 3x3 / stride 1 / pad 1) and the 2x2 stride-2 maxpool behind it that
+ * forward_convolutional_maxpool_gpu serves in one pass. */
+static int conv_pool_pair(const network *net, int i)
+{
+    const layer *l, *m;
+    if (!g_fuse_shortcut || i < 0 || i + 1 >= net->n) return 0;
+    l = &net->layers[i];
+    m = &net->layers[i + 1];
+    if (l->type != CONVOLUTIONAL || l->xnor || m->type != MAXPOOL) return 0;
+    if (m->size != 2 || m->stride != 2 || m->pad / 2 != 0) return 0;
+    if (m->h != l->out_h || m->w != l->out_w || m->c != l->out_c || m->batch != l->batch) return 0;
+    if (m->out_h * 2 != m->h || m->out_w * 2 != m->w) return 0;
+    return conv_maxpool_fusable(l->batch, l->c, l->h, l->w, l->n, l->groups, l->size, l->stride, l->pad,
+                                (int)l->activation);
+}
+
 /* The xnor convolution that reads layer q's output as its input and can take its sign bits from
  * the kernel that wrote that output: the layer right behind it.  -1: none. */
 static int xnor_bits_consumer(const network *net, int q)
@@ -112,7 +128,7 @@ static int xnor_bits_ready(const network *net, int i)
 {
     if (i >= 1 && net->layers[i - 1].type == CONVOLUTIONAL && net->layers[i - 1].xnor)
         return xnor_bits_consumer(net, i - 1) == i;
-    if (i >= 2 && net->layers[i - 1].type == MAXPOOL && xnor_pool_pair(net, i - 2))
+    if (i >= 2 && net->layers[i - 1].type == MAXPOOL && (xnor_pool_pair(net, i - 2) || conv_pool_pair(net, i - 2)))
         return xnor_bits_consumer(net, i - 1) == i;
     return 0;
 }
@@ -132,10 +148,27 @@ static int layer_output_read_elsewhere(const network *net, int i)
     return 0;
 }
 
-/* lean mode: the map of xnor convolution i is not written */
+/* lean mode: the map of convolution i, which only the maxpool fused behind it reads, is not written */
 static int xnor_map_skipped(const network *net, int i)
 {
-    return g_fuse_shortcut == 2 && xnor_pool_pair(net, i) && !layer_output_read_elsewhere(net, i);
+    return g_fuse_shortcut == 2 && (xnor_pool_pair(net, i) || conv_pool_pair(net, i)) &&
+           !layer_output_read_elsewhere(net, i);
+}
+
+/* Runs convolution i and the maxpool behind it as one pass when conv_pool_pair says so.  Returns 1 if it did. */
+static int forward_conv_pool_pair(network net, int i)
+{
+    layer l, m;
+    int k;
+    if (!conv_pool_pair(&net, i)) return 0;
+    l = net.layers[i];
+    m = net.layers[i + 1];
+    k = xnor_bits_consumer(&net, i + 1);
+    forward_convolutional_maxpool_gpu(net.input_gpu, l.weights_gpu, l.biases_gpu, l.scales_gpu, l.rolling_mean_gpu,
+                                      l.rolling_variance_gpu, xnor_map_skipped(&net, i) ? 0 : l.output_gpu,
+                                      m.output_gpu, k >= 0 ? net.layers[k].xnor_xbits_gpu : 0, l.batch, l.c, l.h, l.w,
+                                      l.n, l.groups, l.size, l.stride, l.pad, l.batch_normalize, (int)l.activation);
+    return 1;
 }
 
 /* Runs xnor convolution i, with the maxpool behind it when xnor_pool_pair says so.  Returns the
@@ -213,7 +246,8 @@ void dn_forward_gated(network *netp, int gate_layer, void (*gate)(void *), void 
         if (l.type == CONVOLUTIONAL && l.xnor && g_fuse_shortcut) {
             i += forward_xnor(net, i);
             l = net.layers[i];
-        } else if (forward_conv_shortcut_pair(net, i) || forward_conv_yolo_pair(net, i)) {
+        } else if (forward_conv_shortcut_pair(net, i) || forward_conv_yolo_pair(net, i) ||
+                   forward_conv_pool_pair(net, i)) {
             ++i;
             l = net.layers[i];
         } else {
@@ -268,7 +302,8 @@ float forward_network_profiled_kernels(network *netp, float *layer_ms, float *ke
                 if (kernel_ms) kernel_ms[i] = -1.f;
                 l = net.layers[i];
             }
-        } else if (forward_conv_shortcut_pair(net, i) || forward_conv_yolo_pair(net, i)) {
+        } else if (forward_conv_shortcut_pair(net, i) || forward_conv_yolo_pair(net, i) ||
+                   forward_conv_pool_pair(net, i)) {
             hip_event_record(ev[i + 1]);
             ++i;
             if (kernel_ms) kernel_ms[i] = -1.f;

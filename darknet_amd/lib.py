@@ -61,6 +61,8 @@ SIGNATURES = {
     "forward_convolutional_xnor_gpu": (None, [V] * 10 + [i] * 10),
     "forward_convolutional_xnor_packed_gpu": (None, [V] * 9 + [i] * 10),
     "forward_convolutional_xnor_fused_gpu": (None, [V] * 4 + [i] + [V] * 7 + [i] * 10),
+    "conv_maxpool_fusable": (i, [i] * 10),
+    "forward_convolutional_maxpool_gpu": (None, [V] * 9 + [i] * 11),
     "forward_maxpool_gpu": (None, [V, V, V] + [i] * 7),
     "forward_route_gpu": (None, [C.POINTER(V), I, i, V, i]),
     "forward_shortcut_gpu": (None, [V, V, V] + [i] * 7 + [f, f, i]),

@@ -343,12 +343,13 @@ float forward_network_profiled(network *net, float *layer_ms);
 float forward_network_profiled_kernels(network *net, float *layer_ms, float *kernel_ms);
 /* 1 (default): forward_network_device runs a convolution and the same-geometry shortcut right
  * after it as one pass (forward_convolutional_shortcut_gpu), likewise a convolution and the yolo
- * head it feeds (forward_convolutional_yolo_gpu) and an xnor convolution and the 2x2 stride-2
- * maxpool behind it, and an xnor convolution writes the sign bits the xnor convolution behind it
- * reads (forward_convolutional_xnor_fused_gpu); 0: layer by layer as src/network.c:773-785
- * does.  Every layer's output buffer is written in both modes and holds the same bits.
- * 2 (lean): as 1, except that the map of an xnor convolution which nothing but the maxpool fused
- * behind it reads is not written: its output buffer is stale, layer_output_host() refuses it. */
+ * head it feeds (forward_convolutional_yolo_gpu), a first layer or an xnor convolution and the 2x2
+ * stride-2 maxpool behind it (forward_convolutional_maxpool_gpu, forward_convolutional_xnor_fused_gpu),
+ * and the layer in front of an xnor convolution writes the sign bits that convolution reads;
+ * 0: layer by layer as src/network.c:773-785 does.  Every layer's output buffer is written in both
+ * modes and holds the same bits.
+ * 2 (lean): as 1, except that the map of a convolution which nothing but the maxpool fused behind
+ * it reads is not written: its output buffer is stale, layer_output_host() refuses it. */
 void network_set_fusion(int on);
 float *layer_output_host(network *net, int i);
 int *layer_indexes_host(network *net, int i);

@@ -304,6 +304,24 @@ void forward_convolutional_xnor_packed_gpu(const float *input, const unsigned *w
                                            float *output, int batch, int c, int h, int w, int n, int size,
                                            int stride, int pad, int batch_normalize, int activation);
 
+/* A first layer and the 2x2 stride-2 maxpool layer behind it in one pass (no counterpart in the
+ * reference): forward_convolutional_gpu (src/convolutional_kernels.cu:73-135) for a 3-channel 3x3 /
+ * stride 1 / pad 1 convolution of up to 64 filters, plus forward_maxpool_layer_gpu
+ * (src/maxpool_layer_kernels.cu:87-99; size 2, stride 2, padding 0 or 1) on its output.
+ *   output       the convolution's map [batch][n][h][w], or NULL: then only the pooled map is written
+ *   pool_output  [batch][n][h/2][w/2]
+ *   next_xbits   NULL, or where to write the sign bits (x > 0) of pool_output for an xnor convolution
+ *                that reads it, in the layout of xnor_pack_input_gpu: xnor_input_words(batch, n, h/2, w/2)
+ * Every buffer written holds the bits of the separate calls.  conv_maxpool_fusable() says whether a
+ * geometry and activation are served; anything else ends the process. */
+int conv_maxpool_fusable(int batch, int c, int h, int w, int n, int groups, int size, int stride, int pad,
+                         int activation);
+void forward_convolutional_maxpool_gpu(const float *input, const float *weights, const float *biases,
+                                       const float *scales, const float *rolling_mean,
+                                       const float *rolling_variance, float *output, float *pool_output,
+                                       unsigned *next_xbits, int batch, int c, int h, int w, int n, int groups,
+                                       int size, int stride, int pad, int batch_normalize, int activation);
+
 /* forward_convolutional_xnor_packed_gpu with what the layers around an xnor convolution otherwise do
  * in passes of their own (no counterpart in the reference):
  *   xbits_ready != 0  xbits already holds the sign bits of the input (the layer that produced the

@@ -1,0 +1,131 @@
+"""The first-layer kernel (3 channels, 3x3, stride 1, pad 1) through the C-ABI: against the CPU
+checker and the fp64 convolution as every convolution is, and its pooled forms against the separate
+calls they stand for - forward_convolutional_gpu, forward_maxpool_gpu, xnor_pack_input_gpu - bit
+for bit.  Widths of one to several 128-column tiles with and without a ragged last tile, two-row
+images, 1 to 64 filters, batches whose tiles cross images, both signs of the batch-norm scale."""
+import numpy as np
+import pytest
+
+from darknet_amd import api, cfgs, synth
+from oracle.cpu import ACTIVATIONS
+
+from util import REL_TOL, fill_params, norm_err
+
+pytestmark = pytest.mark.gpu
+D = api.DeviceArray
+
+
+class First:
+    def __init__(self, dn, seed, b, h, w, n, act="leaky", bn=1):
+        self.dn, self.geom, self.act, self.bn = dn, (b, h, w, n), act, bn
+        self.x = synth.uniform(seed, b * 3 * h * w).reshape(b, 3, h, w)
+        self.wt = synth.conv_weights(seed + 1, n, 3, 3)
+        self.bias, self.sc, self.mu, self.var = synth.bn_random(seed + 2, n)
+        self.sc = self.sc.copy()
+        self.sc[1::3] *= -1.0
+        self.dev = [D(a) for a in (self.x, self.wt, self.bias, self.sc, self.mu, self.var)]
+
+    def tail(self):
+        b, h, w, n = self.geom
+        return [b, 3, h, w, n, 1, 3, 1, 1, self.bn, ACTIVATIONS.index(self.act)]
+
+    def conv(self):
+        b, h, w, n = self.geom
+        d = self.dev
+        out = D(np.full(b * n * h * w, np.nan, np.float32))
+        self.dn.forward_convolutional_gpu(d[0].ptr, d[1].ptr, None, d[2].ptr, d[3].ptr, d[4].ptr, d[5].ptr, out.ptr,
+                                          *self.tail())
+        return out
+
+    def separate(self):
+        b, h, w, n = self.geom
+        out = self.conv()
+        pooled = D(np.full(b * n * (h // 2) * (w // 2), np.nan, np.float32))
+        self.dn.forward_maxpool_gpu(out.ptr, pooled.ptr, None, b, n, h, w, 2, 2, 1)
+        bits = D(n=self.dn.xnor_input_words(b, n, h // 2, w // 2), dtype=np.int32)
+        self.dn.xnor_pack_input_gpu(pooled.ptr, bits.ptr, b, n, h // 2, w // 2)
+        return out.numpy().view(np.uint32), pooled.numpy().view(np.uint32), bits.numpy().view(np.uint32)
+
+    def fused(self, write_map=True):
+        b, h, w, n = self.geom
+        d = self.dev
+        out = D(np.full(b * n * h * w, np.nan, np.float32))
+        pooled = D(np.full(b * n * (h // 2) * (w // 2), np.nan, np.float32))
+        bits = D(np.full(self.dn.xnor_input_words(b, n, h // 2, w // 2), -1, np.int32))
+        self.dn.forward_convolutional_maxpool_gpu(d[0].ptr, d[1].ptr, d[2].ptr, d[3].ptr, d[4].ptr, d[5].ptr,
+                                                  out.ptr if write_map else None, pooled.ptr, bits.ptr, *self.tail())
+        return out.numpy().view(np.uint32), pooled.numpy().view(np.uint32), bits.numpy().view(np.uint32)
+
+
+GEOMS = [(1, 2, 32, 16), (2, 6, 64, 32), (3, 10, 160, 17), (1, 16, 416, 32), (2, 8, 128, 64), (5, 4, 96, 33),
+         (1, 34, 256, 1), (2, 12, 288, 48)]
+
+
+@pytest.mark.parametrize("b,h,w,n", GEOMS)
+def test_first_layer_against_the_checker(dn, orc, b, h, w, n):
+    assert dn.conv_maxpool_fusable(b, 3, h, w, n, 1, 3, 1, 1, ACTIVATIONS.index("leaky")) == 1
+    assert dn.conv_kernel_name_geometry(b, 3, h, w, n, 1, 3, 1, 1).decode().startswith("conv_first_kernel")
+    cs = First(dn, 3, b, h, w, n)
+    got = cs.conv().numpy((b, n, h, w))
+    want = orc.conv(cs.x, cs.wt, cs.bias, cs.sc, cs.mu, cs.var, n=n, size=3, stride=1, pad=1, groups=1,
+                    batch_normalize=1, activation="leaky")
+    assert not np.isnan(got).any()
+    assert norm_err(got, want) <= REL_TOL
+    # the same layer on the generic kernel (conv_set_algo(3) leaves the first-layer kernels out), which pairs
+    # the k of an MFMA differently: the same values to rounding
+    dn.conv_set_algo(3)
+    try:
+        other = cs.conv().numpy((b, n, h, w))
+    finally:
+        dn.conv_set_algo(0)
+    assert norm_err(got, other) <= 2e-6
+
+
+@pytest.mark.parametrize("b,h,w,n", GEOMS)
+@pytest.mark.parametrize("act,bn", [("leaky", 1), ("relu", 0), ("linear", 1)])
+def test_first_layer_with_pool_and_bits_in_one_pass(dn, b, h, w, n, act, bn):
+    cs = First(dn, 11, b, h, w, n, act=act, bn=bn)
+    want_map, want_pool, want_bits = cs.separate()
+    got_map, got_pool, got_bits = cs.fused()
+    assert np.array_equal(got_map, want_map)
+    assert np.array_equal(got_pool, want_pool)
+    assert np.array_equal(got_bits, want_bits)
+    lean_map, lean_pool, lean_bits = cs.fused(write_map=False)
+    assert np.array_equal(lean_pool, want_pool) and np.array_equal(lean_bits, want_bits)
+    assert np.isnan(lean_map.view(np.float32)).all()
+
+
+def test_geometries_the_pair_does_not_serve(dn):
+    leaky, logistic = ACTIVATIONS.index("leaky"), ACTIVATIONS.index("logistic")
+    assert dn.conv_maxpool_fusable(1, 3, 416, 416, 16, 1, 3, 1, 1, logistic) == 0     # activation outside the tail
+    assert dn.conv_maxpool_fusable(1, 3, 417, 416, 16, 1, 3, 1, 1, leaky) == 0        # odd height
+    assert dn.conv_maxpool_fusable(1, 3, 416, 400, 16, 1, 3, 1, 1, leaky) == 0        # width not a multiple of 32
+    assert dn.conv_maxpool_fusable(1, 3, 416, 416, 65, 1, 3, 1, 1, leaky) == 0        # more than 64 filters
+    assert dn.conv_maxpool_fusable(1, 4, 416, 416, 16, 1, 3, 1, 1, leaky) == 0        # not 3 channels
+    assert dn.conv_maxpool_fusable(1, 3, 416, 416, 16, 1, 3, 2, 1, leaky) == 0        # stride 2
+
+
+def test_tiny_network_fused_equals_layer_by_layer(dn):
+    """yolov3-tiny: first layer + maxpool in one pass (and in the xnor variant the sign bits for layer 2):
+    every layer holds the bits of the layer-by-layer run; lean mode leaves only layer 0's map out."""
+    for xnor in (False, True):
+        net = api.Network(cfg_text=cfgs.yolov3_tiny(2, 160, xnor=xnor))
+        fill_params(net.set_conv, net.layers)
+        x = synth.uniform01(7, net.inputs * 2)
+        try:
+            dn.network_set_fusion(0)
+            net.predict(x)
+            want = [net.layer_output(i) for i in range(net.n)]
+            dn.network_set_fusion(1)
+            net.predict(x)
+            for i in range(net.n):
+                assert np.array_equal(net.layer_output(i), want[i]), (xnor, i)
+            dn.network_set_fusion(2)
+            net.predict(x)
+            skipped = [0, 2, 4, 6] if xnor else [0]
+            for i in range(net.n):
+                if i not in skipped:
+                    assert np.array_equal(net.layer_output(i), want[i]), (xnor, i)
+        finally:
+            dn.network_set_fusion(1)
+        net.free()

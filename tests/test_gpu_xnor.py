@@ -215,9 +215,9 @@ def test_xnor_network_fused_equals_layer_by_layer(dn):
         dn.network_set_fusion(2)
         net.predict(x)
         skipped = [i for i, L in enumerate(net.layers)
-                   if L["type"] == "convolutional" and L["xnor"] and net.layers[i + 1]["type"] == "maxpool"
+                   if L["type"] == "convolutional" and net.layers[i + 1]["type"] == "maxpool"
                    and net.layers[i + 1]["stride"] == 2 and i != 8]         # layer 8 is also read by a route
-        assert skipped == [2, 4, 6]
+        assert skipped == [0, 2, 4, 6]                                      # the first layer pairs with its pool too
         for i in range(net.n):
             if i not in skipped:
                 assert np.array_equal(net.layer_output(i), want[i]), i
