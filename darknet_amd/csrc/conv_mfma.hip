@@ -71,7 +71,7 @@ extern "C" void conv_direct_forward(const float *, const float *, const float *,
 
 /* conv_first.hip: the kernel of 3-channel first layers */
 extern "C" int conv_first_serves(int batch, int c, int h, int w, int n, int groups, int size, int stride, int pad);
-extern "C" const char *conv_first_kernel_name(int n, int pooled);
+extern "C" const char *conv_first_kernel_name(int n, int pooled, int h, int w);
 extern "C" void conv_first_forward(const float *input, const float *weights, const float *biases, const float *scales,
                                    const float *rolling_mean, const float *rolling_variance, float *out, float *pool,
                                    unsigned *bits, int batch, int h, int w, int n, int batch_normalize, double slope,
@@ -1486,7 +1486,7 @@ extern "C" const char *conv_kernel_name_geometry(int batch, int c, int h, int w,
     if (g_algo != 1 && !(size == 3 && pad != 1) && conv_grouped_tile(n, c, groups, size)) mode = 10 + size;
     if (columns >= (1L << 31) - 512) mode = -1;
     if (g_algo == 0 && mode == 3 && conv_first_serves(batch, c, h, w, n, groups, size, stride, pad))
-        return conv_first_kernel_name(n, 0);
+        return conv_first_kernel_name(n, 0, h, w);
     const int patch = g_algo == 0 && mode == 3 && conv_patch_floats(c, h, w, n, groups, size, stride, pad) > 0;
     return kernel_name(n, c, groups, size, columns, patch, mode);
 }

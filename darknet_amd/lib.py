@@ -54,7 +54,7 @@ SIGNATURES = {
     "conv_packed_floats": (z, [i, i, i, i]), "conv_pack_weights_gpu": (None, [V, V, i, i, i, i]),
     "conv_packed_cached_gpu": (V, [V, i, i, i, i]), "conv_packed_forget": (None, [V]),
     "conv_packed_cached_count": (i, []),
-    "conv_set_algo": (None, [i]), "conv_set_ksplit": (None, [i, i]), "conv_set_bands": (None, [i]),
+    "conv_set_algo": (None, [i]), "conv_set_ksplit": (None, [i, i]), "conv_set_bands": (None, [i]), "conv_first_set_shape": (None, [i]),
     "xnor_weight_words": (z, [i, i, i]), "xnor_input_words": (z, [i, i, i, i]),
     "xnor_pack_weights_gpu": (None, [V, V, V, i, i, i]),
     "xnor_pack_input_gpu": (None, [V, V, i, i, i, i]),

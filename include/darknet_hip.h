@@ -252,7 +252,8 @@ void conv_set_algo(int algo);
 /* Tuning hooks of the K-split (no counterpart in the reference).  When a layer's last round of
  * tiles would leave most of the chip idle, those tiles are cut along K into slices that a second
  * launch sums in slice order.
- *   split   0 = the cost model decides, n > 0 = n slices for every such tile (1 = none)
+ *   split   0 = the cost model decides, n > 0 = n slices for every such tile (1 = none),
+ *           -n (n = 2..32) = n slices for EVERY tile of the layer, not only the last round's
  *   tile_n  0 = automatic, 64 or 128 = column width of the tile of layers with more than 64 filters
  *           (64 also gives layers of 33..64 filters the 64x64 tile), 1 = 64x64 tiles for every layer */
 void conv_set_ksplit(int split, int tile_n);
@@ -262,6 +263,12 @@ void conv_set_ksplit(int split, int tile_n);
  * XCD's consecutive share of the tiles then reads 1/bands of the weights and bands/8 of the input
  * through its private L2.  0 = automatic: the count that minimises weights*8/bands + input*bands. */
 void conv_set_bands(int bands);
+
+/* Tuning hook of the first-layer kernel (3 input channels, 3x3; no counterpart in the reference).
+ * Its 256-pixel tile is 2 rows x 128 columns, 4 x 64 or 8 x 32; waves_across = 4, 2 or 1 forces that
+ * shape where it divides the image (4 always applies, with a short last column of tiles), 0 = the
+ * widest one that divides it (default).  The outputs do not depend on the shape. */
+void conv_first_set_shape(int waves_across);
 
 /* Operand precision of the tap-blocked MFMA convolution kernels (channels a multiple of 16, 1x1 or
  * 3x3 pad 1; grouped 32-filter tiles):

@@ -95,6 +95,26 @@ def test_first_layer_with_pool_and_bits_in_one_pass(dn, b, h, w, n, act, bn):
     assert np.isnan(lean_map.view(np.float32)).all()
 
 
+@pytest.mark.parametrize("b,h,w,n", [(2, 8, 128, 32), (1, 16, 192, 17), (3, 8, 64, 64), (1, 24, 416, 33), (2, 16, 256, 5)])
+def test_every_tile_shape_gives_the_same_bits(dn, b, h, w, n):
+    """The tile is 2 x 128, 4 x 64 or 8 x 32 pixels by what divides the image; forced one after the other
+    on images that allow several, the map, the pooled map and the bits are the same."""
+    cs = First(dn, 23, b, h, w, n)
+    results, names = [], set()
+    try:
+        for shape in (4, 2, 1):
+            dn.conv_first_set_shape(shape)
+            names.add(dn.conv_kernel_name_geometry(b, 3, h, w, n, 1, 3, 1, 1).decode())
+            results.append((cs.conv().numpy().view(np.uint32),) + cs.fused() + cs.fused(write_map=False)[1:])
+    finally:
+        dn.conv_first_set_shape(0)
+    assert len(names) == (3 if w % 64 == 0 else 2), names
+    for other in results[1:]:
+        for got, want in zip(other, results[0]):
+            assert np.array_equal(got, want)
+    assert np.array_equal(results[0][0], results[0][1])
+
+
 def test_geometries_the_pair_does_not_serve(dn):
     leaky, logistic = ACTIVATIONS.index("leaky"), ACTIVATIONS.index("logistic")
     assert dn.conv_maxpool_fusable(1, 3, 416, 416, 16, 1, 3, 1, 1, logistic) == 0     # activation outside the tail
