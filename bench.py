@@ -506,6 +506,9 @@ def measure(L, api, synth, workload, batch, precision, steps, warmup, per_layer=
                          "bitop_twords_per_s": round(words_per_s / 1e12, 3), "bitop_frac": round(bit_frac, 4),
                          "bitop_peak_note": "32 words/clk/CU (64 lanes, 2 instructions per word) x 256 CUs x 2.4 GHz",
                          "bytes_per_launch": dom["bytes"] / dom["launches"],
+                         "kernel_family": "every instance of xnor_conv_kernel<ACT,SIZE,BITS> and "
+                                          "xnor_conv_pool_kernel<ACT> (the variant that also writes the 2x2 maxpool "
+                                          "and the next layer's sign bits), accounted as one kernel",
                          "equivalent_fp32_tflops": round(dom["flops"] / dom_ms / 1e9, 3)})
     else:
         achieved = dom["flops"] / dom_ms / 1e9  # TFLOP/s
