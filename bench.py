@@ -450,17 +450,10 @@ def measure(L, api, synth, workload, batch, precision, steps, warmup, per_layer=
             k["flops"] += fl
             k["bytes"] += row["bytes"]
             k["launches"] += 1
-        # a same-geometry shortcut right after a convolution runs inside that convolution's
-        # epilogue: its event interval is empty and its traffic belongs to the conv kernel
-        prev = net.layers[i - 1] if i else None
-        row["fused"] = bool(Ly["type"] == "shortcut" and prev and prev["type"] == "convolutional"
-                            and not prev["xnor"] and 0 <= Ly["index"] < i - 1
-                            and (Ly["w"], Ly["h"], Ly["c"]) == (Ly["out_w"], Ly["out_h"], Ly["out_c"])
-                            and (Ly["out_w"], Ly["out_h"], Ly["out_c"]) == (prev["out_w"], prev["out_h"], prev["out_c"]))
-        # likewise a yolo head right after the convolution that feeds it
-        row["fused"] = row["fused"] or bool(Ly["type"] == "yolo" and prev and prev["type"] == "convolutional"
-                                            and not prev["xnor"] and prev["n"] == Ly["n"] * (5 + Ly["classes"])
-                                            and (prev["out_w"], prev["out_h"]) == (Ly["w"], Ly["h"]))
+        # a same-geometry shortcut, a yolo head or a 2x2 stride-2 maxpool right after a convolution can
+        # run inside that convolution's kernel (the library says which do at the present fusion level):
+        # its event interval is empty and its traffic belongs to the conv kernel
+        row["fused"] = bool(L.network_layer_runs_fused(net.net, i))
         # a route of one source is a view of that source's buffer: no launch, no traffic
         view = Ly["type"] == "route" and len(Ly.get("input_layers", [])) == 1
         row["fused"] = row["fused"] or view
@@ -468,6 +461,7 @@ def measure(L, api, synth, workload, batch, precision, steps, warmup, per_layer=
         if row["fused"] and not view:
             # the conv kernel reads the shortcut's second operand and writes the fused layer's output
             # beside its own (both layer outputs stay observable, as in the reference)
+            # (a fused maxpool's input is the conv's own output: only its output is added)
             extra = 4 * Ly["batch"] * Ly["outputs"] * (2 if Ly["type"] == "shortcut" else 1)
             kernels[rows[i - 1]["kernel"]]["fused_bytes"] = kernels[rows[i - 1]["kernel"]].get("fused_bytes", 0.0) + extra
         rows.append(row)

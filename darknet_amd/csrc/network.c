@@ -190,16 +190,25 @@ static int forward_xnor(network net, int i)
 
 /* Runs layers i and i+1 together when they are a convolution and the residual add of a
  * darknet53 block (src/shortcut_layer.c:77-83 with equal geometries).  Returns 1 if it did. */
+static int conv_shortcut_pair(const network *net, int i)
+{
+    const layer *l, *s;
+    if (!g_fuse_shortcut || i < 0 || i + 1 >= net->n) return 0;
+    l = &net->layers[i];
+    s = &net->layers[i + 1];
+    if (l->type != CONVOLUTIONAL || l->xnor || s->type != SHORTCUT) return 0;
+    if (s->index < 0 || s->index >= i) return 0; /* the residual must come from an earlier layer */
+    if (s->w != s->out_w || s->h != s->out_h || s->c != s->out_c) return 0;
+    if (s->out_w != l->out_w || s->out_h != l->out_h || s->out_c != l->out_c || s->batch != l->batch) return 0;
+    return 1;
+}
+
 static int forward_conv_shortcut_pair(network net, int i)
 {
     layer l, s;
-    if (!g_fuse_shortcut || i + 1 >= net.n) return 0;
+    if (!conv_shortcut_pair(&net, i)) return 0;
     l = net.layers[i];
     s = net.layers[i + 1];
-    if (l.type != CONVOLUTIONAL || l.xnor || s.type != SHORTCUT) return 0;
-    if (s.index < 0 || s.index >= i) return 0; /* the residual must come from an earlier layer */
-    if (s.w != s.out_w || s.h != s.out_h || s.c != s.out_c) return 0;
-    if (s.out_w != l.out_w || s.out_h != l.out_h || s.out_c != l.out_c || s.batch != l.batch) return 0;
     forward_convolutional_shortcut_gpu(net.input_gpu, l.weights_gpu, l.weights_packed_gpu, l.biases_gpu,
                                        l.scales_gpu, l.rolling_mean_gpu, l.rolling_variance_gpu, l.output_gpu,
                                        l.batch, l.c, l.h, l.w, l.n, l.groups, l.size, l.stride, l.pad,
@@ -211,19 +220,44 @@ static int forward_conv_shortcut_pair(network net, int i)
 /* Runs layers i and i+1 together when they are a convolution and the yolo head it feeds
  * (src/yolo_layer.c:347-361): the head's copy + logistic rides in the convolution's epilogue.
  * Returns 1 if it did. */
+static int conv_yolo_pair(const network *net, int i)
+{
+    const layer *l, *y;
+    if (!g_fuse_shortcut || i < 0 || i + 1 >= net->n) return 0;
+    l = &net->layers[i];
+    y = &net->layers[i + 1];
+    if (l->type != CONVOLUTIONAL || l->xnor || y->type != YOLO) return 0;
+    if (y->w != l->out_w || y->h != l->out_h || y->batch != l->batch || y->n * (5 + y->classes) != l->n) return 0;
+    return 1;
+}
+
 static int forward_conv_yolo_pair(network net, int i)
 {
     layer l, y;
-    if (!g_fuse_shortcut || i + 1 >= net.n) return 0;
+    if (!conv_yolo_pair(&net, i)) return 0;
     l = net.layers[i];
     y = net.layers[i + 1];
-    if (l.type != CONVOLUTIONAL || l.xnor || y.type != YOLO) return 0;
-    if (y.w != l.out_w || y.h != l.out_h || y.batch != l.batch || y.n * (5 + y.classes) != l.n) return 0;
     forward_convolutional_yolo_gpu(net.input_gpu, l.weights_gpu, l.weights_packed_gpu, l.biases_gpu, l.scales_gpu,
                                    l.rolling_mean_gpu, l.rolling_variance_gpu, l.output_gpu, l.batch, l.c, l.h,
                                    l.w, l.n, l.groups, l.size, l.stride, l.pad, l.batch_normalize,
                                    (int)l.activation, y.output_gpu, y.n, y.classes);
     return 1;
+}
+
+/* Whether layer i runs inside the kernel of the convolution in front of it at the present fusion
+ * level (a residual add, a yolo head, a 2x2 stride-2 maxpool), so that no launch is its own; and
+ * whether, in lean mode, layer i's own output is left unwritten. */
+int network_layer_runs_fused(network *net, int i)
+{
+    if (i < 1 || i >= net->n) return 0;
+    return conv_shortcut_pair(net, i - 1) || conv_yolo_pair(net, i - 1) || xnor_pool_pair(net, i - 1) ||
+           conv_pool_pair(net, i - 1);
+}
+
+int network_layer_output_skipped(network *net, int i)
+{
+    if (i < 0 || i >= net->n) return 0;
+    return xnor_map_skipped(net, i);
 }
 
 /* The layer loop of src/network.c:773-785 without the copies around it.  `gate` (may be NULL) is

@@ -98,6 +98,7 @@ SIGNATURES = {
     "pull_network_output": (None, [V]), "network_width": (i, [V]), "network_height": (i, [V]),
     "forward_network_device": (None, [V]), "forward_network_profiled": (f, [V, F]),
     "network_set_fusion": (None, [i]),
+    "network_layer_runs_fused": (i, [V, i]), "network_layer_output_skipped": (i, [V, i]),
     "network_predict_submit": (None, [V, F]), "network_predict_collect": (F, [V]),
     "network_collected_output": (F, [V, i]), "network_predict_in_flight": (i, [V]),
     "forward_network_profiled_kernels": (f, [V, F, F]),

@@ -351,6 +351,10 @@ float forward_network_profiled_kernels(network *net, float *layer_ms, float *ker
  * 2 (lean): as 1, except that the map of a convolution which nothing but the maxpool fused behind
  * it reads is not written: its output buffer is stale, layer_output_host() refuses it. */
 void network_set_fusion(int on);
+/* At the present fusion level: whether layer i runs inside the kernel of the convolution in front
+ * of it (no launch of its own), and whether layer i's own output is left unwritten (lean mode). */
+int network_layer_runs_fused(network *net, int i);
+int network_layer_output_skipped(network *net, int i);
 float *layer_output_host(network *net, int i);
 int *layer_indexes_host(network *net, int i);
 void network_set_verbose(int on);

@@ -134,15 +134,23 @@ def test_tiny_network_fused_equals_layer_by_layer(dn):
         x = synth.uniform01(7, net.inputs * 2)
         try:
             dn.network_set_fusion(0)
+            assert not any(dn.network_layer_runs_fused(net.net, i) for i in range(net.n))
             net.predict(x)
             want = [net.layer_output(i) for i in range(net.n)]
             dn.network_set_fusion(1)
+            # what runs inside the convolution in front of it: the 2x2/2 maxpools behind the first layer and,
+            # in the xnor network, behind the xnor convolutions (not the stride-1 pool 11), and the yolo heads
+            # behind fp32 convolutions (in the xnor network only the last convolution is one)
+            assert [i for i in range(net.n) if dn.network_layer_runs_fused(net.net, i)] == \
+                ([1, 3, 5, 7, 9, 23] if xnor else [1, 16, 23])
+            assert not any(dn.network_layer_output_skipped(net.net, i) for i in range(net.n))
             net.predict(x)
             for i in range(net.n):
                 assert np.array_equal(net.layer_output(i), want[i]), (xnor, i)
             dn.network_set_fusion(2)
             net.predict(x)
             skipped = [0, 2, 4, 6] if xnor else [0]
+            assert [i for i in range(net.n) if dn.network_layer_output_skipped(net.net, i)] == skipped
             for i in range(net.n):
                 if i not in skipped:
                     assert np.array_equal(net.layer_output(i), want[i]), (xnor, i)
