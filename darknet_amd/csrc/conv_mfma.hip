@@ -884,6 +884,10 @@ __global__ __launch_bounds__(DN_THREADS, ((BM == 128 && BF16 != 3) ? 3 : 2)) voi
         __builtin_amdgcn_s_waitcnt(0);
         __syncthreads();
     };
+    /* The last chunk requests nothing.  Invariant of every way out of the chunk loop: no wave leaves it
+     * with a direct-to-LDS load in flight (vmcnt = 0) - every step above ends with s_waitcnt(0) in
+     * front of its barrier, and `last` issues no load - so neither the epilogue's reuse of the LDS
+     * buffers nor the end of a K-slice workgroup (which gives its LDS back) can meet a pending write. */
     auto last = [&](int buf) {
         read_operands(buf, 0);
         mfma_chunk(0);
@@ -967,6 +971,7 @@ __global__ __launch_bounds__(DN_THREADS, ((BM == 128 && BF16 != 3) ? 3 : 2)) voi
 
     }
 
+    /* here vmcnt = 0 on every path (see `last` and `fstep`) */
     if (slice_id >= 0) {
         /* K-slice: park the raw accumulators, lane-major so every store is a full 256-byte row */
         float *ws = a.partial + (long)slice_id * (BM * BN);
