@@ -574,7 +574,13 @@ __global__ __launch_bounds__(DN_THREADS, ((BM == 128 && BF16 != 3) ? 3 : 2)) voi
 
     typedef __attribute__((address_space(3))) void *lds_ptr;
 
-    auto load_chunk = [&](int kc, int buf) {
+    /* `live` = false: the request is only there to keep a schedule region free of branches (the last
+     * step of a loop form that always requests "the next chunk").  Its weights are chunk kc's again
+     * (in range by construction); its input lanes all carry the out-of-range offset, so they write
+     * zeros to LDS and read no memory: the tap-blocked input address is built from a scalar offset the
+     * buffer's range check does not cover, and one chunk past the last would reach up to 16 channel
+     * planes beyond the end of the tensor for the last image of the batch. */
+    auto load_chunk = [&](int kc, int buf, bool live = true) {
         /* A */
         if constexpr (BF16) {
             /* bf16 copy: [chunk][k half][Mpad16 rows][8 bf16]; LDS image [k half][BM][16 bytes].
@@ -637,9 +643,10 @@ __global__ __launch_bounds__(DN_THREADS, ((BM == 128 && BF16 != 3) ? 3 : 2)) voi
             const int ky = (ld_tap * 11) >> 5, kx = ld_tap - 3 * ((ld_tap * 11) >> 5); /* tap/3, tap%3 */
             const int shift = (ky - 1) * a.W + (kx - 1);
             const unsigned soff0 = (unsigned)(((long)2 * ld_cb * HW + shift + bias) * 16); /* wave-uniform */
+            const int tap_bit = live ? ld_tap : 31; /* bit 31 of a tap mask is never set */
 #pragma unroll
             for (int g = 0; g < NBW; ++g) {
-                const unsigned voff = ((c_mask[g] >> ld_tap) & 1u) ? c_voff[g] : 0xFFFFFFF0u;
+                const unsigned voff = ((c_mask[g] >> tap_bit) & 1u) ? c_voff[g] : 0xFFFFFFF0u;
                 __builtin_amdgcn_raw_ptr_buffer_load_lds(in_rsrc, (lds_ptr)&B_BUF(buf)[(lkh * BN + (lblk0 + g) * 64) * 4], 16,
                                                          voff, soff0, 0, 0);
             }
@@ -651,9 +658,10 @@ __global__ __launch_bounds__(DN_THREADS, ((BM == 128 && BF16 != 3) ? 3 : 2)) voi
             const int ky = (ld_tap * 11) >> 5, kx = ld_tap - 3 * ((ld_tap * 11) >> 5); /* tap/3, tap%3 */
             const int shift = KS == 1 ? 0 : (ky - 1) * a.W + (kx - 1);       /* pad == 1 for 3x3 */
             const unsigned soff0 = (unsigned)((ld_cb * 16 * HW + shift + bias) * 4); /* wave-uniform */
+            const int tap_bit = live ? ld_tap : 31; /* bit 31 of a tap mask is never set */
 #pragma unroll
             for (int g = 0; g < NG_PER_WAVE; ++g) {
-                const unsigned voff = ((vmask[g] >> ld_tap) & 1u) ? voff_px[g] : 0xFFFFFFFCu;
+                const unsigned voff = ((vmask[g] >> tap_bit) & 1u) ? voff_px[g] : 0xFFFFFFFCu;
                 const int ng = wave * NG_PER_WAVE + g;
 #pragma unroll
                 for (int q = 0; q < 4; ++q)
@@ -682,7 +690,7 @@ __global__ __launch_bounds__(DN_THREADS, ((BM == 128 && BF16 != 3) ? 3 : 2)) voi
 #pragma unroll
                 for (int q = 0; q < 4; ++q) {
                     const int ky = kyx[q] >> 16, kx = kyx[q] & 0xffff;
-                    const bool ok = ((unsigned)(iy0[g] + ky) < (unsigned)a.H) & ((unsigned)(ix0[g] + kx) < (unsigned)a.W);
+                    const bool ok = live & ((unsigned)(iy0[g] + ky) < (unsigned)a.H) & ((unsigned)(ix0[g] + kx) < (unsigned)a.W);
                     const unsigned voff = ok ? voff_px[g] + (unsigned)koff[q] : 0xFFFFFFFCu;
                     __builtin_amdgcn_raw_ptr_buffer_load_lds(in_rsrc, (lds_ptr)&B_BUF(buf)[(q * BN + ng * 16) * 4], 4,
                                                              voff, 0, 0, 0);
@@ -938,7 +946,7 @@ __global__ __launch_bounds__(DN_THREADS, ((BM == 128 && BF16 != 3) ? 3 : 2)) voi
             __builtin_amdgcn_sched_barrier(0);
             /* the next chunk's loads go between this chunk's MFMAs (the last step requests its own
              * chunk again: no branch inside the schedule region) */
-            load_chunk(rem >= 1 ? kcur + 1 : kcur, buf ^ 1);
+            load_chunk(rem >= 1 ? kcur + 1 : kcur, buf ^ 1, rem >= 1);
             mfma_chunk(0);
 #pragma unroll
             for (int g = 0; g < LPC_F; ++g) {

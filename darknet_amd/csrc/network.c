@@ -60,6 +60,8 @@ void set_batch_network(network *net, int b)
 {
     int i;
     if (b < 1) dn_fatal("set_batch_network: batch must be at least 1");
+    if (network_predict_in_flight(net))
+        dn_fatal("set_batch_network: batches submitted with network_predict_submit are in flight; collect them first");
     if (net->max_batch < net->batch) net->max_batch = net->batch; /* a network built without the parser */
     if (b > net->max_batch)
         dn_fatal("set_batch_network: buffers were allocated for a smaller batch (the cfg's batch is the limit)");
@@ -395,6 +397,10 @@ void forward_network_gpu(network *netp)
     DN_NEED_DEVICE("forward_network_gpu");
     network net = *netp;
     int i;
+    /* a batch submitted with network_predict_submit is still being computed or copied out of the very
+     * buffers this pass would write */
+    if (network_predict_in_flight(netp))
+        dn_fatal("forward_network_gpu: batches submitted with network_predict_submit are in flight; collect them first");
     hip_set_device(net.gpu_index);
     hip_push_array(net.input_gpu, net.input, (size_t)net.inputs * net.batch);
     forward_network_device(netp);

@@ -498,3 +498,27 @@ def test_pipelined_predict_on_a_classifier_and_at_a_smaller_batch(dn):
     net.submit(xs[0][:net.inputs * 2])
     assert np.array_equal(net.collect(), small)
     net.free()
+
+
+@pytest.mark.parametrize("misuse,message", [
+    ("net.submit(x); net.submit(x); net.submit(x)", "two batches are in flight already"),
+    ("net.collect()", "no batch is in flight"),
+    ("net.submit(x); net.predict(x)", "collect them first"),
+    ("net.submit(x); net.set_batch(1)", "collect them first"),
+])
+def test_pipelined_predict_misuse_ends_with_a_message(misuse, message):
+    """A third submit, a collect with nothing in flight, and the synchronous calls that would write the
+    buffers a batch in flight is still being copied out of end the process with a message, as every
+    argument the library cannot honour does (a process of its own: the library exits)."""
+    import os
+    import subprocess
+    import sys
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    code = ("from darknet_amd import api, cfgs, synth\napi.set_gpu(0)\n"
+            "net = api.Network(cfg_text=cfgs.yolov3_tiny(2, 96))\n"
+            "x = synth.uniform01(1, net.inputs * 2)\nnet.predict(x)\nprint('ready', flush=True)\n"
+            + "\n".join(part.strip() for part in misuse.split(";")) + "\nprint('survived', flush=True)\n")
+    r = subprocess.run([sys.executable, "-c", code], cwd=root, capture_output=True, text=True, timeout=100)
+    assert "ready" in r.stdout and "survived" not in r.stdout and r.returncode != 0, (r.stdout, r.stderr[-400:])
+    assert message in r.stderr, r.stderr[-400:]
+
