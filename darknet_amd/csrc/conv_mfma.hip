@@ -71,11 +71,11 @@ extern "C" void conv_direct_forward(const float *, const float *, const float *,
 
 /* conv_first.hip: the kernel of 3-channel first layers */
 extern "C" int conv_first_serves(int batch, int c, int h, int w, int n, int groups, int size, int stride, int pad);
-extern "C" const char *conv_first_kernel_name(int n, int pooled, int h, int w);
+extern "C" const char *conv_first_kernel_name(int c, int n, int pooled, int h, int w);
 extern "C" void conv_first_forward(const float *input, const float *weights, const float *biases, const float *scales,
                                    const float *rolling_mean, const float *rolling_variance, float *out, float *pool,
-                                   unsigned *bits, int batch, int h, int w, int n, int batch_normalize, double slope,
-                                   int cus, void *start, void *stop);
+                                   unsigned *bits, int batch, int c, int h, int w, int n, int batch_normalize,
+                                   double slope, int cus, void *start, void *stop);
 
 struct mfma_args {
     const float *in;
@@ -1430,6 +1430,16 @@ extern "C" void conv_set_algo(int algo) { g_algo = algo; }
  * and sum six piece-products in fp32 (fp32-level accuracy on the bf16 matrix cores).  Layers on
  * other kernels stay fp32. */
 static int g_precision = 0;
+
+/* Whether a layer of conv_mode `mode` goes to the first-layer kernel when its geometry fits: the
+ * 3-channel layers of the reference-order mode, and 16-channel 3x3 layers of the tap-blocked mode
+ * while the operands are fp32 (the bf16 modes keep such a layer on their own pipeline). */
+static int conv_first_takes(int mode, int c)
+{
+    if (g_algo != 0) return 0;
+    return (mode == 3 && c == 3) || (mode == 13 && c == 16 && g_precision == 0);
+}
+
 extern "C" void conv_set_precision(int precision)
 {
     if (precision < 0 || precision > 2)
@@ -1498,8 +1508,8 @@ extern "C" const char *conv_kernel_name_geometry(int batch, int c, int h, int w,
     int mode = conv_mode(c, groups, size, stride, pad, (long)batch * in_img);
     if (g_algo != 1 && !(size == 3 && pad != 1) && conv_grouped_tile(n, c, groups, size)) mode = 10 + size;
     if (columns >= (1L << 31) - 512) mode = -1;
-    if (g_algo == 0 && mode == 3 && conv_first_serves(batch, c, h, w, n, groups, size, stride, pad))
-        return conv_first_kernel_name(n, 0, h, w);
+    if (conv_first_takes(mode, c) && conv_first_serves(batch, c, h, w, n, groups, size, stride, pad))
+        return conv_first_kernel_name(c, n, 0, h, w);
     const int patch = g_algo == 0 && mode == 3 && conv_patch_floats(c, h, w, n, groups, size, stride, pad) > 0;
     return kernel_name(n, c, groups, size, columns, patch, mode);
 }
@@ -1882,11 +1892,12 @@ static void conv_forward(const float *input, const float *weights, const float *
         return;
     }
 
-    /* first layers (3 channels, 3x3 / 1 / pad 1, even height, width a multiple of 32): their own kernel */
-    if (g_algo == 0 && mode == 3 && !sum && conv_first_serves(batch, c, h, w, n, groups, size, stride, pad)) {
+    /* first layers (3 channels, or 16 behind a pooled first layer; 3x3 / 1 / pad 1, even height, width a
+     * multiple of 32): their own kernel */
+    if (conv_first_takes(mode, c) && !sum && conv_first_serves(batch, c, h, w, n, groups, size, stride, pad)) {
         const int dev = hip_get_device();
         if (dev >= 0 && dev < DN_MAX_DEVICES && !g_cus_dev[dev]) conv_device_setup();
-        conv_first_forward(input, weights, biases, scales, rolling_mean, rolling_variance, output, 0, 0, batch, h, w, n,
+        conv_first_forward(input, weights, biases, scales, rolling_mean, rolling_variance, output, 0, 0, batch, c, h, w, n,
                            batch_normalize, slope, dev >= 0 && dev < DN_MAX_DEVICES ? g_cus_dev[dev] : 0,
                            (void *)g_prof_start, (void *)g_prof_stop);
         g_prof_start = g_prof_stop = 0;
@@ -2079,7 +2090,8 @@ extern "C" int conv_maxpool_fusable(int batch, int c, int h, int w, int n, int g
                                     int activation)
 {
     double slope;
-    if (g_algo != 0 || !conv_inline_activation(activation, &slope)) return 0;
+    if (!conv_inline_activation(activation, &slope)) return 0;
+    if (!conv_first_takes(c == 3 ? 3 : 13, c)) return 0;
     return conv_first_serves(batch, c, h, w, n, groups, size, stride, pad);
 }
 
@@ -2095,14 +2107,14 @@ extern "C" void forward_convolutional_maxpool_gpu(const float *input, const floa
     if (!input || !weights || !biases || !pool_output) dn_fatal("forward_convolutional_maxpool_gpu: null pointer");
     if (batch_normalize && (!scales || !rolling_mean || !rolling_variance))
         dn_fatal("forward_convolutional_maxpool_gpu: batch_normalize needs scales, rolling_mean, rolling_variance");
-    if (!conv_inline_activation(activation, &slope) ||
-        !conv_first_serves(batch, c, h, w, n, groups, size, stride, pad))
-        dn_fatal("forward_convolutional_maxpool_gpu: serves 3-channel 3x3 / 1 / pad 1 layers of up to 64 filters with a "
-                 "leaky, linear or relu activation, even height and a width that is a multiple of 32 "
-                 "(conv_maxpool_fusable)");
+    if (!conv_maxpool_fusable(batch, c, h, w, n, groups, size, stride, pad, activation))
+        dn_fatal("forward_convolutional_maxpool_gpu: serves 3x3 / 1 / pad 1 layers of 3 channels (up to 64 filters) or 16 "
+                 "channels (up to 32) with a leaky, linear or relu activation, even height and a width that is a multiple "
+                 "of 32, in the default fp32 mode (conv_maxpool_fusable)");
+    conv_inline_activation(activation, &slope);
     const int dev = hip_get_device();
     if (dev < 0 || dev >= DN_MAX_DEVICES) dn_fatal("forward_convolutional_maxpool_gpu: device index out of range");
     if (!g_cus_dev[dev]) conv_device_setup();
     conv_first_forward(input, weights, biases, scales, rolling_mean, rolling_variance, output, pool_output, next_xbits,
-                       batch, h, w, n, batch_normalize, slope, g_cus_dev[dev], 0, 0);
+                       batch, c, h, w, n, batch_normalize, slope, g_cus_dev[dev], 0, 0);
 }

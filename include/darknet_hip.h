@@ -264,10 +264,11 @@ void conv_set_ksplit(int split, int tile_n);
  * through its private L2.  0 = automatic: the count that minimises weights*8/bands + input*bands. */
 void conv_set_bands(int bands);
 
-/* Tuning hook of the first-layer kernel (3 input channels, 3x3; no counterpart in the reference).
+/* Tuning hook of the first-layer kernel (3 or 16 input channels, 3x3; no counterpart in the reference).
  * Its 256-pixel tile is 2 rows x 128 columns, 4 x 64 or 8 x 32; waves_across = 4, 2 or 1 forces that
- * shape where it divides the image (4 always applies, with a short last column of tiles), 0 = the
- * widest one that divides it (default).  The outputs do not depend on the shape. */
+ * shape where its height divides the image's (the 2-row shape always applies), 0 = the shape that
+ * wastes the fewest columns in the last tile of a row (default).  The outputs do not depend on the
+ * shape. */
 void conv_first_set_shape(int waves_across);
 
 /* Operand precision of the tap-blocked MFMA convolution kernels (channels a multiple of 16, 1x1 or
@@ -312,9 +313,12 @@ void forward_convolutional_xnor_packed_gpu(const float *input, const unsigned *w
                                            int stride, int pad, int batch_normalize, int activation);
 
 /* A first layer and the 2x2 stride-2 maxpool layer behind it in one pass (no counterpart in the
- * reference): forward_convolutional_gpu (src/convolutional_kernels.cu:73-135) for a 3-channel 3x3 /
- * stride 1 / pad 1 convolution of up to 64 filters, plus forward_maxpool_layer_gpu
- * (src/maxpool_layer_kernels.cu:87-99; size 2, stride 2, padding 0 or 1) on its output.
+ * reference): forward_convolutional_gpu (src/convolutional_kernels.cu:73-135) for a 3x3 / stride 1 /
+ * pad 1 convolution of 3 channels into up to 64 filters, or of 16 channels into up to 32 (the second
+ * convolution of the tiny networks), over an image of even height and a width that is a multiple of
+ * 8, plus forward_maxpool_layer_gpu (src/maxpool_layer_kernels.cu:87-99; size 2, stride 2, padding 0
+ * or 1) on its output.  forward_convolutional_gpu runs such a layer on the same kernel without the
+ * pooled outputs, so the map is the same bits either way.
  *   output       the convolution's map [batch][n][h][w], or NULL: then only the pooled map is written
  *   pool_output  [batch][n][h/2][w/2]
  *   next_xbits   NULL, or where to write the sign bits (x > 0) of pool_output for an xnor convolution

@@ -1,4 +1,5 @@
-"""The first-layer kernel (3 channels, 3x3, stride 1, pad 1) through the C-ABI: against the CPU
+"""The first-layer kernel (3x3, stride 1, pad 1 over 3 channels, or over the 16 channels behind a pooled
+first layer) through the C-ABI: against the CPU
 checker and the fp64 convolution as every convolution is, and its pooled forms against the separate
 calls they stand for - forward_convolutional_gpu, forward_maxpool_gpu, xnor_pack_input_gpu - bit
 for bit.  Widths of one to several 128-column tiles with and without a ragged last tile, two-row
@@ -16,10 +17,10 @@ D = api.DeviceArray
 
 
 class First:
-    def __init__(self, dn, seed, b, h, w, n, act="leaky", bn=1):
-        self.dn, self.geom, self.act, self.bn = dn, (b, h, w, n), act, bn
-        self.x = synth.uniform(seed, b * 3 * h * w).reshape(b, 3, h, w)
-        self.wt = synth.conv_weights(seed + 1, n, 3, 3)
+    def __init__(self, dn, seed, b, h, w, n, act="leaky", bn=1, c=3):
+        self.dn, self.geom, self.act, self.bn, self.c = dn, (b, h, w, n), act, bn, c
+        self.x = synth.uniform(seed, b * c * h * w).reshape(b, c, h, w)
+        self.wt = synth.conv_weights(seed + 1, n, c, 3)
         self.bias, self.sc, self.mu, self.var = synth.bn_random(seed + 2, n)
         self.sc = self.sc.copy()
         self.sc[1::3] *= -1.0
@@ -27,7 +28,7 @@ class First:
 
     def tail(self):
         b, h, w, n = self.geom
-        return [b, 3, h, w, n, 1, 3, 1, 1, self.bn, ACTIVATIONS.index(self.act)]
+        return [b, self.c, h, w, n, 1, 3, 1, 1, self.bn, ACTIVATIONS.index(self.act)]
 
     def conv(self):
         b, h, w, n = self.geom
@@ -58,7 +59,10 @@ class First:
 
 
 GEOMS = [(1, 2, 32, 16), (2, 6, 64, 32), (3, 10, 160, 17), (1, 16, 416, 32), (2, 8, 128, 64), (5, 4, 96, 33),
-         (1, 34, 256, 1), (2, 12, 288, 48)]
+         (1, 34, 256, 1), (2, 12, 288, 48), (2, 8, 104, 24), (1, 4, 40, 64), (3, 6, 200, 9)]
+# 16 channels, up to 32 filters: the second convolution of the tiny networks (16 -> 32 at 208 x 208)
+GEOMS16 = [(1, 2, 32, 32), (2, 8, 64, 32), (1, 16, 208, 32), (3, 12, 128, 17), (2, 24, 96, 1), (1, 6, 160, 31),
+           (2, 8, 56, 32), (1, 4, 104, 20)]
 
 
 @pytest.mark.parametrize("b,h,w,n", GEOMS)
@@ -95,20 +99,21 @@ def test_first_layer_with_pool_and_bits_in_one_pass(dn, b, h, w, n, act, bn):
     assert np.isnan(lean_map.view(np.float32)).all()
 
 
-@pytest.mark.parametrize("b,h,w,n", [(2, 8, 128, 32), (1, 16, 192, 17), (3, 8, 64, 64), (1, 24, 416, 33), (2, 16, 256, 5)])
-def test_every_tile_shape_gives_the_same_bits(dn, b, h, w, n):
+@pytest.mark.parametrize("c,b,h,w,n", [(3, 2, 8, 128, 32), (3, 1, 16, 192, 17), (3, 3, 8, 64, 64), (3, 1, 24, 416, 33),
+                                       (3, 2, 16, 256, 5), (16, 2, 8, 128, 32), (16, 1, 16, 192, 17), (16, 1, 24, 416, 9)])
+def test_every_tile_shape_gives_the_same_bits(dn, c, b, h, w, n):
     """The tile is 2 x 128, 4 x 64 or 8 x 32 pixels by what divides the image; forced one after the other
     on images that allow several, the map, the pooled map and the bits are the same."""
-    cs = First(dn, 23, b, h, w, n)
+    cs = First(dn, 23, b, h, w, n, c=c)
     results, names = [], set()
     try:
         for shape in (4, 2, 1):
             dn.conv_first_set_shape(shape)
-            names.add(dn.conv_kernel_name_geometry(b, 3, h, w, n, 1, 3, 1, 1).decode())
+            names.add(dn.conv_kernel_name_geometry(b, c, h, w, n, 1, 3, 1, 1).decode())
             results.append((cs.conv().numpy().view(np.uint32),) + cs.fused() + cs.fused(write_map=False)[1:])
     finally:
         dn.conv_first_set_shape(0)
-    assert len(names) == (3 if w % 64 == 0 else 2), names
+    assert len(names) == 3, names                      # all three heights divide these images
     for other in results[1:]:
         for got, want in zip(other, results[0]):
             assert np.array_equal(got, want)
@@ -119,7 +124,7 @@ def test_geometries_the_pair_does_not_serve(dn):
     leaky, logistic = ACTIVATIONS.index("leaky"), ACTIVATIONS.index("logistic")
     assert dn.conv_maxpool_fusable(1, 3, 416, 416, 16, 1, 3, 1, 1, logistic) == 0     # activation outside the tail
     assert dn.conv_maxpool_fusable(1, 3, 417, 416, 16, 1, 3, 1, 1, leaky) == 0        # odd height
-    assert dn.conv_maxpool_fusable(1, 3, 416, 400, 16, 1, 3, 1, 1, leaky) == 0        # width not a multiple of 32
+    assert dn.conv_maxpool_fusable(1, 3, 416, 404, 16, 1, 3, 1, 1, leaky) == 0        # width not a multiple of 8
     assert dn.conv_maxpool_fusable(1, 3, 416, 416, 65, 1, 3, 1, 1, leaky) == 0        # more than 64 filters
     assert dn.conv_maxpool_fusable(1, 4, 416, 416, 16, 1, 3, 1, 1, leaky) == 0        # not 3 channels
     assert dn.conv_maxpool_fusable(1, 3, 416, 416, 16, 1, 3, 2, 1, leaky) == 0        # stride 2
@@ -138,18 +143,19 @@ def test_tiny_network_fused_equals_layer_by_layer(dn):
             net.predict(x)
             want = [net.layer_output(i) for i in range(net.n)]
             dn.network_set_fusion(1)
-            # what runs inside the convolution in front of it: the 2x2/2 maxpools behind the first layer and,
-            # in the xnor network, behind the xnor convolutions (not the stride-1 pool 11), and the yolo heads
+            # what runs inside the convolution in front of it: the 2x2/2 maxpools behind the first layer, behind
+            # the 16-channel second layer when it is an fp32 convolution and, in the xnor network, behind the
+            # xnor convolutions (not the stride-1 pool 11), and the yolo heads
             # behind fp32 convolutions (in the xnor network only the last convolution is one)
             assert [i for i in range(net.n) if dn.network_layer_runs_fused(net.net, i)] == \
-                ([1, 3, 5, 7, 9, 23] if xnor else [1, 16, 23])
+                ([1, 3, 5, 7, 9, 23] if xnor else [1, 3, 16, 23])
             assert not any(dn.network_layer_output_skipped(net.net, i) for i in range(net.n))
             net.predict(x)
             for i in range(net.n):
                 assert np.array_equal(net.layer_output(i), want[i]), (xnor, i)
             dn.network_set_fusion(2)
             net.predict(x)
-            skipped = [0, 2, 4, 6] if xnor else [0]
+            skipped = [0, 2, 4, 6] if xnor else [0, 2]
             assert [i for i in range(net.n) if dn.network_layer_output_skipped(net.net, i)] == skipped
             for i in range(net.n):
                 if i not in skipped:
@@ -157,3 +163,45 @@ def test_tiny_network_fused_equals_layer_by_layer(dn):
         finally:
             dn.network_set_fusion(1)
         net.free()
+
+
+@pytest.mark.parametrize("b,h,w,n", GEOMS16)
+def test_sixteen_channel_layer_against_the_checker(dn, orc, b, h, w, n):
+    leaky = ACTIVATIONS.index("leaky")
+    assert dn.conv_maxpool_fusable(b, 16, h, w, n, 1, 3, 1, 1, leaky) == 1
+    assert dn.conv_maxpool_fusable(b, 16, h, w, 33, 1, 3, 1, 1, leaky) == 0     # a lane's registers hold 32 filters' weights
+    name = dn.conv_kernel_name_geometry(b, 16, h, w, n, 1, 3, 1, 1).decode()
+    assert name.startswith("conv_first_kernel") and name.endswith(",16>"), name
+    cs = First(dn, 5, b, h, w, n, c=16)
+    got = cs.conv().numpy((b, n, h, w))
+    want = orc.conv(cs.x, cs.wt, cs.bias, cs.sc, cs.mu, cs.var, n=n, size=3, stride=1, pad=1, groups=1,
+                    batch_normalize=1, activation="leaky")
+    assert not np.isnan(got).any()
+    assert norm_err(got, want) <= REL_TOL
+    # exact on small integers: every product and partial sum is representable, so the order of the k pairs
+    # (tap by tap over channels ch and ch + 8) cannot show
+    xi = np.round(cs.x * 4).astype(np.float32)
+    wi = np.round(cs.wt * 8).astype(np.float32)
+    ones, zeros = np.ones(n, np.float32), np.zeros(n, np.float32)
+    d = [D(a) for a in (xi, wi, zeros)]
+    out = D(np.full(b * n * h * w, np.nan, np.float32))
+    dn.forward_convolutional_gpu(d[0].ptr, d[1].ptr, None, d[2].ptr, None, None, None, out.ptr, b, 16, h, w, n, 1, 3, 1, 1,
+                                 0, ACTIVATIONS.index("linear"))
+    exact = orc.conv(xi.reshape(b, 16, h, w), wi, zeros, ones, zeros, ones, n=n, size=3, stride=1, pad=1, groups=1,
+                     batch_normalize=0, activation="linear")
+    assert np.array_equal(out.numpy((b, n, h, w)), exact)
+
+
+@pytest.mark.parametrize("b,h,w,n", GEOMS16)
+@pytest.mark.parametrize("act,bn", [("leaky", 1), ("linear", 0)])
+def test_sixteen_channel_layer_with_pool_and_bits_in_one_pass(dn, b, h, w, n, act, bn):
+    cs = First(dn, 13, b, h, w, n, act=act, bn=bn, c=16)
+    want_map, want_pool, want_bits = cs.separate()
+    got_map, got_pool, got_bits = cs.fused()
+    assert np.array_equal(got_map, want_map)
+    assert np.array_equal(got_pool, want_pool)
+    assert np.array_equal(got_bits, want_bits)
+    lean_map, lean_pool, lean_bits = cs.fused(write_map=False)
+    assert np.array_equal(lean_pool, want_pool) and np.array_equal(lean_bits, want_bits)
+    assert np.isnan(lean_map.view(np.float32)).all()
+
