@@ -81,7 +81,11 @@ def test_route_bit_exact(dn, orc, sizes, batch):
     ((2, 256, 14, 14), (2, 64, 14, 14), 1.0, 1.0, "leaky"),      # resnext: fewer channels in `add`
     ((2, 32, 7, 7), (2, 16, 14, 14), 1.0, 1.0, "leaky"),         # resnext: `add` twice as large
     ((1, 8, 6, 6), (1, 8, 3, 3), 0.5, 2.0, "logistic"),          # `add` smaller, general scales
-    ((1, 3, 5, 5), (1, 3, 5, 5), 1.0, 1.0, "relu")])             # odd size -> scalar path
+    ((1, 3, 5, 5), (1, 3, 5, 5), 1.0, 1.0, "relu"),              # odd size -> scalar path
+    ((2, 16, 8, 8), (2, 64, 8, 8), 1.0, 1.0, "linear"),          # more channels in `add` than in the output
+    ((1, 8, 7, 7), (1, 4, 7, 7), 1.0, 1.0, "leaky"),             # odd plane, fewer channels in `add`
+    ((3, 20, 6, 10), (3, 12, 12, 20), 1.0, 0.5, "leaky"),        # `add` twice as large, not square
+    ((2, 6, 12, 20), (2, 10, 6, 10), 1.0, 1.0, "linear")])       # `add` half as large, not square
 def test_shortcut_bit_exact(dn, orc, shape_in, shape_add, alpha, beta, act):
     x = synth.uniform(1, int(np.prod(shape_in)), -2, 2).reshape(shape_in)
     add = synth.uniform(2, int(np.prod(shape_add)), -2, 2).reshape(shape_add)
