@@ -443,6 +443,231 @@ __global__ __launch_bounds__(CF_THREADS, C > 3 ? 2 : TM == 1 ? (POOL ? 3 : 4) : 
     __builtin_amdgcn_s_waitcnt(0); /* no wave ends with a direct-to-LDS load in flight */
 }
 
+/* ---- up to 16 filters over 3 channels (the first layer of the tiny networks) ----------------------
+ * The same workgroup, tile, patch and staging scheme on v_mfma_f32_16x16x4_f32: with 16 filters or
+ * fewer the 32x32 MFMA multiplies sixteen rows of zeros and the tail runs on them too.  Here the
+ * pixels are again the row operand: lane (p = lane % 16, g = lane / 16) feeds pixel p and k = 4s + g
+ * of MFMA s (seven of them for K = 27, padded to 28), and owns filter lane % 16 at pixels 4g .. 4g+3
+ * of each 16-pixel block - a wave's 2 rows x 32 columns are four blocks (row j, half h), sixteen
+ * outputs per lane instead of thirty-two.  The 2x2 pooling window still lies inside one lane; a
+ * ballot's 64 bits are four 16-filter words (one per g). */
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+
+template <bool POOL, int WC>
+__global__ __launch_bounds__(CF_THREADS, 4) void conv_first16_kernel(first_args a)
+{
+    constexpr int C = 3, COLS = CF_COLS(WC), NRP = CF_NRP(WC), RS = CF_RS(WC), PR = CF_PR(WC), QR = RS / 4;
+    constexpr int R = 2 * NRP, PQ = CF_PATCH_QUADS(WC, C), ROUNDS = CF_ROUNDS(WC, C);
+    constexpr int K = 27, NS = 7; /* MFMA k quads */
+    typedef __attribute__((address_space(3))) void *lds_ptr;
+    __shared__ __attribute__((aligned(16))) float patch0[ROUNDS * 1024];
+    __shared__ __attribute__((aligned(16))) float patch1[ROUNDS * 1024];
+    __shared__ __attribute__((aligned(16))) float stage[16 * 256]; /* 16 filters x the tile's 256 pixels, then the pooled map */
+    const int tid = threadIdx.x, lane = tid & 63, f = lane & 15, g = lane >> 4;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int wr = wave / WC, wx = wave % WC;
+    const int H = a.H, W = a.W, M = a.M, H2 = H >> 1, W2 = W >> 1;
+    const dn_f2 slope = {a.slope_hi, a.slope_lo};
+
+    int t, t_end;
+    {
+        const int G = gridDim.x, xcd = blockIdx.x & 7, slot = blockIdx.x >> 3;
+        const int gx = (G >> 3) + (xcd < (G & 7) ? 1 : 0);
+        const int q = a.ntiles >> 3, r = a.ntiles & 7;
+        const int x0 = xcd * q + (xcd < r ? xcd : r), nx = q + (xcd < r ? 1 : 0);
+        t = x0 + (int)((long)nx * slot / gx);
+        t_end = x0 + (int)((long)nx * (slot + 1) / gx);
+    }
+    if (t >= t_end) return;
+
+    /* once per workgroup: this lane's filter - the weight of its k of every MFMA, the tail constants */
+    float aw[NS];
+    int koff[NS];
+#pragma unroll
+    for (int s = 0; s < NS; ++s) {
+        const int k = 4 * s + g;
+        const int ch = k / 9, r9 = k - 9 * ch, ky = r9 / 3, kx = r9 - 3 * ky;
+        koff[s] = k < K ? (ch * PR + ky) * RS + kx + 3 : 0; /* pixel x sits in column x + 4 */
+        aw[s] = (k < K && f < M) ? a.w[f * K + k] : 0.f;
+    }
+    const int mf = f < M ? f : M - 1;
+    const dn_tail_row row = dn_tail_make(a.bn, a.biases[mf], a.bn ? a.scales[mf] : 1.f, a.bn ? a.mean[mf] : 0.f,
+                                         a.bn ? a.var[mf] : 1.f);
+
+    int q_rel[ROUNDS], q_rq[ROUNDS];
+#pragma unroll
+    for (int it = 0; it < ROUNDS; ++it) {
+        const int e = it * 256 + tid;
+        const int cr = e / QR, qx = e - QR * cr, ch = cr / PR, r = cr - PR * ch;
+        q_rel[it] = e < PQ ? ((ch * H + r) * W + 4 * qx) * 4 : -1;
+        q_rq[it] = r | (qx << 8);
+    }
+    const __amdgpu_buffer_rsrc_t in_rsrc =
+        __builtin_amdgcn_make_buffer_rsrc((void *)a.in, 0, (int)a.in_bytes, 0x00020000);
+
+    int cb = t % a.tiles_per_row, u = t / a.tiles_per_row;
+    int rp = u % a.bands, b = u / a.bands; /* rp: the band */
+
+    auto load_patch = [&](float *__restrict__ buf, int lb, int lrp, int lcb) {
+        const int y_top = R * lrp - 1, x_left = COLS * lcb - 4;
+        const unsigned origin = (((unsigned)(lb * C * H) + (unsigned)y_top) * (unsigned)W + (unsigned)x_left) * 4u;
+#pragma unroll
+        for (int it = 0; it < ROUNDS; ++it) {
+            const int iy = y_top + (q_rq[it] & 255), xq = x_left + 4 * (q_rq[it] >> 8);
+            const bool ok = q_rel[it] >= 0 && (unsigned)iy < (unsigned)H && (unsigned)xq < (unsigned)W;
+            const unsigned voff = ok ? origin + (unsigned)q_rel[it] : 0xFFFFFFF0u;
+            __builtin_amdgcn_raw_ptr_buffer_load_lds(in_rsrc, (lds_ptr)&buf[(it * 256 + wave * 64) * 4], 16, voff, 0, 0, 0);
+        }
+    };
+
+    load_patch(patch0, b, rp, cb);
+    auto do_tile = [&](const float *__restrict__ buf, float *__restrict__ nbuf, float *__restrict__ stg) {
+        int ncb = cb + 1, nrp = rp, nb = b;
+        if (ncb == a.tiles_per_row) {
+            ncb = 0;
+            if (++nrp == a.bands) {
+                nrp = 0;
+                ++nb;
+            }
+        }
+        CF_BARRIER(); /* the staging buffer's last readers are done */
+        const int x0 = COLS * cb;
+        const int tc = W - x0 < COLS ? W - x0 : COLS;
+        const bool active = 32 * wx < tc; /* wave-uniform */
+
+        f32x4 acc[2][2]; /* [row j][16-column half h]: filter f, columns x0 + 32wx + 16h + 4g + (0..3) */
+#pragma unroll
+        for (int j = 0; j < 2; ++j)
+#pragma unroll
+            for (int h = 0; h < 2; ++h) acc[j][h] = (f32x4){0.f, 0.f, 0.f, 0.f};
+        if (active) {
+            const int base = 2 * wr * RS + 32 * wx + f; /* as the pixel operand, lane % 16 is the pixel of the block */
+#pragma unroll
+            for (int s = 0; s < NS; ++s)
+#pragma unroll
+                for (int j = 0; j < 2; ++j)
+#pragma unroll
+                    for (int h = 0; h < 2; ++h)
+                        acc[j][h] = __builtin_amdgcn_mfma_f32_16x16x4f32(buf[base + j * RS + 16 * h + koff[s]], aw[s],
+                                                                         acc[j][h], 0, 0, 0);
+        }
+        if (t + 1 < t_end) load_patch(nbuf, nb, nrp, ncb);
+
+        float pooled[2][2]; /* [half h][e]: pooled column 8h + 2g + e of the wave's sixteen */
+        if (a.out) {
+#pragma unroll
+            for (int j = 0; j < 2; ++j)
+#pragma unroll
+                for (int h = 0; h < 2; ++h)
+#pragma unroll
+                    for (int r = 0; r < 4; ++r) acc[j][h][r] = dn_tail(acc[j][h][r], row, slope);
+            if (POOL) {
+#pragma unroll
+                for (int h = 0; h < 2; ++h)
+#pragma unroll
+                    for (int e = 0; e < 2; ++e) {
+                        float m = -FLT_MAX; /* the window in the pooling layer's order: first maximum wins */
+                        if (acc[0][h][2 * e] > m) m = acc[0][h][2 * e];
+                        if (acc[0][h][2 * e + 1] > m) m = acc[0][h][2 * e + 1];
+                        if (acc[1][h][2 * e] > m) m = acc[1][h][2 * e];
+                        if (acc[1][h][2 * e + 1] > m) m = acc[1][h][2 * e + 1];
+                        pooled[h][e] = m;
+                    }
+            }
+        }
+        CF_WAIT_VM0(); /* the next patch has landed (every path comes by here); the next barrier publishes it */
+        if (a.out) {
+            if (active) {
+#pragma unroll
+                for (int j = 0; j < 2; ++j)
+#pragma unroll
+                    for (int h = 0; h < 2; ++h) {
+                        const int qd = (2 * wr + j) * (8 * WC) + 8 * wx + 4 * h + g; /* quad of the tile */
+                        float4 o;
+                        o.x = acc[j][h][0];
+                        o.y = acc[j][h][1];
+                        o.z = acc[j][h][2];
+                        o.w = acc[j][h][3];
+                        *(float4 *)&stg[(f * 64 + (qd ^ f)) * 4] = o;
+                    }
+            }
+            CF_BARRIER();
+#pragma unroll
+            for (int it = 0; it < 4; ++it) {
+                const int id = it * 256 + tid;
+                const int m = id >> 6, qd = id & 63, j = qd / (8 * WC), q = qd % (8 * WC);
+                if (4 * q < tc && m < M) {
+                    const float4 o = *(const float4 *)&stg[(m * 64 + (qd ^ m)) * 4];
+                    *(float4u *)(a.out + (((long)b * M + m) * H + R * rp + j) * W + x0 + 4 * q) =
+                        (float4u){o.x, o.y, o.z, o.w};
+                }
+            }
+        } else if (POOL) {
+            /* the map is not wanted: the tail once per pooled pixel, on the sum it is largest for */
+#pragma unroll
+            for (int h = 0; h < 2; ++h)
+#pragma unroll
+                for (int e = 0; e < 2; ++e) {
+                    const float s0 = acc[0][h][2 * e], s1 = acc[0][h][2 * e + 1];
+                    const float s2 = acc[1][h][2 * e], s3 = acc[1][h][2 * e + 1];
+                    const float hi = fmaxf(fmaxf(s0, s1), fmaxf(s2, s3)), lo = fminf(fminf(s0, s1), fminf(s2, s3));
+                    const float v = dn_tail(row.scale >= 0.f ? hi : lo, row, slope);
+                    pooled[h][e] = v > -FLT_MAX ? v : -FLT_MAX;
+                }
+        }
+
+        if (POOL) {
+            const int PW = W2, px0 = x0 >> 1, pc = tc >> 1; /* pooled columns of this tile */
+            float *__restrict__ pstg = stg;
+            if (a.out) CF_BARRIER(); /* the map's rows have been read */
+            if (active) {
+#pragma unroll
+                for (int h = 0; h < 2; ++h) {
+                    const int p2 = wr * (8 * WC) + 8 * wx + 4 * h + g; /* pair of the tile's 64 pooled pixels */
+                    *(float2 *)&pstg[(f * 32 + (p2 ^ (f << 1))) * 2] = make_float2(pooled[h][0], pooled[h][1]);
+                }
+                if (a.bits) {
+                    /* one ballot per (h, e): its four 16-bit fields are the words of pooled columns 8h + 2g' + e */
+                    unsigned word = 0;
+#pragma unroll
+                    for (int h = 0; h < 2; ++h)
+#pragma unroll
+                        for (int e = 0; e < 2; ++e) {
+                            const unsigned long long m64 = __ballot(pooled[h][e] > 0.f);
+#pragma unroll
+                            for (int gg = 0; gg < 4; ++gg)
+                                if (lane == 8 * h + 2 * gg + e) word = (unsigned)(m64 >> (16 * gg)) & 0xFFFFu;
+                        }
+                    if (M < 16) word &= (1u << M) - 1u;
+                    if (lane < 16 && 16 * wx + lane < pc)
+                        a.bits[((long)b * H2 + NRP * rp + wr) * PW + px0 + 16 * wx + lane] = word;
+                }
+            }
+            CF_BARRIER();
+            {
+                const int m = tid >> 4, qq = tid & 15, pj = qq / (4 * WC), pq = qq % (4 * WC);
+                if (4 * pq < pc && m < M) {
+                    const float4 o = *(const float4 *)&pstg[(m * 16 + (qq ^ m)) * 4];
+                    *(float4u *)(a.pool + (((long)b * M + m) * H2 + NRP * rp + pj) * PW + px0 + 4 * pq) =
+                        (float4u){o.x, o.y, o.z, o.w};
+                }
+            }
+        }
+        cb = ncb;
+        rp = nrp;
+        b = nb;
+    };
+    __builtin_amdgcn_s_waitcnt(0); /* the first patch */
+    CF_BARRIER();
+    for (;;) {
+        do_tile(patch0, patch1, stage);
+        if (++t >= t_end) break;
+        do_tile(patch1, patch0, stage);
+        if (++t >= t_end) break;
+    }
+    __builtin_amdgcn_s_waitcnt(0); /* no wave ends with a direct-to-LDS load in flight */
+}
+
 /* Whether conv_first_kernel serves the layer (then also with the pooled outputs): 3x3 / stride 1 / pad 1
  * over 3 channels (up to 64 filters) or 16 channels (up to 32 filters: a lane keeps its filter's 144
  * weights in registers), even height, width a multiple of 8 (pooled rows leave in 16-byte quads). */
@@ -491,18 +716,28 @@ static const void *kernel_of_shape(int wc)
                    : (const void *)conv_first_kernel<TM, POOL, 1, C>;
 }
 
-/* variant index: [16 channels | 3 channels with more than 32 filters | 3 channels][pooled][shape] */
-static int variant_of(int c, int n) { return c == 16 ? 2 : n > 32 ? 1 : 0; }
+template <bool POOL>
+static const void *kernel16_of_shape(int wc)
+{
+    return wc == 4 ? (const void *)conv_first16_kernel<POOL, 4>
+         : wc == 2 ? (const void *)conv_first16_kernel<POOL, 2>
+                   : (const void *)conv_first16_kernel<POOL, 1>;
+}
+
+/* variant index: [3 channels, up to 16 filters | 16 channels | 3 channels, more than 32 filters | 3 channels, 17..32] */
+static int variant_of(int c, int n) { return c == 16 ? 2 : n > 32 ? 1 : n <= 16 ? 3 : 0; }
 
 extern "C" const char *conv_first_kernel_name(int c, int n, int pooled, int h, int w)
 {
-    static const char *const names[3][2][3] = {
+    static const char *const names[4][2][3] = {
         {{"conv_first_kernel<1,false,1,3>", "conv_first_kernel<1,false,2,3>", "conv_first_kernel<1,false,4,3>"},
          {"conv_first_kernel<1,true,1,3>", "conv_first_kernel<1,true,2,3>", "conv_first_kernel<1,true,4,3>"}},
         {{"conv_first_kernel<2,false,1,3>", "conv_first_kernel<2,false,2,3>", "conv_first_kernel<2,false,4,3>"},
          {"conv_first_kernel<2,true,1,3>", "conv_first_kernel<2,true,2,3>", "conv_first_kernel<2,true,4,3>"}},
         {{"conv_first_kernel<1,false,1,16>", "conv_first_kernel<1,false,2,16>", "conv_first_kernel<1,false,4,16>"},
-         {"conv_first_kernel<1,true,1,16>", "conv_first_kernel<1,true,2,16>", "conv_first_kernel<1,true,4,16>"}}};
+         {"conv_first_kernel<1,true,1,16>", "conv_first_kernel<1,true,2,16>", "conv_first_kernel<1,true,4,16>"}},
+        {{"conv_first16_kernel<false,1>", "conv_first16_kernel<false,2>", "conv_first16_kernel<false,4>"},
+         {"conv_first16_kernel<true,1>", "conv_first16_kernel<true,2>", "conv_first16_kernel<true,4>"}}};
     const int wc = pick_shape(c, h, w);
     return names[variant_of(c, n)][pooled != 0][wc >> 1];
 }
@@ -541,12 +776,13 @@ extern "C" void conv_first_forward(const float *input, const float *weights, con
     a.slope_hi = s.hi;
     a.slope_lo = s.lo;
     const int v = variant_of(c, n);
-    const void *kernel = v == 2 ? (pool ? kernel_of_shape<1, true, 16>(wc) : kernel_of_shape<1, false, 16>(wc))
+    const void *kernel = v == 3 ? (pool ? kernel16_of_shape<true>(wc) : kernel16_of_shape<false>(wc))
+                       : v == 2 ? (pool ? kernel_of_shape<1, true, 16>(wc) : kernel_of_shape<1, false, 16>(wc))
                        : v == 1 ? (pool ? kernel_of_shape<2, true, 3>(wc) : kernel_of_shape<2, false, 3>(wc))
                                 : (pool ? kernel_of_shape<1, true, 3>(wc) : kernel_of_shape<1, false, 3>(wc));
     /* exactly as many workgroups as stay resident (two to four per CU, by the variant's registers and
      * LDS), each walking its run: one more per CU would start when the others end and run alone */
-    static int resident[3][2][3];
+    static int resident[4][2][3];
     int *per_cu = &resident[v][pool != 0][wc >> 1];
     if (!*per_cu) {
         int nb = 0;

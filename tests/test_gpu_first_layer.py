@@ -68,7 +68,7 @@ GEOMS16 = [(1, 2, 32, 32), (2, 8, 64, 32), (1, 16, 208, 32), (3, 12, 128, 17), (
 @pytest.mark.parametrize("b,h,w,n", GEOMS)
 def test_first_layer_against_the_checker(dn, orc, b, h, w, n):
     assert dn.conv_maxpool_fusable(b, 3, h, w, n, 1, 3, 1, 1, ACTIVATIONS.index("leaky")) == 1
-    assert dn.conv_kernel_name_geometry(b, 3, h, w, n, 1, 3, 1, 1).decode().startswith("conv_first_kernel")
+    assert dn.conv_kernel_name_geometry(b, 3, h, w, n, 1, 3, 1, 1).decode().startswith("conv_first")
     cs = First(dn, 3, b, h, w, n)
     got = cs.conv().numpy((b, n, h, w))
     want = orc.conv(cs.x, cs.wt, cs.bias, cs.sc, cs.mu, cs.var, n=n, size=3, stride=1, pad=1, groups=1,
