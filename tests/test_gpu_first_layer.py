@@ -30,13 +30,27 @@ class First:
         b, h, w, n = self.geom
         return [b, self.c, h, w, n, 1, 3, 1, 1, self.bn, ACTIVATIONS.index(self.act)]
 
+    GUARD = 256  # floats behind every output buffer that no kernel may touch
+
+    def guarded(self, count, dtype=np.float32):
+        """A device buffer of `count` elements plus GUARD sentinels behind it, all preset to a NaN pattern."""
+        host = np.full(count + self.GUARD, 0x7FC0BEEF, np.uint32).view(dtype)
+        return D(host, dtype=dtype)
+
+    def unguard(self, dev, count):
+        """The buffer's first `count` elements as uint32, after checking that the sentinels are intact."""
+        bits = dev.numpy().view(np.uint32)
+        assert (bits[count:] == 0x7FC0BEEF).all(), "a kernel wrote past the end of its output"
+        return bits[:count].copy()
+
     def conv(self):
         b, h, w, n = self.geom
         d = self.dev
-        out = D(np.full(b * n * h * w, np.nan, np.float32))
+        count = b * n * h * w
+        out = self.guarded(count)
         self.dn.forward_convolutional_gpu(d[0].ptr, d[1].ptr, None, d[2].ptr, d[3].ptr, d[4].ptr, d[5].ptr, out.ptr,
                                           *self.tail())
-        return out
+        return D(self.unguard(out, count).view(np.float32))
 
     def separate(self):
         b, h, w, n = self.geom
@@ -50,12 +64,11 @@ class First:
     def fused(self, write_map=True):
         b, h, w, n = self.geom
         d = self.dev
-        out = D(np.full(b * n * h * w, np.nan, np.float32))
-        pooled = D(np.full(b * n * (h // 2) * (w // 2), np.nan, np.float32))
-        bits = D(np.full(self.dn.xnor_input_words(b, n, h // 2, w // 2), -1, np.int32))
+        n_map, n_pool, n_bits = b * n * h * w, b * n * (h // 2) * (w // 2), self.dn.xnor_input_words(b, n, h // 2, w // 2)
+        out, pooled, bits = self.guarded(n_map), self.guarded(n_pool), self.guarded(n_bits, np.int32)
         self.dn.forward_convolutional_maxpool_gpu(d[0].ptr, d[1].ptr, d[2].ptr, d[3].ptr, d[4].ptr, d[5].ptr,
                                                   out.ptr if write_map else None, pooled.ptr, bits.ptr, *self.tail())
-        return out.numpy().view(np.uint32), pooled.numpy().view(np.uint32), bits.numpy().view(np.uint32)
+        return self.unguard(out, n_map), self.unguard(pooled, n_pool), self.unguard(bits, n_bits)
 
 
 GEOMS = [(1, 2, 32, 16), (2, 6, 64, 32), (3, 10, 160, 17), (1, 16, 416, 32), (2, 8, 128, 64), (5, 4, 96, 33),
