@@ -677,6 +677,7 @@ extern "C" int conv_first_serves(int batch, int c, int h, int w, int n, int grou
     if (!((c == 3 && n <= 64) || (c == 16 && n <= 32))) return 0;
     if (batch < 1 || h < 2 || (h & 1) || w < 32 || (w & 7)) return 0;
     if ((long)batch * c * h * w * 4 >= (1L << 32) - 64) return 0; /* 32-bit buffer offsets */
+    if ((long)c * h * w * 4 >= (1L << 31)) return 0;              /* a lane's offsets inside one image are signed */
     if ((long)batch * (h / 2) * ((w + 31) / 32) >= (1L << 31)) return 0;
     return 1;
 }
