@@ -18,7 +18,7 @@ OBJDIR = os.path.join(HERE, "build")
 LIB = os.path.join(HERE, "libdarknet_hip.so")
 ROCM = os.environ.get("ROCM_PATH", "/opt/rocm")
 
-HIP_SOURCES = ["pointwise.hip", "pool.hip", "conv_direct.hip", "conv_mfma.hip", "conv_first.hip", "xnor.hip", "detect.hip", "image.hip", "local.hip"]
+HIP_SOURCES = ["pointwise.hip", "pool.hip", "conv_direct.hip", "conv_mfma.hip", "conv_first.hip", "conv_group.hip", "xnor.hip", "detect.hip", "image.hip", "local.hip"]
 C_SOURCES = ["hip.c", "cfg_reader.c", "cfg_parser.c", "layers.c", "network.c", "weights_io.c", "boxes.c", "images.c", "pipeline.c"]
 
 # -packed-fp32-ops: keep the compiler from forming packed fp32 instructions.

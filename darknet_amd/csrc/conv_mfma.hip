@@ -69,6 +69,12 @@ extern "C" void conv_direct_forward(const float *, const float *, const float *,
                                     const float *, const float *, float *, int, int, int, int, int,
                                     int, int, int, int, int, int);
 
+/* conv_group.hip: grouped 3x3 layers of 4 or 8 channels per group, on the vector ALU */
+extern "C" int conv_group_serves(int batch, int c, int h, int w, int n, int groups, int size, int stride, int pad);
+extern "C" const char *conv_group_kernel_name(int c, int groups, int stride);
+extern "C" void conv_group_forward(const float *input, const float *weights, const float *biases, const float *scales,
+                                   const float *rolling_mean, const float *rolling_variance, float *output, int batch,
+                                   int c, int h, int w, int n, int groups, int stride, int batch_normalize, double slope);
 /* conv_first.hip: the kernel of 3-channel first layers */
 extern "C" int conv_first_serves(int batch, int c, int h, int w, int n, int groups, int size, int stride, int pad);
 extern "C" const char *conv_first_kernel_name(int c, int n, int pooled, int h, int w);
@@ -1440,6 +1446,10 @@ static int conv_first_takes(int mode, int c)
     return (mode == 3 && c == 3) || (mode == 13 && c == 16 && g_precision == 0);
 }
 
+/* Whether a grouped layer goes to the vector-ALU kernel of small groups when its geometry fits: in
+ * the default mode only (conv_set_algo(3) keeps such a layer on the matrix cores: the cross-check). */
+static int conv_group_takes(void) { return g_algo == 0 && g_precision == 0; }
+
 extern "C" void conv_set_precision(int precision)
 {
     if (precision < 0 || precision > 2)
@@ -1510,6 +1520,8 @@ extern "C" const char *conv_kernel_name_geometry(int batch, int c, int h, int w,
     if (columns >= (1L << 31) - 512) mode = -1;
     if (conv_first_takes(mode, c) && conv_first_serves(batch, c, h, w, n, groups, size, stride, pad))
         return conv_first_kernel_name(c, n, 0, h, w);
+    if (conv_group_takes() && conv_group_serves(batch, c, h, w, n, groups, size, stride, pad))
+        return conv_group_kernel_name(c, groups, stride);
     const int patch = g_algo == 0 && mode == 3 && conv_patch_floats(c, h, w, n, groups, size, stride, pad) > 0;
     return kernel_name(n, c, groups, size, columns, patch, mode);
 }
@@ -1892,6 +1904,13 @@ static void conv_forward(const float *input, const float *weights, const float *
         return;
     }
 
+    /* grouped 3x3 layers of 4 or 8 channels per group: the vector-ALU kernel (a block-diagonal tile on the
+     * matrix cores would multiply 7/8 or 3/4 zeros) */
+    if (conv_group_takes() && !sum && conv_group_serves(batch, c, h, w, n, groups, size, stride, pad)) {
+        conv_group_forward(input, weights, biases, scales, rolling_mean, rolling_variance, output, batch, c, h, w, n,
+                           groups, stride, batch_normalize, slope);
+        return; /* a pending timing pair stays pending: conv_profile_pending() tells the caller it was not used */
+    }
     /* first layers (3 channels, or 16 behind a pooled first layer; 3x3 / 1 / pad 1, even height, width a
      * multiple of 32): their own kernel */
     if (conv_first_takes(mode, c) && !sum && conv_first_serves(batch, c, h, w, n, groups, size, stride, pad)) {

@@ -228,6 +228,8 @@ def test_grouped_mfma_tiles_agree_with_direct_kernel_and_unpacked_call(dn):
     bias, sc, mu, var = synth.bn_random(6, n)
     kw = dict(n=n, size=3, stride=2, pad=1, groups=groups, bn=1, act="leaky")
     assert dn.conv_kernel_name(n, c, groups, 3).decode() == "conv_mfma_kernel<32,256,32,64,13>"
+    # (8 per group at stride 1 would run on the vector-ALU kernel of small groups; at stride 2 the matrix cores keep it)
+    assert dn.conv_kernel_name_geometry(b, c, h, w, n, groups, 3, 2, 1).decode() == "conv_mfma_kernel<32,256,32,64,13>"
     fast = run_conv(dn, x, wt, bias, sc, mu, var, **kw)
     assert np.array_equal(fast, run_conv(dn, x, wt, bias, sc, mu, var, packed=False, **kw))
     dn.conv_set_algo(1)
@@ -237,6 +239,49 @@ def test_grouped_mfma_tiles_agree_with_direct_kernel_and_unpacked_call(dn):
     finally:
         dn.conv_set_algo(0)
     assert norm_err(fast, direct) <= 2e-6
+
+
+@pytest.mark.parametrize("b,c,h,w,groups,stride,act,bn", [
+    (2, 128, 56, 56, 32, 1, "leaky", 1),      # resnext50 stage 1: 4 per group
+    (1, 128, 57, 41, 32, 2, "leaky", 1),      # 4 per group, stride 2, odd sizes: ragged tiles on both axes
+    (3, 16, 9, 70, 4, 1, "linear", 0),        # 4 per group, three tiles across, no batch-norm
+    (2, 64, 33, 8, 8, 1, "relu", 1),          # 8 per group, narrower than a tile
+    (2, 16, 12, 66, 4, 2, "relu", 1),         # 4 per group, stride 2, one column into the second tile
+    (1, 8, 1, 1, 2, 1, "leaky", 1),           # a single pixel
+    (2, 32, 17, 33, 4, 1, "leaky", 1)])       # 8 per group, stride 1, one column into the second tile
+def test_small_group_kernel(dn, orc, b, c, h, w, groups, stride, act, bn):
+    """Grouped 3x3 layers of 4 or 8 channels per group on the vector-ALU kernel: against the CPU checker and
+    the fp64 convolution as every convolution, and against the same layer on the matrix cores; sentinels
+    behind the output."""
+    n = c
+    name = dn.conv_kernel_name_geometry(b, c, h, w, n, groups, 3, stride, 1).decode()
+    assert name == f"conv_group_kernel<{c // groups},{stride}>", name
+    x = synth.uniform(41, b * c * h * w).reshape(b, c, h, w)
+    wt = synth.conv_weights(42, n, c // groups, 3)
+    bias, sc, mu, var = synth.bn_random(43, n)
+    sc = sc.copy()
+    sc[2::5] *= -1.0
+    kw = dict(n=n, size=3, stride=stride, pad=1, groups=groups)
+    oh, ow = (h - 1) // stride + 1, (w - 1) // stride + 1
+    count, guard = b * n * oh * ow, 512
+    dev = [D(a) for a in (x, wt, bias, sc, mu, var)]
+    out = D(np.full(count + guard, 0x7FC0BEEF, np.uint32).view(np.float32))
+    dn.forward_convolutional_gpu(dev[0].ptr, dev[1].ptr, None, dev[2].ptr, *[d.ptr if bn else None for d in dev[3:]],
+                                 out.ptr, b, c, h, w, n, groups, 3, stride, 1, bn, ACTIVATIONS.index(act))
+    bits = out.numpy().view(np.uint32)
+    assert (bits[count:] == 0x7FC0BEEF).all(), "the kernel wrote past the end of its output"
+    got = bits[:count].view(np.float32).reshape(b, n, oh, ow)
+    assert not np.isnan(got).any()
+    args = (x, wt, bias, sc, mu, var) if bn else (x, wt, bias)
+    want = orc.conv(*args, batch_normalize=bn, activation=act, **kw)
+    assert norm_err(got, want) <= REL_TOL
+    assert norm_err(got, orc.conv_f64(*args, batch_normalize=bn, activation=act, **kw)) <= 5e-6
+    dn.conv_set_algo(3)
+    try:
+        mfma = run_conv(dn, x, wt, bias, sc if bn else None, mu if bn else None, var if bn else None, bn=bn, act=act, **kw)
+    finally:
+        dn.conv_set_algo(0)
+    assert norm_err(got, mfma) <= 2e-6
 
 
 def test_conv_golden_vectors(dn):
