@@ -266,7 +266,7 @@ __global__ void shortcut_general_kernel(const float *in, const float *add, float
     }
 }
 
-/* The same, one output plane (image b, channel k) per blockIdx.y and 32-bit index arithmetic: the
+/* The same, one output plane (image b, channel k) per blockIdx.x and 32-bit index arithmetic: the
  * residual adds of the first block of a ResNeXt stage (more channels out than in, with or without a
  * halved map) are launches of 50-200 MB in which the 64-bit divisions of the kernel above cost more
  * than the memory traffic.  Four consecutive pixels per thread where the plane allows 16-byte
@@ -276,13 +276,13 @@ __global__ void shortcut_planes_kernel(const float *in, const float *add, float 
                                        int w2, int h2, int c2, int stride, int sample, int minw, int minh,
                                        int minc, float s1, float s2, int a)
 {
-    const int plane = blockIdx.y, b = plane / c2, k = plane - b * c2;
+    const int plane = blockIdx.x, b = plane / c2, k = plane - b * c2;
     const int hw2 = h2 * w2;
     const long obase = (long)plane * hw2;
     const bool has_add = k < minc;
     const long abase = ((long)b * c1 + k) * h1 * w1;
     if (QUAD) { /* stride == sample == 1, w1 == w2, h1 == h2, hw2 % 4 == 0 */
-        for (int q = blockIdx.x * blockDim.x + threadIdx.x; q < hw2 / 4; q += gridDim.x * blockDim.x) {
+        for (int q = blockIdx.y * blockDim.x + threadIdx.x; q < hw2 / 4; q += gridDim.y * blockDim.x) {
             float4 v = *(const float4 *)(in + obase + 4 * q);
             if (has_add) {
                 const float4 r = *(const float4 *)(add + abase + 4 * q);
@@ -298,7 +298,7 @@ __global__ void shortcut_planes_kernel(const float *in, const float *add, float 
             *(float4 *)(out + obase + 4 * q) = v;
         }
     } else {
-        for (int p = blockIdx.x * blockDim.x + threadIdx.x; p < hw2; p += gridDim.x * blockDim.x) {
+        for (int p = blockIdx.y * blockDim.x + threadIdx.x; p < hw2; p += gridDim.y * blockDim.x) {
             const int y = p / w2, x = p - y * w2;
             float v = in[obase + p];
             const int xi = x / sample, yi = y / sample;
@@ -327,13 +327,16 @@ extern "C" void forward_shortcut_gpu(const float *in, const float *add, float *o
         hipLaunchKernelGGL(shortcut_same4_kernel, dim3(dn_blocks(n / 4)), dim3(DN_BLOCK), 0, dn_stream(),
                            (const float4 *)in, (const float4 *)add, (float4 *)out, n / 4, s1, s2,
                            activation);
-    } else if ((long)batch * c2 <= 65535 && (long)h2 * w2 < (1L << 30) && (long)h1 * w1 < (1L << 30)) {
+    } else if ((long)h2 * w2 >= 512 && (long)batch * c2 < (1L << 31) && (long)h2 * w2 < (1L << 24) &&
+               (long)h1 * w1 < (1L << 30)) {
+        /* (planes of a few hundred pixels leave most of a workgroup idle: the flat kernel below is faster there -
+         * 46 against 66 us on 1024 planes of 14 x 14 per image, batch 64) */
         const long hw2 = (long)h2 * w2;
         const bool quad = w1 == w2 && h1 == h2 && (hw2 & 3) == 0 && aligned16(in) && aligned16(add) && aligned16(out);
         const long per_plane = quad ? hw2 / 4 : hw2;
         /* about four elements (or quads) per thread: the small planes of the late stages would otherwise be
          * tens of thousands of workgroups of one element per thread */
-        const dim3 grid((unsigned)((per_plane + 4 * DN_BLOCK - 1) / (4 * DN_BLOCK)), (unsigned)(batch * c2));
+        const dim3 grid((unsigned)(batch * c2), (unsigned)((per_plane + 4 * DN_BLOCK - 1) / (4 * DN_BLOCK)));
         if (quad)
             hipLaunchKernelGGL(shortcut_planes_kernel<true>, grid, dim3(DN_BLOCK), 0, dn_stream(), in, add, out, w1, h1,
                                c1, w2, h2, c2, stride, sample, minw, minh, minc, s1, s2, activation);
