@@ -140,6 +140,11 @@ __device__ __forceinline__ void split_k(int k, int size, int &ci, int &ky, int &
         const int r = k - ci * 9;
         ky = (r * 11) >> 5;    /* r/3 for r < 9 */
         kx = r - ky * 3;
+    } else if (KS == 7) { /* the 7x7 stems: constant divisors, a few multiplies instead of two 32-bit divisions per k */
+        ci = k / 49;
+        const int r = k - ci * 49;
+        ky = r / 7;
+        kx = r - ky * 7;
     } else {
         const int ss = size * size;
         ci = k / ss;
@@ -583,9 +588,10 @@ __global__ __launch_bounds__(DN_THREADS, ((BM == 128 && BF16 != 3) ? 3 : 2)) voi
     /* `live` = false: the request is only there to keep a schedule region free of branches (the last
      * step of a loop form that always requests "the next chunk").  Its weights are chunk kc's again
      * (in range by construction); its input lanes all carry the out-of-range offset, so they write
-     * zeros to LDS and read no memory: the tap-blocked input address is built from a scalar offset the
-     * buffer's range check does not cover, and one chunk past the last would reach up to 16 channel
-     * planes beyond the end of the tensor for the last image of the batch. */
+     * zeros to LDS and read no memory.  (The tap-blocked input address of such a request would be one
+     * chunk past the layer's channels; for the last image that lies past the tensor, where only the
+     * buffer's range check - which on this part covers the scalar offset too - stands between the
+     * request and the memory behind the tensor.  A request that is not live does not lean on it.) */
     auto load_chunk = [&](int kc, int buf, bool live = true) {
         /* A */
         if constexpr (BF16) {
@@ -1712,6 +1718,7 @@ static conv_kernel_t pick_kernel(int mode, int bf16, int x3, int sparse)
         case 13: return conv_mfma_kernel<BM, BN, WM, WN, 13>;
         case 1: return conv_mfma_kernel<BM, BN, WM, WN, 1>;
         case 3: return conv_mfma_kernel<BM, BN, WM, WN, 3>;
+        case 7: return conv_mfma_kernel<BM, BN, WM, WN, 7>;
         default: return conv_mfma_kernel<BM, BN, WM, WN, 0>;
         }
     } else {
@@ -1738,6 +1745,7 @@ static conv_kernel_t pick_kernel(int mode, int bf16, int x3, int sparse)
             if constexpr (BM <= 128 && !X3_ONLY) {
                 if (mode == 1) return conv_mfma_kernel<BM, BN, WM, WN, 1>;
                 if (mode == 3) return conv_mfma_kernel<BM, BN, WM, WN, 3>;
+                if (mode == 7) return conv_mfma_kernel<BM, BN, WM, WN, 7>;
                 return conv_mfma_kernel<BM, BN, WM, WN, 0>;
             }
             break;
@@ -1823,7 +1831,7 @@ static int conv_mode(int c, int groups, int size, int stride, int pad, long in_b
         if (size == 3 && pad != 1) return -1;
         return 10 + size;
     }
-    return size == 1 ? 1 : size == 3 ? 3 : 0;
+    return size == 1 ? 1 : size == 3 ? 3 : size == 7 ? 7 : 0;
 }
 
 extern "C" void forward_shortcut_gpu(const float *, const float *, float *, int, int, int, int, int, int, int,
