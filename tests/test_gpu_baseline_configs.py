@@ -152,4 +152,20 @@ def test_yolov3_tiny_xnor_416_batch_64(dn):
     for j in (1, 17, 63):
         twin = int(np.flatnonzero(perm == perm[j])[0])
         assert np.abs(first[j] - first[twin]).max() <= 1e-5, j
+    # at this size too, the passes that run several layers in one launch (first layer + maxpool + sign bits,
+    # xnor convolution + maxpool + sign bits) leave the bits of the layer-by-layer run in both yolo heads, and
+    # so does the mode that does not write the maps only a fused maxpool reads
+    heads = [i for i, L in enumerate(net.layers) if L["type"] == "yolo"]
+    xin = np.ascontiguousarray(x4.reshape(4, -1)[perm])
+    try:
+        lib.network_set_fusion(0)
+        net.predict(xin)
+        plain = [net.layer_output(i) for i in heads]
+        for level in (1, 2):
+            lib.network_set_fusion(level)
+            net.predict(xin)
+            for i, ref in zip(heads, plain):
+                assert np.array_equal(net.layer_output(i), ref), (level, i)
+    finally:
+        lib.network_set_fusion(1)
     net.free()
