@@ -218,3 +218,24 @@ def test_sixteen_channel_layer_with_pool_and_bits_in_one_pass(dn, b, h, w, n, ac
     assert np.array_equal(lean_pool, want_pool) and np.array_equal(lean_bits, want_bits)
     assert np.isnan(lean_map.view(np.float32)).all()
 
+
+def test_tiny_network_at_416_batch_64_fused_equals_layer_by_layer(dn):
+    """The benchmark size: both pooled first layers (3 -> 16 and 16 -> 32 with their maxpools) and both yolo
+    heads of yolov3-tiny hold the bits of the layer-by-layer run at fusion levels 1 and 2."""
+    net = api.Network(cfg_text=cfgs.yolov3_tiny(64, 416))
+    fill_params(net.set_conv, net.layers)
+    x = synth.uniform01(9, net.inputs * 64)
+    watch = [1, 3] + [i for i, L in enumerate(net.layers) if L["type"] == "yolo"]
+    try:
+        dn.network_set_fusion(0)
+        net.predict(x)
+        want = {i: net.layer_output(i) for i in watch}
+        for level in (1, 2):
+            dn.network_set_fusion(level)
+            net.predict(x)
+            for i in watch:
+                assert np.array_equal(net.layer_output(i), want[i]), (level, i)
+    finally:
+        dn.network_set_fusion(1)
+    net.free()
+
