@@ -72,10 +72,11 @@ class First:
 
 
 GEOMS = [(1, 2, 32, 16), (2, 6, 64, 32), (3, 10, 160, 17), (1, 16, 416, 32), (2, 8, 128, 64), (5, 4, 96, 33),
-         (1, 34, 256, 1), (2, 12, 288, 48), (2, 8, 104, 24), (1, 4, 40, 64), (3, 6, 200, 9)]
+         (1, 34, 256, 1), (2, 12, 288, 48), (2, 8, 104, 24), (1, 4, 40, 64), (3, 6, 200, 9),
+         (2, 416, 416, 16), (1, 416, 416, 32), (1, 448, 448, 64)]   # the first layers of yolov3-tiny, yolov3 and yolov1 at full size
 # 16 channels, up to 32 filters: the second convolution of the tiny networks (16 -> 32 at 208 x 208)
 GEOMS16 = [(1, 2, 32, 32), (2, 8, 64, 32), (1, 16, 208, 32), (3, 12, 128, 17), (2, 24, 96, 1), (1, 6, 160, 31),
-           (2, 8, 56, 32), (1, 4, 104, 20)]
+           (2, 8, 56, 32), (1, 4, 104, 20), (2, 208, 208, 32)]   # the last: yolov3-tiny's second convolution at full size
 
 
 @pytest.mark.parametrize("b,h,w,n", GEOMS)
