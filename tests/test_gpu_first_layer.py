@@ -240,3 +240,32 @@ def test_tiny_network_at_416_batch_64_fused_equals_layer_by_layer(dn):
         dn.network_set_fusion(1)
     net.free()
 
+
+def random_first_layers(seed, count):
+    rng = np.random.default_rng(seed)
+    out = []
+    for _ in range(count):
+        c = int(rng.choice([3, 3, 16]))
+        n = int(rng.integers(1, 65 if c == 3 else 33))
+        h = 2 * int(rng.integers(1, 21))
+        w = 8 * int(rng.integers(4, 38))
+        b = int(rng.integers(1, 5))
+        act, bn = [("leaky", 1), ("linear", 0), ("relu", 1)][int(rng.integers(0, 3))]
+        out.append((c, b, h, w, n, act, bn))
+    return out
+
+
+@pytest.mark.parametrize("c,b,h,w,n,act,bn", random_first_layers(20250, 32))
+def test_random_first_layers(dn, orc, c, b, h, w, n, act, bn):
+    """Random heights, widths (any multiple of 8: short last tiles, every tile shape the height allows), filter
+    counts and batches: the map against the checker, the one-pass pooled forms against the separate calls."""
+    cs = First(dn, 77, b, h, w, n, act=act, bn=bn, c=c)
+    want_map, want_pool, want_bits = cs.separate()
+    args = (cs.x, cs.wt, cs.bias, cs.sc, cs.mu, cs.var) if bn else (cs.x, cs.wt, cs.bias)
+    ref = orc.conv(*args, n=n, size=3, stride=1, pad=1, groups=1, batch_normalize=bn, activation=act)
+    assert norm_err(want_map.view(np.float32).reshape(b, n, h, w), ref) <= REL_TOL
+    got_map, got_pool, got_bits = cs.fused()
+    assert np.array_equal(got_map, want_map) and np.array_equal(got_pool, want_pool) and np.array_equal(got_bits, want_bits)
+    lean = cs.fused(write_map=False)
+    assert np.array_equal(lean[1], want_pool) and np.array_equal(lean[2], want_bits)
+
