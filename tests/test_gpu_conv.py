@@ -381,3 +381,23 @@ def test_batches_beyond_4_gib_run_in_slices_of_whole_images(dn):
     for i in (0, per - 1, per, b - 1):
         alone = run_conv(dn, x[i:i + 1], wt, bias, sc, mu, var, **kw)
         assert norm_err(got[i:i + 1], alone) <= 1e-5, i
+
+
+def random_small_groups(seed, count):
+    rng = np.random.default_rng(seed)
+    out = []
+    for _ in range(count):
+        cg = int(rng.choice([4, 8]))
+        groups = int(rng.choice([2, 3, 8, 32]))
+        stride = 1 if cg == 8 else int(rng.choice([1, 2]))
+        h, w = int(rng.integers(1, 40)), int(rng.integers(1, 80))
+        b = int(rng.integers(1, 4))
+        act, bn = [("leaky", 1), ("linear", 0), ("relu", 1)][int(rng.integers(0, 3))]
+        out.append((b, cg * groups, h, w, groups, stride, act, bn))
+    return out
+
+
+@pytest.mark.parametrize("b,c,h,w,groups,stride,act,bn", random_small_groups(20251, 16))
+def test_small_group_kernel_random_geometries(dn, orc, b, c, h, w, groups, stride, act, bn):
+    test_small_group_kernel(dn, orc, b, c, h, w, groups, stride, act, bn)
+
