@@ -728,6 +728,30 @@ static const void *kernel16_of_shape(int wc)
 /* variant index: [3 channels, up to 16 filters | 16 channels | 3 channels, more than 32 filters | 3 channels, 17..32] */
 static int variant_of(int c, int n) { return c == 16 ? 2 : n > 32 ? 1 : n <= 16 ? 3 : 0; }
 
+/* Resident workgroups per CU of every variant [variant_of][pooled][shape], asked of the runtime once (from
+ * the library's device set-up, so that no launch path has to: a caller may be capturing its stream). */
+static int g_resident[4][2][3];
+
+static const void *kernel_of(int v, int pooled, int wc)
+{
+    return v == 3 ? (pooled ? kernel16_of_shape<true>(wc) : kernel16_of_shape<false>(wc))
+         : v == 2 ? (pooled ? kernel_of_shape<1, true, 16>(wc) : kernel_of_shape<1, false, 16>(wc))
+         : v == 1 ? (pooled ? kernel_of_shape<2, true, 3>(wc) : kernel_of_shape<2, false, 3>(wc))
+                  : (pooled ? kernel_of_shape<1, true, 3>(wc) : kernel_of_shape<1, false, 3>(wc));
+}
+
+extern "C" __attribute__((visibility("hidden"))) void conv_first_device_setup(void)
+{
+    if (g_resident[0][0][0]) return;
+    for (int v = 3; v >= 0; --v) /* [0][0][0] last: it is the flag */
+        for (int p = 1; p >= 0; --p)
+            for (int s = 2; s >= 0; --s) {
+                int nb = 0;
+                hip_check_error(hipOccupancyMaxActiveBlocksPerMultiprocessor(&nb, kernel_of(v, p, 1 << s), CF_THREADS, 0));
+                g_resident[v][p][s] = nb < 1 ? 1 : nb > 4 ? 4 : nb;
+            }
+}
+
 extern "C" const char *conv_first_kernel_name(int c, int n, int pooled, int h, int w)
 {
     static const char *const names[4][2][3] = {
@@ -777,19 +801,11 @@ extern "C" void conv_first_forward(const float *input, const float *weights, con
     a.slope_hi = s.hi;
     a.slope_lo = s.lo;
     const int v = variant_of(c, n);
-    const void *kernel = v == 3 ? (pool ? kernel16_of_shape<true>(wc) : kernel16_of_shape<false>(wc))
-                       : v == 2 ? (pool ? kernel_of_shape<1, true, 16>(wc) : kernel_of_shape<1, false, 16>(wc))
-                       : v == 1 ? (pool ? kernel_of_shape<2, true, 3>(wc) : kernel_of_shape<2, false, 3>(wc))
-                                : (pool ? kernel_of_shape<1, true, 3>(wc) : kernel_of_shape<1, false, 3>(wc));
+    const void *kernel = kernel_of(v, pool != 0, wc);
     /* exactly as many workgroups as stay resident (two to four per CU, by the variant's registers and
      * LDS), each walking its run: one more per CU would start when the others end and run alone */
-    static int resident[4][2][3];
-    int *per_cu = &resident[v][pool != 0][wc >> 1];
-    if (!*per_cu) {
-        int nb = 0;
-        hip_check_error(hipOccupancyMaxActiveBlocksPerMultiprocessor(&nb, kernel, CF_THREADS, 0));
-        *per_cu = nb < 1 ? 1 : nb > 4 ? 4 : nb;
-    }
+    if (!g_resident[0][0][0]) conv_first_device_setup();
+    const int *per_cu = &g_resident[v][pool != 0][wc >> 1];
     long grid = (long)(cus > 0 ? cus : 256) * *per_cu;
     if (grid > a.ntiles) grid = a.ntiles;
     void *args[] = {&a};

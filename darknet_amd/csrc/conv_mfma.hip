@@ -76,6 +76,7 @@ extern "C" void conv_group_forward(const float *input, const float *weights, con
                                    const float *rolling_mean, const float *rolling_variance, float *output, int batch,
                                    int c, int h, int w, int n, int groups, int stride, int batch_normalize, double slope);
 /* conv_first.hip: the kernel of 3-channel first layers */
+extern "C" void conv_first_device_setup(void);
 extern "C" int conv_first_serves(int batch, int c, int h, int w, int n, int groups, int size, int stride, int pad);
 extern "C" const char *conv_first_kernel_name(int c, int n, int pooled, int h, int w);
 extern "C" void conv_first_forward(const float *input, const float *weights, const float *biases, const float *scales,
@@ -1601,6 +1602,7 @@ extern "C" __attribute__((visibility("hidden"))) void conv_device_setup(void)
         hip_check_error(hipGetDeviceProperties(&prop, dev));
         g_cus_dev[dev] = prop.multiProcessorCount;
     }
+    conv_first_device_setup(); /* resident workgroups per CU of the first-layer kernels */
 }
 
 static int g_tune_bands = 0;
