@@ -217,3 +217,35 @@ def test_parse_only_mode_computes_nothing():
     r = subprocess.run([sys.executable, "-c", code], cwd=ROOT, capture_output=True, text=True, timeout=120)
     assert "parsed 24" in r.stdout and "computed" not in r.stdout
     assert r.returncode != 0 and "parse-only" in r.stderr
+
+
+def test_which_layers_run_inside_the_convolution_in_front_of_them(parse_only):
+    """network_layer_runs_fused / network_layer_output_skipped are host decisions over the parsed layer table:
+    yolov3's 23 residual adds and 3 yolo heads; in yolov3-tiny the maxpools behind the two first-layer
+    convolutions and the two heads; with xnor=1 also the maxpools behind the xnor convolutions (not the
+    stride-1 pool), and no yolo head behind an xnor convolution; nothing at level 0; at level 2 the maps only
+    a fused maxpool reads are reported as not written."""
+    L = parse_only
+    cases = [(cfgs.yolov3(1, 416), None, []),
+             (cfgs.yolov3_tiny(2, 416), [1, 3, 16, 23], [0, 2]),
+             (cfgs.yolov3_tiny(2, 416, xnor=True), [1, 3, 5, 7, 9, 23], [0, 2, 4, 6])]
+    try:
+        for text, fused, skipped in cases:
+            net = api.Network(cfg_text=text)
+            types = [Ly["type"] for Ly in net.layers]
+            L.network_set_fusion(0)
+            assert not any(L.network_layer_runs_fused(net.net, i) for i in range(net.n))
+            L.network_set_fusion(1)
+            got = [i for i in range(net.n) if L.network_layer_runs_fused(net.net, i)]
+            if fused is None:
+                assert sorted(types[i] for i in got) == ["shortcut"] * 23 + ["yolo"] * 3
+            else:
+                assert got == fused
+            assert not any(L.network_layer_output_skipped(net.net, i) for i in range(net.n))
+            L.network_set_fusion(2)
+            assert [i for i in range(net.n) if L.network_layer_output_skipped(net.net, i)] == skipped
+            assert not L.network_layer_runs_fused(net.net, 0) and not L.network_layer_runs_fused(net.net, net.n)
+            net.free()
+    finally:
+        L.network_set_fusion(1)
+
