@@ -137,7 +137,13 @@ void binarize_weights_gpu(float *weights, int n, int size, float *binary); /* co
  * only to rounding (measured <= 1e-5 of the layer's largest value, tests hold 2e-5), where the
  * reference's per-image GEMM gives the same bits.  conv_set_algo(3), or conv_set_ksplit(1, 0),
  * switches the cut off: then every output sums K in one fixed order and the bits no longer depend
- * on the batch size (tested). */
+ * on the batch size (tested).
+ * Which kernel runs is decided by the geometry (conv_kernel_name_geometry names it): the implicit-GEMM
+ * kernel on the fp32 matrix cores for nearly everything; kernels of their own for the first layers
+ * of an image network (3x3 / 1 / pad 1 over 3 channels, or over 16 channels into up to 32 filters)
+ * and for grouped 3x3 layers of 4 or 8 channels per group (vector ALU); a plain direct kernel for the
+ * rest (groups that fit no tile scheme, 3x3 without padding on tap-blocked layers, one image beyond
+ * 4 GiB).  `packed` is only read by the implicit-GEMM kernel. */
 void forward_convolutional_gpu(const float *input, const float *weights, const float *packed,
                                const float *biases, const float *scales,
                                const float *rolling_mean, const float *rolling_variance,
